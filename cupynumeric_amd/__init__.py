@@ -1,0 +1,65 @@
+"""MI355X-native sort / argsort behind the cuPyNumeric API.
+
+    import cupynumeric_amd as num
+    a = num.array(host_array)
+    num.sort(a, axis=0); num.argsort(a, kind="stable"); a.sort()
+
+Only the sort path of cuPyNumeric is provided (`cupynumeric/_module/ssc_sorting.py:29-121`,
+`cupynumeric/_array/array.py:3773-3824`).  Every sort runs in hand-written HIP kernels of
+`libcpnsort.so`; there is no CPU fallback.
+"""
+from __future__ import annotations
+
+from typing import Any
+
+import numpy as np
+
+from . import random  # noqa: F401
+from ._array import convert_to_ndarray, ndarray
+from ._thunk import SUPPORTED_DTYPES, DeviceArray, check_dtype
+
+__all__ = ["ndarray", "array", "asarray", "sort", "argsort", "random", "SUPPORTED_DTYPES"]
+
+__version__ = "0.1.0"
+
+
+def array(obj: Any, dtype: Any = None, copy: bool = True) -> ndarray:
+    """Create an array from an array-like (host data is uploaded on first device use)."""
+    if isinstance(obj, ndarray) and dtype is None and not copy:
+        return obj
+    host = np.array(obj, dtype=dtype, copy=True)
+    check_dtype(host.dtype)
+    return ndarray(host.shape, host.dtype, thunk=DeviceArray.from_numpy(host))
+
+
+def asarray(obj: Any, dtype: Any = None) -> ndarray:
+    if isinstance(obj, ndarray) and (dtype is None or np.dtype(dtype) == obj.dtype):
+        return obj
+    return array(obj, dtype=dtype)
+
+
+def argsort(a: Any, axis: int | None = -1, kind: str = "quicksort", order: Any = None) -> ndarray:
+    """Indices that would sort `a` (`cupynumeric/_module/ssc_sorting.py:29-74`).
+
+    `kind` is 'quicksort', 'mergesort', 'heapsort' or 'stable'; every kind is served by the same
+    stable kernels.  `order` is not supported.  The result is int64, of `a.shape`, or flat when
+    `axis` is None.
+    """
+    a = convert_to_ndarray(a)
+    if axis is None:
+        result = ndarray((a.size,), np.int64)
+    else:
+        result = ndarray(a.shape, np.int64)
+    result._thunk.sort(rhs=a._thunk, argsort=True, axis=axis, kind=kind, order=order)
+    return result
+
+
+def sort(a: Any, axis: int | None = -1, kind: str = "quicksort", order: Any = None) -> ndarray:
+    """Sorted copy of `a` (`cupynumeric/_module/ssc_sorting.py:77-121`); flat when `axis` is None."""
+    a = convert_to_ndarray(a)
+    if axis is None:
+        result = ndarray((a.size,), a.dtype)
+    else:
+        result = ndarray(a.shape, a.dtype)
+    result._thunk.sort(rhs=a._thunk, axis=axis, kind=kind, order=order)
+    return result

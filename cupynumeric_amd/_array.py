@@ -1,0 +1,100 @@
+"""`ndarray`: the part of `cupynumeric/_array/array.py` that the sort path and its tests use
+(`sort` :3773-3796, `argsort` :3798-3824, `__array__` :820-832, shape/dtype accessors).
+"""
+from __future__ import annotations
+
+from typing import Any
+
+import numpy as np
+
+from ._thunk import DeviceArray, check_dtype
+
+
+def convert_to_ndarray(obj: Any) -> "ndarray":
+    """What `@add_boilerplate` does to array-like arguments (`cupynumeric/_array/util.py:115-182`)."""
+    if isinstance(obj, ndarray):
+        return obj
+    host = np.asarray(obj)
+    check_dtype(host.dtype)
+    return ndarray(host.shape, host.dtype, thunk=DeviceArray.from_numpy(host))
+
+
+class ndarray:
+    def __init__(self, shape: Any, dtype: Any = np.float64, thunk: DeviceArray | None = None) -> None:
+        if isinstance(shape, (int, np.integer)):
+            shape = (int(shape),)
+        dtype = check_dtype(dtype)
+        self._thunk = thunk if thunk is not None else DeviceArray(tuple(shape), dtype)
+        self._writeable = True
+
+    # -- metadata -----------------------------------------------------------------------------
+    @property
+    def shape(self) -> tuple[int, ...]:
+        return self._thunk.shape
+
+    @property
+    def ndim(self) -> int:
+        return self._thunk.ndim
+
+    @property
+    def dtype(self) -> np.dtype:
+        return self._thunk.dtype
+
+    @property
+    def size(self) -> int:
+        return self._thunk.size
+
+    @property
+    def itemsize(self) -> int:
+        return self._thunk.dtype.itemsize
+
+    @property
+    def nbytes(self) -> int:
+        return self.size * self.itemsize
+
+    def __len__(self) -> int:
+        if self.ndim == 0:
+            raise TypeError("len() of unsized object")
+        return self.shape[0]
+
+    def __repr__(self) -> str:
+        return f"cupynumeric_amd.ndarray(shape={self.shape}, dtype={self.dtype})"
+
+    # -- host interop -------------------------------------------------------------------------
+    def __array__(self, dtype: Any = None, copy: bool | None = None) -> np.ndarray:
+        out = self._thunk.__numpy_array__()
+        if dtype is not None and np.dtype(dtype) != out.dtype:
+            out = out.astype(dtype)
+        return out
+
+    def flatten(self, order: str = "C") -> "ndarray":
+        """Dense 1-D copy (C order)."""
+        if order not in ("C", "K", "A"):
+            raise NotImplementedError("only C-order flatten is supported")
+        return convert_to_ndarray(self.__array__().reshape(-1))
+
+    def setflags(self, write: bool | None = None) -> None:
+        if write is not None:
+            self._writeable = bool(write)
+
+    # -- sorting ------------------------------------------------------------------------------
+    def sort(self, axis: Any = -1, kind: str = "quicksort", order: Any = None) -> None:
+        """a.sort(axis=-1, kind=None, order=None): sort in place
+        (`cupynumeric/_array/array.py:3773-3796`)."""
+        if not self._writeable:
+            raise ValueError("array is not writeable")
+        self._thunk.sort(rhs=self._thunk, axis=axis, kind=kind, order=order)
+        _adopt_shape(self, self, axis)
+
+    def argsort(self, axis: Any = -1, kind: str = "quicksort", order: Any = None) -> "ndarray":
+        """a.argsort(axis=-1, kind=None, order=None) (`cupynumeric/_array/array.py:3798-3824`)."""
+        result = ndarray(self.shape, np.int64)
+        result._thunk.sort(rhs=self._thunk, argsort=True, axis=axis, kind=kind, order=order)
+        _adopt_shape(result, self, axis)
+        return result
+
+
+def _adopt_shape(result: ndarray, source: ndarray, axis: Any) -> None:
+    """Results of `axis=None` sorts are flat; nothing else changes shape."""
+    if axis is None and source.ndim > 1:
+        result._thunk.shape = (source.size,)

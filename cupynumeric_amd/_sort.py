@@ -1,0 +1,139 @@
+"""Axis dispatch of sort/argsort, following `cupynumeric/_thunk/_sort.py` function by
+function; `sort_task` calls the C ABI (`cpn_local_sort`) where the reference launches the
+Legate SORT task.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import TYPE_CHECKING
+
+from numpy.exceptions import AxisError
+from numpy.lib.array_utils import normalize_axis_index
+
+from . import _lib
+from .runtime import runtime
+
+if TYPE_CHECKING:
+    from ._thunk import DeviceArray
+
+
+def sort_flattened(output: "DeviceArray", input: "DeviceArray", argsort: bool, stable: bool) -> None:
+    """`cupynumeric/_thunk/_sort.py:37-47`."""
+    from ._thunk import DeviceArray
+
+    flattened = input.reshape((input.size,), order="C")
+
+    # run sort flattened -- return 1D solution
+    sort_result = DeviceArray(flattened.shape, dtype=output.dtype)
+    sort_deferred(sort_result, flattened, argsort, stable=stable)
+    output.base = sort_result.base
+
+
+def sort_swapped(output: "DeviceArray", input: "DeviceArray", argsort: bool, sort_axis: int, stable: bool) -> None:
+    """`cupynumeric/_thunk/_sort.py:50-76`.  The reference hands back a transposed view of the
+    sorted copy; here the result is copied back so that every array stays dense row-major."""
+    from ._thunk import DeviceArray
+
+    sort_axis = normalize_axis_index(sort_axis, input.ndim)
+    last = input.ndim - 1
+
+    # swap axes (dense copy)
+    swapped_copy = input.swapaxes_copy(sort_axis, last)
+
+    # run sort on last axis
+    if argsort is True:
+        sort_result = DeviceArray(swapped_copy.shape, dtype=output.dtype)
+        sort_deferred(sort_result, swapped_copy, argsort, stable=stable)
+        output.base = sort_result.swapaxes_copy(last, sort_axis).base
+    else:
+        sort_deferred(swapped_copy, swapped_copy, argsort, stable=stable)
+        output.base = swapped_copy.swapaxes_copy(last, sort_axis).base
+
+
+def sort_task(output: "DeviceArray", input: "DeviceArray", argsort: bool, stable: bool) -> None:
+    """`cupynumeric/_thunk/_sort.py:79-107`: sort the rows (last axis) of a dense array.
+
+    The task's scalars (argsort flag, shape, stable flag) become arguments of `cpn_local_sort`;
+    the output is aligned with the input (same shape), values for `sort`, int64 row positions
+    for `argsort`.
+    """
+    lib = _lib.load()
+    volume = input.size
+    if volume == 0:
+        return  # empty rectangle: nothing to do (`src/cupynumeric/sort/sort_template.inl:67-72`)
+    seg = input.shape[-1]
+    code = _lib.DTYPE_CODES[input.dtype]
+    in_place = (not argsort) and (output.base is input.base)
+
+    values_in = input.base.ptr()
+    if argsort:
+        values_out = None
+        indices_out = output.base.ptr()
+    else:
+        values_out = output.base.ptr()
+        indices_out = None
+
+    temp_bytes = lib.cpn_local_sort_temp_bytes(code, volume, seg, int(not argsort), int(argsort), int(in_place))
+    if temp_bytes == 0:
+        _lib.check(
+            lib.cpn_local_sort(code, values_in, values_out, indices_out, volume, seg, 0, int(stable), None, 0, None),
+            "cpn_local_sort",
+        )
+        raise NotImplementedError(f"cpn_local_sort: no workspace layout for dtype={input.dtype}, shape={input.shape}")
+    temp = runtime.empty_bytes(temp_bytes)
+    stream = runtime.stream_handle()
+    status = lib.cpn_local_sort(
+        code,
+        values_in,
+        values_out,
+        indices_out,
+        volume,
+        seg,
+        0,  # rect.lo[last] of a single-GPU launch (`src/cupynumeric/sort/sort.cu:1851`)
+        int(stable),
+        temp.data_ptr(),
+        temp_bytes,
+        ctypes.c_void_p(stream),
+    )
+    _lib.check(status, "cpn_local_sort")
+    if runtime.check_status:
+        _lib.check(lib.cpn_local_sort_check(temp.data_ptr(), ctypes.c_void_p(stream)), "cpn_local_sort")
+
+
+def sort_deferred(
+    output: "DeviceArray",
+    input: "DeviceArray",
+    argsort: bool,
+    axis: int | None = -1,
+    stable: bool = False,
+) -> None:
+    """`cupynumeric/_thunk/_sort.py:110-136`."""
+    # Handle 0-D arrays (scalars)
+    if input.ndim == 0:
+        if axis is not None:
+            # NumPy raises AxisError for any other axis value
+            raise AxisError(axis, input.ndim)
+        # For 0-D arrays, axis=None just returns the scalar
+        if argsort:
+            # the reference aliases the input store here even for argsort; a value buffer is
+            # not an index buffer, so hand back the only possible index instead
+            import numpy as np
+
+            from ._thunk import Storage
+
+            output.base = Storage(8, host=np.zeros(1, dtype=np.int64))
+        else:
+            output.base = input.base
+    else:
+        if axis is None and input.ndim > 1:
+            sort_flattened(output, input, argsort, stable)
+        else:
+            if axis is None:
+                computed_axis = 0
+            else:
+                computed_axis = normalize_axis_index(axis, input.ndim)
+
+            if computed_axis == input.ndim - 1:
+                sort_task(output, input, argsort, stable)
+            else:
+                sort_swapped(output, input, argsort, computed_axis, stable)

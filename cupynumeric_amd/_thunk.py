@@ -1,0 +1,148 @@
+"""Device-array thunk: the slice of the reference's `DeferredArray` that the sort path uses
+(`cupynumeric/_thunk/deferred.py`: `sort` :5453-5474, `copy` :394-398, `swapaxes` :2341-2351,
+`reshape` :2136-2316), over a dense row-major device buffer instead of a Legate store.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import TYPE_CHECKING, Any
+
+import numpy as np
+
+from . import _lib
+from .runtime import runtime
+
+if TYPE_CHECKING:
+    import torch
+
+# dtypes the reference supports (`cupynumeric/_utils/array.py:28-43`)
+SUPPORTED_DTYPES = tuple(_lib.DTYPE_CODES.keys())
+
+
+def check_dtype(dtype: Any) -> np.dtype:
+    """Same error text as `to_core_type` (`cupynumeric/_utils/array.py:64-68`)."""
+    try:
+        dt = np.dtype(dtype)
+    except TypeError:
+        raise TypeError(f"cuPyNumeric does not support dtype={dtype}")
+    if dt not in _lib.DTYPE_CODES:
+        raise TypeError(f"cuPyNumeric does not support dtype={dt}")
+    return dt
+
+
+class Storage:
+    """A dense device buffer.  Host data handed in at creation is uploaded on first device use,
+    so that building an array does not need a GPU (Legate attaches host data lazily as well)."""
+
+    def __init__(self, nbytes: int, host: np.ndarray | None = None) -> None:
+        self.nbytes = int(nbytes)
+        self._host = host
+        self._dev: "torch.Tensor | None" = None
+
+    def device(self) -> "torch.Tensor":
+        if self._dev is None:
+            if self._host is not None:
+                self._dev = runtime.upload(self._host)
+                self._host = None
+            else:
+                self._dev = runtime.empty_bytes(self.nbytes)
+        return self._dev
+
+    def ptr(self) -> int:
+        return int(self.device().data_ptr())
+
+    def to_numpy(self, shape: tuple[int, ...], dtype: np.dtype) -> np.ndarray:
+        if self._dev is None and self._host is not None:
+            return np.array(self._host, dtype=dtype).reshape(shape)
+        return runtime.download(self.device(), shape, dtype)
+
+
+class DeviceArray:
+    """Shape + dtype + `base` storage.  `base` can be re-bound, as the reference's sort helpers
+    do with `output.base = result.base` (`cupynumeric/_thunk/_sort.py:47,73,76`)."""
+
+    def __init__(self, shape: tuple[int, ...], dtype: Any, base: Storage | None = None) -> None:
+        self.shape = tuple(int(s) for s in shape)
+        self.dtype = check_dtype(dtype)
+        self.base = base if base is not None else Storage(self.size * self.dtype.itemsize)
+
+    @classmethod
+    def from_numpy(cls, arr: np.ndarray) -> "DeviceArray":
+        dt = check_dtype(arr.dtype)
+        host = np.array(arr, dtype=dt, order="C", copy=True)
+        return cls(host.shape, dt, Storage(host.nbytes, host=host))
+
+    @property
+    def ndim(self) -> int:
+        return len(self.shape)
+
+    @property
+    def size(self) -> int:
+        n = 1
+        for s in self.shape:
+            n *= s
+        return n
+
+    def __numpy_array__(self) -> np.ndarray:
+        return self.base.to_numpy(self.shape, self.dtype)
+
+    # -- data movement the sort path needs ------------------------------------------------
+    def reshape(self, newshape: tuple[int, ...], order: str = "C") -> "DeviceArray":
+        """C-order reshape.  Buffers are always dense row-major, so the storage is shared."""
+        if order != "C":
+            raise NotImplementedError("only C-order reshape is used by the sort path")
+        out = DeviceArray(newshape, self.dtype, self.base)
+        if out.size != self.size:
+            raise ValueError("cannot reshape array: sizes differ")
+        return out
+
+    def swapaxes_copy(self, axis1: int, axis2: int) -> "DeviceArray":
+        """Dense copy with two axes exchanged: the reference's `swapaxes` view followed by
+        `copy(deep=True)` (`cupynumeric/_thunk/_sort.py:59-65`) in one kernel."""
+        shape = list(self.shape)
+        shape[axis1], shape[axis2] = shape[axis2], shape[axis1]
+        out = DeviceArray(tuple(shape), self.dtype)
+        if self.size == 0:
+            return out
+        lib = _lib.load()
+        c_shape = (ctypes.c_int64 * max(self.ndim, 1))(*self.shape)
+        status = lib.cpn_swapaxes_copy(
+            self.dtype.itemsize,
+            self.base.ptr(),
+            out.base.ptr(),
+            c_shape,
+            self.ndim,
+            axis1,
+            axis2,
+            runtime.stream_handle(),
+        )
+        _lib.check(status, "cpn_swapaxes_copy")
+        return out
+
+    # -- the sort entry point ---------------------------------------------------------------
+    def sort(
+        self,
+        rhs: "DeviceArray",
+        argsort: bool = False,
+        axis: int | None = -1,
+        kind: str = "quicksort",
+        order: str | list[str] | None = None,
+    ) -> None:
+        """`DeferredArray.sort` (`cupynumeric/_thunk/deferred.py:5453-5474`): `self` receives the
+        result of sorting `rhs`."""
+        from ._sort import sort_deferred
+
+        if kind == "stable":
+            stable = True
+        else:
+            stable = False
+
+        if order is not None:
+            raise NotImplementedError(
+                "cuPyNumeric does not support sorting with 'order' as "
+                "ndarray only supports numeric values"
+            )
+        if axis is not None and (axis >= rhs.ndim or axis < -rhs.ndim):
+            raise ValueError("invalid axis")
+
+        sort_deferred(self, rhs, argsort, axis, stable)

@@ -1,0 +1,206 @@
+// Per-row sort in LDS: one workgroup owns one row (up to BLOCK*ITEMS elements), keeps the
+// keys in registers and runs a stable 8-bit LSD radix sort whose exchange step goes through
+// LDS.  One read and one write of HBM per element, whatever the key width.
+//
+// Replaces, for rows that fit, cub::DeviceSegmentedRadixSort
+// (src/cupynumeric/sort/cub_sort.cuh:81-105,153-182) and the (segment id, value) tuple
+// merge sort used for rows of at most 400 elements (src/cupynumeric/sort/thrust_sort.cuh:68-122).
+//
+// Digits on which every key of the row agrees are found up front with one AND/OR
+// reduction of the ordered keys and their passes are skipped (the pass would be the
+// identity permutation).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "radix_common.h"
+
+namespace cpn {
+
+template <typename T>
+__device__ __forceinline__ T wave_reduce_and(T v)
+{
+#pragma unroll
+  for (int delta = WAVE / 2; delta > 0; delta >>= 1) {
+    v &= __shfl_xor(v, delta, WAVE);
+  }
+  return v;
+}
+template <typename T>
+__device__ __forceinline__ T wave_reduce_or(T v)
+{
+#pragma unroll
+  for (int delta = WAVE / 2; delta > 0; delta >>= 1) {
+    v |= __shfl_xor(v, delta, WAVE);
+  }
+  return v;
+}
+
+// Register type used for shuffles of a key (sub-word keys travel as 32 bits).
+template <typename KeyT>
+struct ShuffleWord {
+  using type = uint32_t;
+};
+template <>
+struct ShuffleWord<uint64_t> {
+  using type = unsigned long long;
+};
+
+template <typename KeyT, int CODEC, bool HAS_IDX, int BLOCK, int ITEMS>
+__global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in,
+                                                              KeyT* keys_out,
+                                                              int64_t* idx_out,
+                                                              uint32_t seg,
+                                                              int64_t index_offset)
+{
+  constexpr int WAVES  = BLOCK / WAVE;
+  constexpr int TILE   = BLOCK * ITEMS;
+  constexpr int WTILE  = ITEMS * WAVE;
+  constexpr int PASSES = sizeof(KeyT);
+  using DT             = DigitThreads<BLOCK>;
+  using SW             = typename ShuffleWord<KeyT>::type;
+  using IdxS           = uint16_t;  // row position while staged in LDS
+  static_assert(TILE <= 65536, "row positions are staged as 16 bits");
+
+  __shared__ __align__(16) KeyT s_keys[TILE];
+  __shared__ IdxS s_idx[HAS_IDX ? TILE : 1];
+  __shared__ uint32_t s_ctr[WAVES * RADIX];
+  __shared__ uint32_t s_wsum[DT::WAVES];
+  __shared__ SW s_red[2 * WAVES];
+
+  const int tid       = threadIdx.x;
+  const int lane      = tid & (WAVE - 1);
+  const int wave      = tid / WAVE;
+  const uint64_t base = static_cast<uint64_t>(blockIdx.x) * seg;
+  const uint32_t woff = wave * WTILE + lane;
+  const bool full     = (seg == TILE);
+
+  KeyT key[ITEMS];
+  uint32_t idx[HAS_IDX ? ITEMS : 1];
+  SW all_and = ~static_cast<SW>(0), all_or = 0;
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t o = woff + i * WAVE;
+    if (full || o < seg) {
+      key[i]     = keys_in[base + o];
+      const SW v = static_cast<SW>(ordered_bits<CODEC, KeyT>(key[i]));
+      all_and &= v;
+      all_or |= v;
+    } else {
+      key[i] = static_cast<KeyT>(0);
+    }
+    if constexpr (HAS_IDX) {
+      idx[i] = o;
+    }
+  }
+  // bits on which the keys of the row differ
+  all_and = wave_reduce_and(all_and);
+  all_or  = wave_reduce_or(all_or);
+  if (lane == 0) {
+    s_red[2 * wave]     = all_and;
+    s_red[2 * wave + 1] = all_or;
+  }
+  __syncthreads();
+  SW varying;
+  {
+    SW a = s_red[0], o = s_red[1];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) {
+      a &= s_red[2 * w];
+      o |= s_red[2 * w + 1];
+    }
+    varying = a ^ o;
+  }
+
+  uint32_t* wctr = s_ctr + wave * RADIX;
+  for (int pass = 0; pass < PASSES; ++pass) {
+    const int shift = pass * RADIX_BITS;
+    if (((varying >> shift) & 0xFFu) == 0) {
+      continue;  // uniform for the block
+    }
+    for (int j = tid; j < WAVES * RADIX; j += BLOCK) {
+      s_ctr[j] = 0;
+    }
+    __syncthreads();
+    uint32_t rnk[ITEMS];
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      const bool valid = full || (woff + i * WAVE < seg);
+      rnk[i]           = wave_match_rank(radix_digit<CODEC, KeyT>(key[i], shift), valid, wctr);
+    }
+    __syncthreads();
+    // exclusive scan over (digit, wave) in digit-major order
+    uint32_t tsum = 0, tincl = 0;
+    if (tid < DT::THREADS) {
+#pragma unroll
+      for (int j = 0; j < DT::PER_THREAD; ++j) {
+        const int d = tid * DT::PER_THREAD + j;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+          const uint32_t c     = s_ctr[w * RADIX + d];
+          s_ctr[w * RADIX + d] = tsum;
+          tsum += c;
+        }
+      }
+      tincl = wave_inclusive_scan(tsum, lane);
+      if (lane == WAVE - 1) {
+        s_wsum[wave] = tincl;
+      }
+    }
+    __syncthreads();
+    if (tid < DT::THREADS) {
+      uint32_t texcl = tincl - tsum;
+      for (int w = 0; w < wave; ++w) {
+        texcl += s_wsum[w];
+      }
+#pragma unroll
+      for (int j = 0; j < DT::PER_THREAD; ++j) {
+        const int d = tid * DT::PER_THREAD + j;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+          s_ctr[w * RADIX + d] += texcl;
+        }
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      if (full || (woff + i * WAVE < seg)) {
+        const uint32_t d   = radix_digit<CODEC, KeyT>(key[i], shift);
+        const uint32_t pos = wctr[d] + rnk[i];
+        s_keys[pos]        = key[i];
+        if constexpr (HAS_IDX) {
+          s_idx[pos] = static_cast<IdxS>(idx[i]);
+        }
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      const uint32_t o = woff + i * WAVE;
+      if (full || o < seg) {
+        key[i] = s_keys[o];
+        if constexpr (HAS_IDX) {
+          idx[i] = s_idx[o];
+        }
+      }
+    }
+    // the next pass (or nothing) touches s_keys only after its own barriers
+  }
+
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t o = woff + i * WAVE;
+    if (full || o < seg) {
+      if (keys_out != nullptr) {
+        keys_out[base + o] = key[i];
+      }
+      if constexpr (HAS_IDX) {
+        idx_out[base + o] = static_cast<int64_t>(idx[i]) + index_offset;
+      }
+    }
+  }
+}
+
+}  // namespace cpn

@@ -1,0 +1,412 @@
+// Global LSD radix sort ("onesweep"): one histogram sweep over the keys, then one
+// scatter kernel per 8-bit digit in which every workgroup sorts a tile through LDS and
+// finds its global offsets with a decoupled look-back over per-tile descriptors.
+//
+// Replaces cub::DeviceRadixSort::SortKeys / SortPairs and, for rows too long for LDS,
+// cub::DeviceSegmentedRadixSort (src/cupynumeric/sort/cub_sort.cuh:60-182).  Rows are
+// batched into the same launches: a tile never straddles two rows and the look-back
+// stops at the first tile of its row.
+//
+// Data layout in HBM
+//   keys      raw element bits, dense row-major, ping-ponged between caller/workspace buffers
+//   payload   position of the element inside its row, 32-bit while a row is shorter than
+//             2^30 elements (64-bit otherwise), synthesised by the first pass and widened
+//             to int64 (+ index_offset) by the last one
+//   hist      [row][pass][256] counts, exclusive-scanned in place
+//   desc      [pass][tile][256] words: 2 status bits | count   (aggregate or inclusive)
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "radix_common.h"
+
+namespace cpn {
+
+// Widths that depend on the row length.  Rows shorter than 2^30 keep every per-row count
+// and the index payload in 32 bits (two bits of a descriptor word hold its status).
+template <bool BIG>
+struct RowWidth;
+template <>
+struct RowWidth<false> {
+  using off_t = uint32_t;
+};
+template <>
+struct RowWidth<true> {
+  using off_t = uint64_t;
+};
+
+template <typename D>
+struct DescBits {
+  static constexpr int BITS    = sizeof(D) * 8;
+  static constexpr D AGGREGATE = static_cast<D>(1) << (BITS - 2);
+  static constexpr D INCLUSIVE = static_cast<D>(2) << (BITS - 2);
+  static constexpr D STATUS    = static_cast<D>(3) << (BITS - 2);
+  static constexpr D VALUE     = static_cast<D>(~STATUS);
+};
+
+// Upper bound on polls of one descriptor before a tile gives up and flags an error, so
+// that every wave exits even if a predecessor never publishes.
+constexpr uint32_t LOOKBACK_SPIN_LIMIT = 1u << 22;
+
+// Status word values written by kernels into the workspace header.
+constexpr uint32_t DEVICE_ERR_LOOKBACK = 1u;
+
+// ---------------------------------------------------------------------------------------
+// zero fill (capture-safe replacement for a memset node)
+// ---------------------------------------------------------------------------------------
+static __global__ __launch_bounds__(256) void zero_fill_kernel(uint4* p, uint64_t n_vec)
+{
+  const uint64_t stride = static_cast<uint64_t>(gridDim.x) * blockDim.x;
+  for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n_vec; i += stride) {
+    p[i] = make_uint4(0u, 0u, 0u, 0u);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// histogram sweep: all digit histograms of every row in one read of the keys
+// ---------------------------------------------------------------------------------------
+constexpr int HIST_BLOCK = 256;
+
+template <typename KeyT, int CODEC, int PASSES>
+__device__ __forceinline__ void hist_accumulate(uint32_t* s_hist, KeyT raw)
+{
+  const KeyT o = ordered_bits<CODEC, KeyT>(raw);
+#pragma unroll
+  for (int p = 0; p < PASSES; ++p) {
+    atomicAdd(&s_hist[p * RADIX + (static_cast<uint32_t>(o >> (p * RADIX_BITS)) & 0xFFu)], 1u);
+  }
+}
+
+// grid = rows * blocks_per_row; block b of a row covers elements [b*chunk, min(seg, (b+1)*chunk)).
+// 128-bit loads over the 16-byte aligned middle of the chunk, scalar head and tail.
+template <typename KeyT, int CODEC, typename OffT>
+__global__ __launch_bounds__(HIST_BLOCK) void histogram_kernel(const KeyT* __restrict__ keys,
+                                                                 OffT* __restrict__ hist,
+                                                                 uint64_t seg,
+                                                                 uint32_t blocks_per_row,
+                                                                 uint64_t chunk)
+{
+  constexpr int PASSES = sizeof(KeyT);
+  constexpr int VEC    = 16 / sizeof(KeyT);
+  __shared__ uint32_t s_hist[PASSES * RADIX];
+
+  const int tid        = threadIdx.x;
+  const uint64_t row   = blockIdx.x / blocks_per_row;
+  const uint32_t piece = blockIdx.x - static_cast<uint32_t>(row * blocks_per_row);
+  const uint64_t begin = static_cast<uint64_t>(piece) * chunk;
+  uint64_t end         = begin + chunk;
+  if (end > seg) {
+    end = seg;
+  }
+  for (int j = tid; j < PASSES * RADIX; j += HIST_BLOCK) {
+    s_hist[j] = 0;
+  }
+  __syncthreads();
+
+  if (begin < end) {
+    const KeyT* p = keys + row * seg;
+    // elements before the first 16-byte boundary
+    const uintptr_t addr = reinterpret_cast<uintptr_t>(p + begin);
+    uint64_t head        = ((16u - (addr & 15u)) & 15u) / sizeof(KeyT);
+    if (head > end - begin) {
+      head = end - begin;
+    }
+    for (uint64_t i = tid; i < head; i += HIST_BLOCK) {
+      hist_accumulate<KeyT, CODEC, PASSES>(s_hist, p[begin + i]);
+    }
+    const uint64_t vbegin = begin + head;
+    const uint64_t nvec   = (end - vbegin) / VEC;
+    const uint4* vp       = reinterpret_cast<const uint4*>(p + vbegin);
+    for (uint64_t v = tid; v < nvec; v += HIST_BLOCK) {
+      const uint4 q = vp[v];
+      KeyT k[VEC];
+      __builtin_memcpy(k, &q, 16);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        hist_accumulate<KeyT, CODEC, PASSES>(s_hist, k[j]);
+      }
+    }
+    for (uint64_t i = vbegin + nvec * VEC + tid; i < end; i += HIST_BLOCK) {
+      hist_accumulate<KeyT, CODEC, PASSES>(s_hist, p[i]);
+    }
+  }
+  __syncthreads();
+
+  OffT* out = hist + row * (PASSES * RADIX);
+  for (int j = tid; j < PASSES * RADIX; j += HIST_BLOCK) {
+    const uint32_t c = s_hist[j];
+    if (c != 0) {
+      __hip_atomic_fetch_add(&out[j], static_cast<OffT>(c), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
+// One block per (row, pass): exclusive scan of 256 counts in place.
+template <typename OffT>
+__global__ __launch_bounds__(RADIX) void histogram_scan_kernel(OffT* __restrict__ hist)
+{
+  __shared__ OffT s_wsum[RADIX / WAVE];
+  const int tid  = threadIdx.x;
+  const int lane = tid & (WAVE - 1);
+  const int wave = tid / WAVE;
+  OffT* h        = hist + static_cast<uint64_t>(blockIdx.x) * RADIX;
+  const OffT c   = h[tid];
+  OffT incl      = c;
+#pragma unroll
+  for (int delta = 1; delta < WAVE; delta <<= 1) {
+    const OffT t = __shfl_up(incl, delta, WAVE);
+    if (lane >= delta) {
+      incl += t;
+    }
+  }
+  if (lane == WAVE - 1) {
+    s_wsum[wave] = incl;
+  }
+  __syncthreads();
+  OffT prefix = 0;
+  for (int w = 0; w < wave; ++w) {
+    prefix += s_wsum[w];
+  }
+  h[tid] = prefix + incl - c;
+}
+
+// ---------------------------------------------------------------------------------------
+// onesweep scatter pass
+// ---------------------------------------------------------------------------------------
+template <bool BIG>
+struct SweepArgs {
+  using OffT = typename RowWidth<BIG>::off_t;
+  const void* keys_in;     // KeyT[volume]
+  void* keys_out;          // KeyT[volume] or nullptr (last pass of an index-only sort)
+  const OffT* idx_in;      // row positions from the previous pass, nullptr = synthesise
+  void* idx_out;           // OffT[volume], or int64[volume] when idx_final
+  uint32_t* ticket;        // tile ticket counter of this pass (zeroed)
+  const OffT* hist_excl;   // this pass's scanned histogram of row 0; row stride = hist_row_stride
+  OffT* desc;              // [num_tiles][256] descriptors of this pass (zeroed)
+  uint32_t* status;        // device status word
+  uint64_t seg;            // row length
+  uint64_t hist_row_stride;
+  int64_t index_offset;
+  uint32_t tiles_per_row;
+  uint32_t num_tiles;
+  int shift;               // bit position of this pass's digit
+  int idx_final;           // idx_out is the caller's int64 array
+};
+
+template <typename KeyT, int CODEC, bool BIG, bool HAS_IDX, int BLOCK, int ITEMS>
+__global__ __launch_bounds__(BLOCK) void onesweep_kernel(const SweepArgs<BIG> a)
+{
+  using OffT = typename RowWidth<BIG>::off_t;
+  using DB   = DescBits<OffT>;
+  static_assert(BLOCK >= RADIX, "one thread per digit is needed for the look-back");
+  constexpr int WAVES      = BLOCK / WAVE;
+  constexpr int TILE       = BLOCK * ITEMS;
+  constexpr int WTILE      = ITEMS * WAVE;  // keys of one wave, contiguous in the tile
+  constexpr int STAGE_ELEM = (HAS_IDX && sizeof(OffT) > sizeof(KeyT)) ? sizeof(OffT) : sizeof(KeyT);
+
+  __shared__ __align__(16) unsigned char s_stage[TILE * STAGE_ELEM];
+  __shared__ uint32_t s_ctr[WAVES * RADIX];
+  __shared__ uint64_t s_gbase[RADIX];
+  __shared__ uint32_t s_wsum[RADIX / WAVE];
+  __shared__ uint32_t s_tile;
+
+  const int tid  = threadIdx.x;
+  const int lane = tid & (WAVE - 1);
+  const int wave = tid / WAVE;
+
+  // Tiles are handed out in launch order of the workgroups that are actually running, so
+  // every tile a look-back waits for belongs to a resident workgroup.
+  if (tid == 0) {
+    s_tile = __hip_atomic_fetch_add(a.ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  for (int j = tid; j < WAVES * RADIX; j += BLOCK) {
+    s_ctr[j] = 0;
+  }
+  __syncthreads();
+  const uint32_t tile = s_tile;
+  if (tile >= a.num_tiles) {
+    return;  // uniform per block; cannot happen when grid == num_tiles
+  }
+  const uint64_t row      = tile / a.tiles_per_row;
+  const uint32_t trow     = tile - static_cast<uint32_t>(row * a.tiles_per_row);
+  const uint64_t row_base = row * a.seg;
+  const uint64_t tile_off = static_cast<uint64_t>(trow) * TILE;
+  const uint64_t remain   = a.seg - tile_off;
+  const uint32_t count    = remain < static_cast<uint64_t>(TILE) ? static_cast<uint32_t>(remain) : TILE;
+  const bool full         = (count == TILE);
+  const uint32_t woff     = wave * WTILE + lane;
+
+  // ---- load: item i of lane l is element  wave*WTILE + i*64 + l  of the tile ----
+  const KeyT* kin = static_cast<const KeyT*>(a.keys_in) + row_base + tile_off;
+  KeyT key[ITEMS];
+  if (full) {
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      key[i] = kin[woff + i * WAVE];
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      const uint32_t o = woff + i * WAVE;
+      key[i]           = (o < count) ? kin[o] : static_cast<KeyT>(0);
+    }
+  }
+  OffT idx[HAS_IDX ? ITEMS : 1];
+  if constexpr (HAS_IDX) {
+    if (a.idx_in != nullptr) {
+      const OffT* iin = a.idx_in + row_base + tile_off;
+#pragma unroll
+      for (int i = 0; i < ITEMS; ++i) {
+        const uint32_t o = woff + i * WAVE;
+        idx[i]           = (full || o < count) ? iin[o] : static_cast<OffT>(0);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < ITEMS; ++i) {
+        idx[i] = static_cast<OffT>(tile_off + woff + i * WAVE);
+      }
+    }
+  }
+
+  // ---- rank inside the wave, count digits per wave ----
+  uint32_t rnk[ITEMS];
+  uint32_t* wctr = s_ctr + wave * RADIX;
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const bool valid = full || (woff + i * WAVE < count);
+    rnk[i]           = wave_match_rank(radix_digit<CODEC, KeyT>(key[i], a.shift), valid, wctr);
+  }
+  __syncthreads();
+
+  // ---- per digit: offsets of the waves, tile total, publish, scan over digits ----
+  uint32_t dsum = 0, dincl = 0;
+  OffT* my_desc = a.desc + static_cast<uint64_t>(tile) * RADIX + tid;
+  if (tid < RADIX) {
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      const uint32_t c       = s_ctr[w * RADIX + tid];
+      s_ctr[w * RADIX + tid] = dsum;
+      dsum += c;
+    }
+    const OffT first = (trow == 0) ? DB::INCLUSIVE : DB::AGGREGATE;
+    __hip_atomic_store(my_desc, static_cast<OffT>(first | dsum), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    dincl = wave_inclusive_scan(dsum, lane);
+    if (lane == WAVE - 1) {
+      s_wsum[wave] = dincl;
+    }
+  }
+  __syncthreads();
+  if (tid < RADIX) {
+    uint32_t dexcl = dincl - dsum;
+    for (int w = 0; w < wave; ++w) {
+      dexcl += s_wsum[w];
+    }
+    // ---- decoupled look-back over the earlier tiles of this row ----
+    OffT before = 0;
+    if (trow != 0) {
+      uint32_t t        = tile - 1;
+      const uint32_t t0 = tile - trow;  // first tile of the row, always INCLUSIVE
+      bool failed       = false;
+      while (true) {
+        const OffT* dp = a.desc + static_cast<uint64_t>(t) * RADIX + tid;
+        OffT v         = __hip_atomic_load(dp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        uint32_t spins = 0;
+        while ((v & DB::STATUS) == 0) {
+          if (++spins >= LOOKBACK_SPIN_LIMIT) {
+            failed = true;
+            break;
+          }
+          if ((spins & 1023u) == 0 &&
+              __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
+            failed = true;  // another tile already gave up: drain quickly
+            break;
+          }
+          __builtin_amdgcn_s_sleep(2);
+          v = __hip_atomic_load(dp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (failed) {
+          break;
+        }
+        before += (v & DB::VALUE);
+        if ((v & DB::INCLUSIVE) != 0 || t == t0) {
+          break;
+        }
+        --t;
+      }
+      if (failed) {
+        __hip_atomic_fetch_or(a.status, DEVICE_ERR_LOOKBACK, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      __hip_atomic_store(my_desc, static_cast<OffT>(DB::INCLUSIVE | (before + dsum)), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+    }
+    // global element offset of local sorted position 0 for this digit (unsigned wrap is fine)
+    s_gbase[tid] = row_base + static_cast<uint64_t>(a.hist_excl[row * a.hist_row_stride + tid]) +
+                   static_cast<uint64_t>(before) - static_cast<uint64_t>(dexcl);
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      s_ctr[w * RADIX + tid] += dexcl;
+    }
+  }
+  __syncthreads();
+
+  // ---- local scatter into LDS, then coalesced runs to HBM ----
+  KeyT* s_keys = reinterpret_cast<KeyT*>(s_stage);
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    if (full || (woff + i * WAVE < count)) {
+      const uint32_t d   = radix_digit<CODEC, KeyT>(key[i], a.shift);
+      const uint32_t pos = wctr[d] + rnk[i];
+      rnk[i]             = pos;
+      s_keys[pos]        = key[i];
+    }
+  }
+  __syncthreads();
+  uint32_t dig[ITEMS];
+  KeyT* kout = static_cast<KeyT*>(a.keys_out);
+#pragma unroll
+  for (int k = 0; k < ITEMS; ++k) {
+    const uint32_t p = tid + k * BLOCK;
+    if (full || p < count) {
+      const KeyT kk = s_keys[p];
+      dig[k]        = radix_digit<CODEC, KeyT>(kk, a.shift);
+      if (kout != nullptr) {
+        kout[s_gbase[dig[k]] + p] = kk;
+      }
+    } else {
+      dig[k] = 0;
+    }
+  }
+  if constexpr (HAS_IDX) {
+    __syncthreads();
+    OffT* s_idx = reinterpret_cast<OffT*>(s_stage);
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      if (full || (woff + i * WAVE < count)) {
+        s_idx[rnk[i]] = idx[i];
+      }
+    }
+    __syncthreads();
+    if (a.idx_final) {
+      int64_t* iout = static_cast<int64_t*>(a.idx_out);
+#pragma unroll
+      for (int k = 0; k < ITEMS; ++k) {
+        const uint32_t p = tid + k * BLOCK;
+        if (full || p < count) {
+          iout[s_gbase[dig[k]] + p] = static_cast<int64_t>(s_idx[p]) + a.index_offset;
+        }
+      }
+    } else {
+      OffT* iout = static_cast<OffT*>(a.idx_out);
+#pragma unroll
+      for (int k = 0; k < ITEMS; ++k) {
+        const uint32_t p = tid + k * BLOCK;
+        if (full || p < count) {
+          iout[s_gbase[dig[k]] + p] = s_idx[p];
+        }
+      }
+    }
+  }
+}
+
+}  // namespace cpn

@@ -1,0 +1,78 @@
+// Building blocks shared by the global (onesweep) and the per-row (LDS) radix sorts:
+// wave64 match-any ranking, the per-tile digit scan, and small helpers.
+//
+// Replaces what the reference gets from cub's block/warp radix-rank primitives behind
+// cub::DeviceRadixSort / DeviceSegmentedRadixSort (src/cupynumeric/sort/cub_sort.cuh:60-182).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "key_codec.h"
+
+namespace cpn {
+
+constexpr int RADIX_BITS = 8;
+constexpr int RADIX      = 1 << RADIX_BITS;
+constexpr int WAVE       = 64;
+
+__device__ __forceinline__ uint32_t lanes_below(uint64_t mask)
+{
+  return __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(mask >> 32),
+                                   __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0u));
+}
+
+// Stable rank of one key per lane inside a wave, keys ordered by lane id.
+//
+//   digit   8-bit digit of this lane's key
+//   valid   lane holds a real key
+//   wctr    this wave's 256 running digit counters in LDS (count of that digit in the
+//           wave's earlier rounds)
+//
+// Returns the number of keys with the same digit that precede this key in the wave
+// (earlier rounds + lower lanes of this round) and advances the counter.  Eight ballots
+// build the mask of lanes holding the same digit; the highest such lane updates the
+// counter after every peer has read it (LDS operations of one wave execute in order).
+__device__ __forceinline__ uint32_t wave_match_rank(uint32_t digit, bool valid, uint32_t* wctr)
+{
+  uint64_t peers = __builtin_amdgcn_ballot_w64(valid);
+#pragma unroll
+  for (int b = 0; b < RADIX_BITS; ++b) {
+    const bool bit     = (digit >> b) & 1u;
+    const uint64_t bal = __builtin_amdgcn_ballot_w64(bit);
+    peers &= bit ? bal : ~bal;
+  }
+  const uint32_t lower = lanes_below(peers);
+  const uint32_t total = static_cast<uint32_t>(__builtin_popcountll(peers));
+  const uint32_t old   = wctr[digit];
+  __builtin_amdgcn_wave_barrier();
+  if (valid && lower + 1 == total) {
+    wctr[digit] = old + total;
+  }
+  __builtin_amdgcn_wave_barrier();
+  return old + lower;
+}
+
+// Inclusive scan of one 32-bit value per lane across a wave.
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v, int lane)
+{
+#pragma unroll
+  for (int delta = 1; delta < WAVE; delta <<= 1) {
+    const uint32_t t = __shfl_up(v, delta, WAVE);
+    if (lane >= delta) {
+      v += t;
+    }
+  }
+  return v;
+}
+
+// How the 256 digits of a tile are spread over the threads that scan them.
+template <int BLOCK>
+struct DigitThreads {
+  static_assert(BLOCK % WAVE == 0 && BLOCK >= WAVE, "block must be whole waves");
+  static constexpr int PER_THREAD = (BLOCK >= RADIX) ? 1 : RADIX / BLOCK;  // digits per scanning thread
+  static constexpr int THREADS    = RADIX / PER_THREAD;                      // scanning threads
+  static constexpr int WAVES      = THREADS / WAVE;
+};
+
+}  // namespace cpn

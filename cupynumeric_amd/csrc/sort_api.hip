@@ -1,0 +1,200 @@
+// extern "C" surface of libcpnsort.so (declared in include/cpn_sort.h): argument checks,
+// dtype dispatch and the status read-back.  Plays the role of local_sort<CODE>
+// (src/cupynumeric/sort/sort.cu:63-96) plus the type dispatch of sort_template
+// (src/cupynumeric/sort/sort_template.inl:92-120).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdlib.h>
+
+#include <atomic>
+
+#include "sort_driver.h"
+
+namespace cpn {
+
+thread_local int g_last_hip_error = 0;
+
+int swapaxes_copy(int elem_bytes, const void* in, void* out, const int64_t* shape, int ndim, int axis_a, int axis_b,
+                  hipStream_t stream);
+
+// -1 = not overridden.  Initialised from CPN_SORT_LDS_ROW_LIMIT, changed by cpn_set_lds_row_limit.
+static std::atomic<long long> g_lds_row_limit{[] {
+  const char* e = getenv("CPN_SORT_LDS_ROW_LIMIT");
+  return (e != nullptr && *e != 0) ? atoll(e) : -1ll;
+}()};
+
+uint64_t lds_row_limit(int key_bytes)
+{
+  const long long limit = g_lds_row_limit.load(std::memory_order_relaxed);
+  const uint64_t cap    = lds_row_capacity(key_bytes);
+  if (limit >= 0 && static_cast<uint64_t>(limit) < cap) {
+    return static_cast<uint64_t>(limit);
+  }
+  return cap;
+}
+
+struct KeyKind {
+  int bytes;  // 0 = unknown code
+  int codec;  // -1 = known but unsupported
+};
+
+static KeyKind key_kind(int dtype)
+{
+  switch (dtype) {
+    case CPN_BOOL: return {1, CODEC_UNSIGNED};
+    case CPN_INT8: return {1, CODEC_SIGNED};
+    case CPN_INT16: return {2, CODEC_SIGNED};
+    case CPN_INT32: return {4, CODEC_SIGNED};
+    case CPN_INT64: return {8, CODEC_SIGNED};
+    case CPN_UINT8: return {1, CODEC_UNSIGNED};
+    case CPN_UINT16: return {2, CODEC_UNSIGNED};
+    case CPN_UINT32: return {4, CODEC_UNSIGNED};
+    case CPN_UINT64: return {8, CODEC_UNSIGNED};
+    case CPN_FLOAT16: return {2, CODEC_FLOAT};
+    case CPN_FLOAT32: return {4, CODEC_FLOAT};
+    case CPN_FLOAT64: return {8, CODEC_FLOAT};
+    case CPN_COMPLEX64: return {8, -1};
+    case CPN_COMPLEX128: return {16, -1};
+    default: return {0, -1};
+  }
+}
+
+}  // namespace cpn
+
+extern "C" {
+
+int cpn_sort_version(void) { return (0 << 16) | 1; }
+
+const char* cpn_status_string(int status)
+{
+  switch (status) {
+    case CPN_OK: return "ok";
+    case CPN_ERR_DTYPE: return "unknown element type code";
+    case CPN_ERR_NULL: return "required pointer is NULL";
+    case CPN_ERR_SHAPE: return "sort_dim_size is zero or does not divide volume, or bad axes";
+    case CPN_ERR_TEMP: return "workspace missing, too small or not 256-byte aligned";
+    case CPN_ERR_ALIGN: return "data pointer is not aligned to its element size";
+    case CPN_ERR_HIP: return "HIP runtime call failed";
+    case CPN_ERR_DEVICE: return "kernel reported an internal failure";
+    case CPN_ERR_UNSUPPORTED: return "request not implemented by this build";
+    default: return "unknown status";
+  }
+}
+
+int cpn_last_hip_error(void) { return cpn::g_last_hip_error; }
+
+int64_t cpn_set_lds_row_limit(int64_t limit)
+{
+  return static_cast<int64_t>(cpn::g_lds_row_limit.exchange(limit < 0 ? -1ll : static_cast<long long>(limit)));
+}
+
+uint64_t cpn_dtype_size(int dtype) { return static_cast<uint64_t>(cpn::key_kind(dtype).bytes); }
+
+uint64_t cpn_local_sort_temp_bytes(int dtype, uint64_t volume, uint64_t sort_dim_size, int want_values,
+                                   int want_indices, int in_place)
+{
+  const cpn::KeyKind k = cpn::key_kind(dtype);
+  if (k.bytes == 0 || k.codec < 0) {
+    return 0;
+  }
+  if (volume == 0) {
+    return cpn::HEADER_BYTES;
+  }
+  if (sort_dim_size == 0 || volume % sort_dim_size != 0) {
+    return 0;
+  }
+  return cpn::workspace_bytes(k.bytes, volume, sort_dim_size, want_values != 0, want_indices != 0, in_place != 0);
+}
+
+int cpn_local_sort(int dtype, const void* values_in, void* values_out, int64_t* indices_out, uint64_t volume,
+                   uint64_t sort_dim_size, int64_t index_offset, int stable, void* temp, uint64_t temp_bytes,
+                   void* stream)
+{
+  (void)stable;  // every path is stable
+  const cpn::KeyKind k = cpn::key_kind(dtype);
+  if (k.bytes == 0) {
+    return CPN_ERR_DTYPE;
+  }
+  if (k.codec < 0) {
+    return CPN_ERR_UNSUPPORTED;
+  }
+  if (volume == 0) {
+    return CPN_OK;
+  }
+  if (sort_dim_size == 0 || volume % sort_dim_size != 0) {
+    return CPN_ERR_SHAPE;
+  }
+  if (values_in == nullptr || (values_out == nullptr && indices_out == nullptr)) {
+    return CPN_ERR_NULL;
+  }
+  const uintptr_t kmask = static_cast<uintptr_t>(k.bytes - 1);
+  if ((reinterpret_cast<uintptr_t>(values_in) & kmask) != 0 || (reinterpret_cast<uintptr_t>(values_out) & kmask) != 0 ||
+      (reinterpret_cast<uintptr_t>(indices_out) & 7u) != 0) {
+    return CPN_ERR_ALIGN;
+  }
+  cpn::SortRequest r{};
+  r.values_in    = values_in;
+  r.values_out   = values_out;
+  r.indices_out  = indices_out;
+  r.volume       = volume;
+  r.seg          = sort_dim_size;
+  r.index_offset = index_offset;
+  r.temp         = temp;
+  r.temp_bytes   = temp_bytes;
+  r.stream       = static_cast<hipStream_t>(stream);
+  switch (k.bytes) {
+    case 1: return cpn::sort_keys8(k.codec, r);
+    case 2: return cpn::sort_keys16(k.codec, r);
+    case 4: return cpn::sort_keys32(k.codec, r);
+    case 8: return cpn::sort_keys64(k.codec, r);
+    default: return CPN_ERR_UNSUPPORTED;
+  }
+}
+
+int cpn_local_sort_check(const void* temp, void* stream)
+{
+  if (temp == nullptr) {
+    return CPN_ERR_NULL;
+  }
+  uint32_t word = 0;
+  CPN_HIP_TRY(hipMemcpyAsync(&word, temp, sizeof(word), hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)));
+  CPN_HIP_TRY(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  return word == 0 ? CPN_OK : CPN_ERR_DEVICE;
+}
+
+int cpn_swapaxes_copy(int elem_bytes, const void* in, void* out, const int64_t* shape, int ndim, int axis_a, int axis_b,
+                      void* stream)
+{
+  if (shape == nullptr && ndim > 0) {
+    return CPN_ERR_NULL;
+  }
+  if (ndim < 0 || ndim > 8 || (ndim == 0 && (axis_a != 0 || axis_b != 0))) {
+    return CPN_ERR_SHAPE;
+  }
+  if (ndim > 0 && (axis_a < 0 || axis_a >= ndim || axis_b < 0 || axis_b >= ndim)) {
+    return CPN_ERR_SHAPE;
+  }
+  if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8 && elem_bytes != 16) {
+    return CPN_ERR_SHAPE;
+  }
+  uint64_t total = 1;
+  for (int i = 0; i < ndim; ++i) {
+    if (shape[i] < 0) {
+      return CPN_ERR_SHAPE;
+    }
+    total *= static_cast<uint64_t>(shape[i]);
+  }
+  if (total == 0) {
+    return CPN_OK;
+  }
+  if (in == nullptr || out == nullptr) {
+    return CPN_ERR_NULL;
+  }
+  const uintptr_t mask = static_cast<uintptr_t>(elem_bytes - 1);
+  if ((reinterpret_cast<uintptr_t>(in) & mask) != 0 || (reinterpret_cast<uintptr_t>(out) & mask) != 0) {
+    return CPN_ERR_ALIGN;
+  }
+  return cpn::swapaxes_copy(elem_bytes, in, out, shape, ndim, axis_a, axis_b, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

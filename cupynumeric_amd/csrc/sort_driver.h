@@ -1,0 +1,325 @@
+// Host side of the sort: path choice, workspace layout, buffer ping-pong and launches.
+//
+// Plays the role of cub_local_sort / thrust_local_sort and their temporary-buffer handling
+// (src/cupynumeric/sort/cub_sort.cuh:36-193, src/cupynumeric/sort/thrust_sort.cuh:37-124),
+// with the workspace supplied by the caller instead of a Legate pool.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/cpn_sort.h"
+#include "lds_row_sort.h"
+#include "onesweep.h"
+
+namespace cpn {
+
+// Set by HIP_TRY when a runtime call fails; read through cpn_last_hip_error().
+extern thread_local int g_last_hip_error;
+
+#define CPN_HIP_TRY(expr)                        \
+  do {                                           \
+    const hipError_t cpn_err_ = (expr);          \
+    if (cpn_err_ != hipSuccess) {                \
+      ::cpn::g_last_hip_error = (int)cpn_err_;   \
+      (void)hipGetLastError();                   \
+      return CPN_ERR_HIP;                        \
+    }                                            \
+  } while (0)
+
+constexpr uint64_t WORKSPACE_ALIGN  = 256;
+constexpr uint64_t HEADER_BYTES     = 256;  // [0] status word, [64..] tile tickets (one per pass)
+constexpr uint64_t HEADER_TICKETS   = 64;
+constexpr uint64_t BIG_ROW_ELEMENTS = 1ull << 30;
+
+__host__ __device__ constexpr uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
+
+// Tile shape of the global sort per key width.
+__host__ __device__ constexpr int global_block(int /*key_bytes*/) { return 512; }
+// (64-bit keys or 64-bit row positions halve the items per thread so that the LDS staging
+// area stays at 32 KiB)
+__host__ __device__ constexpr int global_items(int key_bytes, bool big) { return (key_bytes == 8 || big) ? 8 : 16; }
+__host__ __device__ constexpr int global_tile(int key_bytes, bool big)
+{
+  return global_block(key_bytes) * global_items(key_bytes, big);
+}
+
+// Longest row the LDS kernel can take, per key width (keeps static LDS below 64 KiB).
+__host__ __device__ constexpr uint64_t lds_row_capacity(int key_bytes) { return key_bytes == 8 ? 4096 : 8192; }
+
+// Row length up to which the LDS kernel is used.  Equals lds_row_capacity unless the
+// environment variable CPN_SORT_LDS_ROW_LIMIT or cpn_set_lds_row_limit lowers it, e.g. to 0
+// to send every request down the global path for an A/B run.
+uint64_t lds_row_limit(int key_bytes);
+
+struct SortRequest {
+  const void* values_in;
+  void* values_out;      // may be nullptr
+  int64_t* indices_out;  // may be nullptr
+  uint64_t volume;
+  uint64_t seg;
+  int64_t index_offset;
+  void* temp;
+  uint64_t temp_bytes;
+  hipStream_t stream;
+};
+
+// Workspace layout of the global path.  Everything in [0, zero_bytes) is cleared per call.
+struct GlobalLayout {
+  bool big;
+  int passes;
+  uint64_t rows;
+  uint32_t tiles_per_row;
+  uint64_t num_tiles;
+  uint64_t off_hist, hist_bytes;
+  uint64_t off_desc, desc_bytes_per_pass;
+  uint64_t zero_bytes;
+  uint64_t off_key1, off_key2, key_bytes_total;
+  uint64_t off_idx, idx_bytes_total;
+  uint64_t total;
+  bool valid;
+};
+
+inline GlobalLayout global_layout(int key_bytes, uint64_t volume, uint64_t seg, bool want_values,
+                                  bool want_indices, bool in_place)
+{
+  GlobalLayout L{};
+  L.big           = seg >= BIG_ROW_ELEMENTS;
+  L.passes        = key_bytes;
+  L.rows          = volume / seg;
+  const uint64_t tile = static_cast<uint64_t>(global_tile(key_bytes, L.big));
+  const uint64_t tpr  = (seg + tile - 1) / tile;
+  L.num_tiles         = tpr * L.rows;
+  L.valid             = (tpr < (1ull << 32)) && (L.num_tiles < (1ull << 32));
+  L.tiles_per_row     = static_cast<uint32_t>(tpr);
+  const uint64_t ow   = L.big ? 8 : 4;
+  L.off_hist          = HEADER_BYTES;
+  L.hist_bytes        = align_up(L.rows * L.passes * RADIX * ow, WORKSPACE_ALIGN);
+  L.off_desc          = L.off_hist + L.hist_bytes;
+  L.desc_bytes_per_pass = align_up(L.num_tiles * RADIX * ow, WORKSPACE_ALIGN);
+  L.zero_bytes        = L.off_desc + L.desc_bytes_per_pass * L.passes;
+  uint64_t off        = L.zero_bytes;
+  L.key_bytes_total   = align_up(volume * key_bytes, WORKSPACE_ALIGN);
+  L.off_key1 = L.off_key2 = 0;
+  bool need_key1, need_key2;
+  if (L.passes == 1) {
+    need_key1 = want_values && in_place;
+    need_key2 = false;
+  } else {
+    need_key1 = true;
+    need_key2 = !want_values && L.passes >= 3;
+  }
+  if (need_key1) {
+    L.off_key1 = off;
+    off += L.key_bytes_total;
+  }
+  if (need_key2) {
+    L.off_key2 = off;
+    off += L.key_bytes_total;
+  }
+  L.off_idx         = 0;
+  L.idx_bytes_total = align_up(volume * ow, WORKSPACE_ALIGN);
+  if (want_indices && L.passes >= 2) {
+    L.off_idx = off;
+    off += L.idx_bytes_total;
+  }
+  L.total = off;
+  return L;
+}
+
+inline uint64_t workspace_bytes(int key_bytes, uint64_t volume, uint64_t seg, bool want_values,
+                                bool want_indices, bool in_place)
+{
+  if (volume == 0 || seg <= lds_row_limit(key_bytes)) {
+    return HEADER_BYTES;
+  }
+  const GlobalLayout L = global_layout(key_bytes, volume, seg, want_values, want_indices, in_place);
+  return L.valid ? L.total : 0;
+}
+
+inline int launch_zero_fill(void* p, uint64_t bytes, hipStream_t stream)
+{
+  const uint64_t n_vec = bytes / 16;  // bytes is a multiple of 256
+  uint64_t blocks      = (n_vec + 255) / 256;
+  if (blocks > 4096) {
+    blocks = 4096;
+  }
+  if (blocks == 0) {
+    return CPN_OK;
+  }
+  hipLaunchKernelGGL(zero_fill_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, stream,
+                     static_cast<uint4*>(p), n_vec);
+  CPN_HIP_TRY(hipGetLastError());
+  return CPN_OK;
+}
+
+// ---- per-row LDS path ------------------------------------------------------------------
+template <typename KeyT, int CODEC, bool HAS_IDX, int BLOCK, int ITEMS>
+inline int launch_lds_rows(const SortRequest& r)
+{
+  const uint64_t rows = r.volume / r.seg;
+  hipLaunchKernelGGL((lds_row_sort_kernel<KeyT, CODEC, HAS_IDX, BLOCK, ITEMS>),
+                     dim3(static_cast<uint32_t>(rows)), dim3(BLOCK), 0, r.stream,
+                     static_cast<const KeyT*>(r.values_in), static_cast<KeyT*>(r.values_out), r.indices_out,
+                     static_cast<uint32_t>(r.seg), r.index_offset);
+  CPN_HIP_TRY(hipGetLastError());
+  return CPN_OK;
+}
+
+// Rows are bucketed by length; each bucket has its own workgroup shape.
+template <typename KeyT, int CODEC, bool HAS_IDX>
+inline int sort_rows_in_lds(const SortRequest& r)
+{
+  if (r.volume / r.seg >= (1ull << 31)) {
+    return CPN_ERR_UNSUPPORTED;
+  }
+  if (r.seg <= 64) {
+    return launch_lds_rows<KeyT, CODEC, HAS_IDX, 64, 1>(r);
+  } else if (r.seg <= 256) {
+    return launch_lds_rows<KeyT, CODEC, HAS_IDX, 64, 4>(r);
+  } else if (r.seg <= 1024) {
+    return launch_lds_rows<KeyT, CODEC, HAS_IDX, 256, 4>(r);
+  } else if (r.seg <= 4096) {
+    return launch_lds_rows<KeyT, CODEC, HAS_IDX, 256, 16>(r);
+  } else {
+    if constexpr (sizeof(KeyT) < 8) {
+      return launch_lds_rows<KeyT, CODEC, HAS_IDX, 512, 16>(r);
+    } else {
+      return CPN_ERR_UNSUPPORTED;  // not reached: lds_row_limit(8) == 4096
+    }
+  }
+}
+
+// ---- global onesweep path --------------------------------------------------------------
+template <typename KeyT, int CODEC, bool BIG, bool HAS_IDX>
+inline int sort_global(const SortRequest& r, const GlobalLayout& L)
+{
+  using OffT           = typename RowWidth<BIG>::off_t;
+  constexpr int KB     = sizeof(KeyT);
+  constexpr int BLOCK  = global_block(KB);
+  constexpr int ITEMS  = global_items(KB, BIG);
+  constexpr int PASSES = KB;
+  unsigned char* ws    = static_cast<unsigned char*>(r.temp);
+  const bool in_place  = (r.values_out == r.values_in);
+  const bool want_vals = (r.values_out != nullptr);
+
+  int rc = launch_zero_fill(ws, L.zero_bytes, r.stream);
+  if (rc != CPN_OK) {
+    return rc;
+  }
+  uint32_t* status  = reinterpret_cast<uint32_t*>(ws);
+  uint32_t* tickets = reinterpret_cast<uint32_t*>(ws + HEADER_TICKETS);
+  OffT* hist        = reinterpret_cast<OffT*>(ws + L.off_hist);
+
+  // histogram sweep: about 2048 blocks in total, at least one per row
+  {
+    uint64_t bpr = 2048 / L.rows;
+    if (bpr < 1) {
+      bpr = 1;
+    }
+    const uint64_t min_chunk = 16384;
+    const uint64_t max_bpr   = (r.seg + min_chunk - 1) / min_chunk;
+    if (bpr > max_bpr) {
+      bpr = max_bpr;
+    }
+    uint64_t chunk = (r.seg + bpr - 1) / bpr;
+    chunk          = align_up(chunk, 4096);
+    bpr            = (r.seg + chunk - 1) / chunk;
+    const uint64_t grid = bpr * L.rows;
+    if (grid >= (1ull << 31)) {
+      return CPN_ERR_UNSUPPORTED;
+    }
+    hipLaunchKernelGGL((histogram_kernel<KeyT, CODEC, OffT>), dim3(static_cast<uint32_t>(grid)),
+                       dim3(HIST_BLOCK), 0, r.stream, static_cast<const KeyT*>(r.values_in), hist, r.seg,
+                       static_cast<uint32_t>(bpr), chunk);
+    CPN_HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL((histogram_scan_kernel<OffT>), dim3(static_cast<uint32_t>(L.rows * PASSES)),
+                       dim3(RADIX), 0, r.stream, hist);
+    CPN_HIP_TRY(hipGetLastError());
+  }
+
+  // key buffers: the last pass writes the caller's array (or nothing), earlier passes
+  // alternate, walking backwards, between workspace buffer 1 and X = values_out or buffer 2
+  void* key1 = L.off_key1 ? ws + L.off_key1 : nullptr;
+  void* key2 = L.off_key2 ? ws + L.off_key2 : nullptr;
+  void* keyX = want_vals ? r.values_out : key2;
+  void* idx1 = L.off_idx ? ws + L.off_idx : nullptr;
+  void* idxX = r.indices_out;  // the int64 output doubles as a narrow scratch array
+
+  const void* key_src = r.values_in;
+  const void* idx_src = nullptr;
+  for (int p = 0; p < PASSES; ++p) {
+    const bool last      = (p == PASSES - 1);
+    const int from_last  = PASSES - 1 - p;
+    void* key_dst;
+    void* idx_dst = nullptr;
+    if (last) {
+      key_dst = (PASSES == 1 && want_vals && in_place) ? key1 : r.values_out;
+    } else {
+      key_dst = (from_last & 1) ? key1 : keyX;
+    }
+    if constexpr (HAS_IDX) {
+      idx_dst = last ? static_cast<void*>(r.indices_out) : ((from_last & 1) ? idx1 : idxX);
+    }
+    SweepArgs<BIG> a{};
+    a.keys_in         = key_src;
+    a.keys_out        = key_dst;
+    a.idx_in          = static_cast<const OffT*>(idx_src);
+    a.idx_out         = idx_dst;
+    a.ticket          = tickets + p;
+    a.hist_excl       = hist + p * RADIX;
+    a.desc            = reinterpret_cast<OffT*>(ws + L.off_desc + L.desc_bytes_per_pass * p);
+    a.status          = status;
+    a.seg             = r.seg;
+    a.hist_row_stride = static_cast<uint64_t>(PASSES) * RADIX;
+    a.index_offset    = r.index_offset;
+    a.tiles_per_row   = L.tiles_per_row;
+    a.num_tiles       = static_cast<uint32_t>(L.num_tiles);
+    a.shift           = p * RADIX_BITS;
+    a.idx_final       = last ? 1 : 0;
+    hipLaunchKernelGGL((onesweep_kernel<KeyT, CODEC, BIG, HAS_IDX, BLOCK, ITEMS>),
+                       dim3(static_cast<uint32_t>(L.num_tiles)), dim3(BLOCK), 0, r.stream, a);
+    CPN_HIP_TRY(hipGetLastError());
+    key_src = key_dst;
+    idx_src = idx_dst;
+  }
+  if (PASSES == 1 && want_vals && in_place) {
+    CPN_HIP_TRY(hipMemcpyAsync(r.values_out, key1, r.volume * KB, hipMemcpyDeviceToDevice, r.stream));
+  }
+  return CPN_OK;
+}
+
+template <typename KeyT, int CODEC>
+int sort_typed(const SortRequest& r)
+{
+  constexpr int KB    = sizeof(KeyT);
+  const bool has_idx  = (r.indices_out != nullptr);
+  const bool in_place = (r.values_out == r.values_in);
+  const uint64_t need = workspace_bytes(KB, r.volume, r.seg, r.values_out != nullptr, has_idx, in_place);
+  if (need == 0) {
+    return CPN_ERR_UNSUPPORTED;
+  }
+  if (r.temp == nullptr || r.temp_bytes < need || (reinterpret_cast<uintptr_t>(r.temp) % WORKSPACE_ALIGN) != 0) {
+    return CPN_ERR_TEMP;
+  }
+  if (r.seg <= lds_row_limit(KB)) {
+    const int rc = launch_zero_fill(r.temp, HEADER_BYTES, r.stream);
+    if (rc != CPN_OK) {
+      return rc;
+    }
+    return has_idx ? sort_rows_in_lds<KeyT, CODEC, true>(r) : sort_rows_in_lds<KeyT, CODEC, false>(r);
+  }
+  const GlobalLayout L = global_layout(KB, r.volume, r.seg, r.values_out != nullptr, has_idx, in_place);
+  if (L.big) {
+    return has_idx ? sort_global<KeyT, CODEC, true, true>(r, L) : sort_global<KeyT, CODEC, true, false>(r, L);
+  }
+  return has_idx ? sort_global<KeyT, CODEC, false, true>(r, L) : sort_global<KeyT, CODEC, false, false>(r, L);
+}
+
+// One translation unit per key width instantiates these (keeps hipcc runs parallel).
+int sort_keys8(int codec, const SortRequest& r);
+int sort_keys16(int codec, const SortRequest& r);
+int sort_keys32(int codec, const SortRequest& r);
+int sort_keys64(int codec, const SortRequest& r);
+
+}  // namespace cpn

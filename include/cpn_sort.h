@@ -1,0 +1,143 @@
+/*
+ * cpn_sort.h -- C ABI of the MI355X (gfx950) sort / argsort library `libcpnsort.so`.
+ *
+ * The library replaces the single-processor GPU sort of cuPyNumeric's SORT task.  In the
+ * reference that work sits behind typed, plain pointer+size functions
+ *
+ *   local_sort<CODE>(const VAL* values_in, VAL* values_out, const int64_t* indices_in,
+ *                    int64_t* indices_out, size_t volume, size_t sort_dim_size,
+ *                    bool stable, cudaStream_t)            src/cupynumeric/sort/sort.cu:63-96
+ *   cub_local_sort(...)   x12 dtypes                        src/cupynumeric/sort/cub_sort.h:21-115
+ *   thrust_local_sort(...) x14 dtypes                       src/cupynumeric/sort/thrust_sort.h:21-145
+ *
+ * which SortImplBody<GPU> (src/cupynumeric/sort/sort.cu:1797-1940) calls after it has picked
+ * the output/temporary buffers.  The entry points below are what a binding for that call
+ * site links against.  Everything is `extern "C"`, takes raw device pointers, sizes and a
+ * `hipStream_t` passed as `void*`; no C++ or torch types cross the boundary.
+ *
+ * All functions are asynchronous with respect to the host unless stated otherwise, never
+ * abort the process and never free caller memory.  They return CPN_OK (0) or a negative
+ * cpn_status.  The caller owns every buffer, including the temporary workspace.
+ */
+#ifndef CPN_SORT_H
+#define CPN_SORT_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Element type codes.  Order follows the per-dtype instantiation list of the reference
+ * (src/cupynumeric/sort/cub_sort.h:21-115, thrust_sort.h:129-145). */
+typedef enum cpn_dtype {
+  CPN_BOOL       = 0,
+  CPN_INT8       = 1,
+  CPN_INT16      = 2,
+  CPN_INT32      = 3,
+  CPN_INT64      = 4,
+  CPN_UINT8      = 5,
+  CPN_UINT16     = 6,
+  CPN_UINT32     = 7,
+  CPN_UINT64     = 8,
+  CPN_FLOAT16    = 9,
+  CPN_FLOAT32    = 10,
+  CPN_FLOAT64    = 11,
+  CPN_COMPLEX64  = 12,
+  CPN_COMPLEX128 = 13
+} cpn_dtype;
+
+typedef enum cpn_status {
+  CPN_OK              = 0,
+  CPN_ERR_DTYPE       = -1, /* unknown or unsupported element type code              */
+  CPN_ERR_NULL        = -2, /* a required pointer is NULL                              */
+  CPN_ERR_SHAPE       = -3, /* sort_dim_size is 0 or does not divide volume, bad axes  */
+  CPN_ERR_TEMP        = -4, /* workspace missing, too small or not 256-byte aligned    */
+  CPN_ERR_ALIGN       = -5, /* a data pointer is not aligned to its element size       */
+  CPN_ERR_HIP         = -6, /* a HIP runtime call failed (see cpn_last_hip_error)      */
+  CPN_ERR_DEVICE      = -7, /* a kernel flagged an internal failure (bounded wait hit) */
+  CPN_ERR_UNSUPPORTED = -8  /* valid request that this build does not implement        */
+} cpn_status;
+
+/* Library version, (major << 16) | minor. */
+int cpn_sort_version(void);
+
+/* Static, human readable text for a cpn_status value. */
+const char* cpn_status_string(int status);
+
+/* hipError_t of the last HIP call that failed on the calling thread (0 if none). */
+int cpn_last_hip_error(void);
+
+/*
+ * Process-wide tunable: rows of at most `limit` elements are sorted by the one-workgroup-
+ * per-row LDS kernel, longer rows by the global radix sort.  Values above the kernel's
+ * capacity are clamped to it, a negative value restores the default; the previous setting is
+ * returned (-1 = default).  Also initialised from the environment variable
+ * CPN_SORT_LDS_ROW_LIMIT.  Plays the role of the reference's compile-time
+ * SEGMENT_THRESHOLD_RADIX_SORT (src/cupynumeric/sort/sort.cu:41).  Sizes returned by
+ * cpn_local_sort_temp_bytes depend on it: do not change it between the size query and the sort.
+ */
+int64_t cpn_set_lds_row_limit(int64_t limit);
+
+/* Size in bytes of one element of `dtype`, or 0 for an unknown code. */
+uint64_t cpn_dtype_size(int dtype);
+
+/*
+ * Workspace size, in bytes, that cpn_local_sort needs for this request.  Pure host
+ * arithmetic (no HIP call); returns 0 when the request itself is invalid.  Replaces the
+ * size query of cub::DeviceRadixSort (src/cupynumeric/sort/cub_sort.cuh:56-63).
+ *
+ *   want_values  != 0  sorted values are written (values_out != NULL)
+ *   want_indices != 0  int64 indices are written (indices_out != NULL)
+ *   in_place     != 0  values_out aliases values_in
+ */
+uint64_t cpn_local_sort_temp_bytes(int dtype, uint64_t volume, uint64_t sort_dim_size,
+                                   int want_values, int want_indices, int in_place);
+
+/*
+ * Stable sort of `volume / sort_dim_size` independent rows of `sort_dim_size` elements,
+ * dense row-major.  Replaces local_sort<CODE> (src/cupynumeric/sort/sort.cu:63-96) together
+ * with the index initialisation that precedes it (sort.cu:1851-1863, sort.h:83-92).
+ *
+ *   values_in    device pointer, read only unless it equals values_out
+ *   values_out   sorted values (same element type), may equal values_in; NULL when only
+ *                indices are wanted
+ *   indices_out  int64 position of every sorted element inside its row plus index_offset
+ *                (the reference's `i % sort_dim_size + offset`); NULL for a plain sort
+ *   stable       accepted for signature parity; the result is always stable, which
+ *                satisfies both settings
+ *   temp         workspace of at least cpn_local_sort_temp_bytes(...) bytes, 256-byte
+ *                aligned; its contents are undefined afterwards
+ *   stream       hipStream_t (NULL = the null stream)
+ *
+ * Ordering is NumPy's: integers by value, bool false < true, floating point ascending with
+ * every NaN after +inf, and -0.0 equal to +0.0 (ties keep input order).  Bit patterns of
+ * the elements are moved unchanged.  volume == 0 is a successful no-op.
+ */
+int cpn_local_sort(int dtype, const void* values_in, void* values_out, int64_t* indices_out,
+                   uint64_t volume, uint64_t sort_dim_size, int64_t index_offset, int stable,
+                   void* temp, uint64_t temp_bytes, void* stream);
+
+/*
+ * Blocks until `stream` has finished, then reports what the kernels of the last
+ * cpn_local_sort call that used `temp` recorded in its status word: CPN_OK, or
+ * CPN_ERR_DEVICE when a bounded wait inside a kernel ran out (the output is then invalid).
+ * The reference has no counterpart: device failures abort the process there
+ * (src/cupynumeric/cuda_help.h:167-180).
+ */
+int cpn_local_sort_check(const void* temp, void* stream);
+
+/*
+ * out = in with axes `axis_a` and `axis_b` exchanged, both dense row-major; `shape` is the
+ * shape of `in`.  Replaces the UNARY_OP(COPY) of a transposed store that sort_swapped
+ * issues (cupynumeric/_thunk/_sort.py:50-76, src/cupynumeric/unary/unary_op.cu:85-96,124-170).
+ * elem_bytes is 1, 2, 4, 8 or 16; ndim <= 8; in and out must not overlap.
+ */
+int cpn_swapaxes_copy(int elem_bytes, const void* in, void* out, const int64_t* shape, int ndim,
+                      int axis_a, int axis_b, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* CPN_SORT_H */
