@@ -1,0 +1,337 @@
+#!/usr/bin/env python3
+"""Benchmark of the sort hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--log2n L] [--no-cpu-baseline]
+
+A step is one pass of the hot path (one `cpn_local_sort` call, plus the two transposes for the
+axis-0 config) over one batch of synthetic input that already sits in HBM.  The default
+workload is the one the headline metric is quoted on: stable argsort of 2^28 float32 keys with
+1 % NaN and 1 % signed zeros (seed 1), int64 indices out.  One JSON line is printed.
+
+Timing follows the reference's microbenchmark loop (`examples/_benchmark/timer.py:199-241`,
+`examples/microbenchmarks/sort_bench.py:104-130`): warm-up calls, then K calls between two
+device synchronisations.  The `roofline` object is for the dominant kernel (the onesweep scatter
+pass, or the per-row LDS sort): algorithmic bytes per launch divided by its average launch
+duration, measured with HIP events that the library records on its own stream.  The
+`cpu_baseline` object times the CPU restatement of the reference's CPU/OpenMP variant
+(oracle/sort_oracle.c) on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_BYTES_PER_S = 8.0e12  # MI355X HBM3E
+
+# HBM bytes per onesweep launch of the default workload, from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE runs scaled by a copy kernel of known size (profiles/onesweep_c2_traffic.txt).
+# None until that measurement exists for the workload being run.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+# -------------------------------------------------------------------------------------------------
+# workloads (the five configurations of the baseline; `log2n` / `rows` shrink them for tests)
+# -------------------------------------------------------------------------------------------------
+def make_config(name: str, log2n: int | None = None, rows: int | None = None) -> dict:
+    """Seeded synthetic input of one workload as a host array plus what to do with it."""
+    if name == "c1":
+        n = 1 << (24 if log2n is None else log2n)
+        rng = np.random.default_rng(0)
+        x = rng.integers(-(2**31), 2**31, size=n, dtype=np.int64).astype(np.int32)
+        return dict(name=name, x=x, op="sort", axis=-1,
+                    workload=f"c1: np.sort int32 1-D N=2^{int(np.log2(n))}, uniform over int32, seed 0")
+    if name == "c2":
+        n = 1 << (28 if log2n is None else log2n)
+        rng = np.random.default_rng(1)
+        x = rng.standard_normal(n, dtype=np.float32)
+        u = rng.random(n)
+        x[u < 0.01] = np.nan
+        m = (u >= 0.01) & (u < 0.02)
+        x[m] = np.where(rng.random(int(m.sum())) < 0.5, np.float32(-0.0), np.float32(0.0))
+        return dict(name=name, x=x, op="argsort", axis=-1,
+                    workload=f"c2: stable argsort float32 1-D N=2^{int(np.log2(n))}, normal + 1% NaN + 1% +-0, "
+                             "seed 1, int64 indices out")
+    if name == "c3":
+        r = 65536 if rows is None else rows
+        rng = np.random.default_rng(2)
+        x = rng.random((r, 1024))
+        return dict(name=name, x=x, op="sort", axis=-1,
+                    workload=f"c3: np.sort float64 ({r},1024) last axis, uniform [0,1), seed 2")
+    if name == "c4":
+        n = 1 << (27 if log2n is None else log2n)
+        rng = np.random.default_rng(3)
+        vals = rng.integers(-(2**63), 2**63 - 1, size=16, dtype=np.int64)
+        x = vals[rng.integers(0, 16, size=n)]
+        return dict(name=name, x=x, op="argsort", axis=-1,
+                    workload=f"c4: stable argsort int64 1-D N=2^{int(np.log2(n))}, 16 distinct keys, seed 3, "
+                             "int64 indices out")
+    if name == "c5":
+        r = 8192 if rows is None else rows
+        rng = np.random.default_rng(4)
+        x = rng.standard_normal((r, r)).astype(np.float16)
+        return dict(name=name, x=x, op="sort", axis=0,
+                    workload=f"c5: np.sort float16 ({r},{r}) axis 0, normal, seed 4")
+    raise ValueError(f"unknown config {name}")
+
+
+def algorithmic_bytes(cfg: dict, lds_limit_rows: bool) -> dict:
+    """Bytes the algorithm has to move, per kernel kind.  `kb` key bytes, `ib` = 4-byte row
+    positions between passes (rows shorter than 2^30) and 8-byte int64 on the final write."""
+    x = cfg["x"]
+    n = x.size
+    kb = x.dtype.itemsize
+    argsort = cfg["op"] == "argsort"
+    out = {"n": n, "kb": kb}
+    if lds_limit_rows:
+        # one read of the keys, one write of values or of int64 indices
+        out["lds_row_sort"] = n * (kb + (8 if argsort else kb))
+    else:
+        passes = kb
+        per_pass = []
+        for p in range(passes):
+            first, last = p == 0, p == passes - 1
+            r = kb + (0 if (first or not argsort) else 4)
+            if argsort:
+                w = (0 if last else kb) + (8 if last else 4)
+            else:
+                w = kb
+            per_pass.append(n * (r + w))
+        out["onesweep_per_pass"] = per_pass
+        out["onesweep"] = sum(per_pass) / passes  # average launch
+        out["histogram"] = n * kb
+    if cfg["axis"] == 0:
+        out["transpose_last"] = n * 2 * kb
+    return out
+
+
+# -------------------------------------------------------------------------------------------------
+# GPU side
+# -------------------------------------------------------------------------------------------------
+class GpuJob:
+    """Device buffers and the call sequence of one workload, through the C ABI."""
+
+    def __init__(self, cfg: dict):
+        import torch
+
+        from cupynumeric_amd import _lib
+
+        self.torch = torch
+        self.lib = _lib.load()
+        self._lib_mod = _lib
+        if not torch.cuda.is_available():
+            raise RuntimeError("bench.py needs a HIP device")
+        dev = torch.device("cuda:0")
+        x = cfg["x"]
+        self.cfg = cfg
+        self.code = _lib.DTYPE_CODES[x.dtype]
+        self.kb = x.dtype.itemsize
+        self.argsort = cfg["op"] == "argsort"
+        self.transposed = cfg["axis"] == 0
+        self.shape = x.shape
+        self.volume = x.size
+        self.seg = x.shape[0] if self.transposed else x.shape[-1]
+        self.d_in = torch.from_numpy(x.reshape(-1).view(np.uint8)).to(dev)
+        self.d_val = None if self.argsort else torch.empty_like(self.d_in)
+        self.d_idx = torch.empty(self.volume, dtype=torch.int64, device=dev) if self.argsort else None
+        self.d_tr = torch.empty_like(self.d_in) if self.transposed else None
+        in_place = self.transposed  # the transposed copy is sorted in place, as sort_swapped does
+        self.temp_bytes = self.lib.cpn_local_sort_temp_bytes(
+            self.code, self.volume, self.seg, int(not self.argsort), int(self.argsort), int(in_place)
+        )
+        self.temp = torch.empty(self.temp_bytes, dtype=torch.uint8, device=dev)
+        self.stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        self.uses_lds_rows = self.temp_bytes == 256
+
+    def step(self) -> None:
+        lib, ck = self.lib, self._lib_mod.check
+        if self.transposed:
+            r, c = self.shape
+            shape = (ctypes.c_int64 * 2)(r, c)
+            ck(lib.cpn_swapaxes_copy(self.kb, self.d_in.data_ptr(), self.d_tr.data_ptr(), shape, 2, 0, 1, self.stream),
+               "cpn_swapaxes_copy")
+            ck(lib.cpn_local_sort(self.code, self.d_tr.data_ptr(), self.d_tr.data_ptr(), None, self.volume, self.seg,
+                                  0, 1, self.temp.data_ptr(), self.temp_bytes, self.stream), "cpn_local_sort")
+            shape_t = (ctypes.c_int64 * 2)(c, r)
+            ck(lib.cpn_swapaxes_copy(self.kb, self.d_tr.data_ptr(), self.d_val.data_ptr(), shape_t, 2, 0, 1,
+                                     self.stream), "cpn_swapaxes_copy")
+        else:
+            ck(lib.cpn_local_sort(
+                self.code, self.d_in.data_ptr(), None if self.argsort else self.d_val.data_ptr(),
+                self.d_idx.data_ptr() if self.argsort else None, self.volume, self.seg, 0, 1,
+                self.temp.data_ptr(), self.temp_bytes, self.stream), "cpn_local_sort")
+
+    def check_status(self) -> None:
+        self._lib_mod.check(self.lib.cpn_local_sort_check(self.temp.data_ptr(), self.stream), "cpn_local_sort")
+
+    def result(self) -> np.ndarray:
+        if self.argsort:
+            return self.d_idx.cpu().numpy().reshape(self.shape)
+        return self.d_val.cpu().numpy().view(self.cfg["x"].dtype).reshape(self.shape)
+
+
+def verify_sample(job: GpuJob, cfg: dict) -> str:
+    """Cheap end-of-run sanity check on the device result (full parity lives in tests/)."""
+    torch = job.torch
+    if cfg["op"] == "argsort" and cfg["x"].ndim == 1:
+        idx = job.d_idx
+        keys = job.d_in.view(torch.float32 if cfg["x"].dtype == np.float32 else torch.int64)[idx]
+        a, b = keys[:-1], keys[1:]
+        if keys.dtype.is_floating_point:
+            ordered = bool(((a <= b) | torch.isnan(b)).all())
+            tie = (a == b) | (torch.isnan(a) & torch.isnan(b))
+        else:
+            ordered = bool((a <= b).all())
+            tie = a == b
+        stable = bool((idx[1:][tie] > idx[:-1][tie]).all())
+        seen = torch.zeros(idx.numel(), dtype=torch.bool, device=idx.device)
+        seen[idx] = True
+        perm = bool(seen.all())
+        return "ok" if (ordered and stable and perm) else f"FAILED ordered={ordered} stable={stable} permutation={perm}"
+    return "not checked here"
+
+
+# -------------------------------------------------------------------------------------------------
+# CPU baseline: restatement of the reference's CPU / OpenMP variant on a bounded sample
+# -------------------------------------------------------------------------------------------------
+def cpu_baseline(cfg: dict) -> dict:
+    from oracle import sort_oracle as oracle
+
+    x = cfg["x"]
+    argsort = cfg["op"] == "argsort"
+    if x.ndim == 1:
+        sample = x[: min(x.size, 1 << 24)]
+        what = f"first 2^{int(np.log2(sample.size))} keys of the workload"
+    elif cfg["axis"] == 0:
+        sample = np.ascontiguousarray(x[:, : min(x.shape[1], 512)].T)
+        what = f"{sample.shape[0]} columns of the workload (transposes not timed)"
+    else:
+        sample = x[: min(x.shape[0], 8192)]
+        what = f"first {sample.shape[0]} rows of the workload"
+    threads = min(oracle.max_threads(), os.cpu_count() or 1, 16)
+    best = None
+    for t in sorted({1, threads}):
+        t0 = time.perf_counter()
+        oracle.local_sort(sample, argsort=argsort, stable=True, threads=t)
+        dt = time.perf_counter() - t0
+        rate = sample.size / dt
+        if best is None or rate > best[0]:
+            best = (rate, t, dt)
+    return {
+        "value": best[0],
+        "unit": "keys/s",
+        "cores": best[1],
+        "kind": "port",
+        "sample": f"{what}; oracle/sort_oracle.c (stable merge sort per row, OpenMP inside a row as in "
+                  f"thrust::omp::par), {best[2]:.2f} s",
+    }
+
+
+# -------------------------------------------------------------------------------------------------
+def main() -> None:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--log2n", type=int, default=None, help="shrink a 1-D workload to 2^L keys")
+    ap.add_argument("--rows", type=int, default=None, help="shrink a 2-D workload to this many rows")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build sorts on one GPU; --gpus must be 1 (no multi-GPU sample sort is built)")
+
+    cfg = make_config(args.config, args.log2n, args.rows)
+    job = GpuJob(cfg)
+    torch = job.torch
+    lib = job.lib
+    from cupynumeric_amd import _lib
+
+    for _ in range(args.warmup):
+        job.step()
+    torch.cuda.synchronize()
+    job.check_status()
+
+    lib.cpn_profile_enable(1)
+    _lib.profile_collect()  # drop anything recorded earlier
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        job.step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    lib.cpn_profile_enable(0)
+    records = _lib.profile_collect()
+    job.check_status()
+
+    ms_per_step = elapsed * 1e3 / args.steps
+    keys_per_s = cfg["x"].size / (elapsed / args.steps)
+
+    # per-kernel launch durations from the library's HIP events
+    by_label: dict[str, list[float]] = {}
+    for label, ms in records:
+        by_label.setdefault(label, []).append(ms)
+    alg = algorithmic_bytes(cfg, job.uses_lds_rows)
+    dominant = "lds_row_sort" if job.uses_lds_rows else "onesweep"
+    avg_ms = float(np.mean(by_label[dominant]))
+    achieved = alg[dominant] / (avg_ms * 1e-3)
+    kernels = {
+        label: {"launches_per_step": len(v) / args.steps, "avg_ms": float(np.mean(v)),
+                "algorithmic_GBps": (alg[label] / (float(np.mean(v)) * 1e-3) / 1e9) if label in alg else None}
+        for label, v in by_label.items()
+    }
+    traffic = MEASURED_TRAFFIC_BYTES.get((args.config, cfg["x"].size))
+    roofline = {
+        "kernel": dominant,
+        "bound": "hbm",
+        "achieved": achieved / 1e9,
+        "peak": HBM_PEAK_BYTES_PER_S / 1e9,
+        "unit": "GB/s",
+        "frac": achieved / HBM_PEAK_BYTES_PER_S,
+        "traffic": traffic,
+        "bytes_per_launch": alg[dominant],
+        "avg_launch_ms": avg_ms,
+        "launches_per_step": len(by_label[dominant]) / args.steps,
+    }
+    step_bytes = sum(alg.get(k, 0) * len(v) / args.steps for k, v in by_label.items() if k in alg)
+
+    line = {
+        "metric": "sorted keys/sec, stable argsort fp32 N=2^28, 1 GPU" if args.config == "c2" and args.log2n is None
+        else f"sorted keys/sec, config {args.config}, 1 GPU",
+        "value": keys_per_s,
+        "unit": "keys/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": {1: "u8", 2: "u16", 4: "u32", 8: "u64"}[cfg["x"].dtype.itemsize],
+        "data": "synthetic",
+        "config": {"workload": cfg["workload"], "keys": int(cfg["x"].size), "op": cfg["op"],
+                   "path": "lds_row_sort" if job.uses_lds_rows else "onesweep, 8-bit digits",
+                   "workspace_bytes": int(job.temp_bytes)},
+        "roofline": roofline,
+        "whole_step": {"algorithmic_bytes": step_bytes, "GBps": step_bytes / (elapsed / args.steps) / 1e9,
+                       "frac_of_hbm_peak": step_bytes / (elapsed / args.steps) / HBM_PEAK_BYTES_PER_S},
+        "kernels": kernels,
+        "verify": verify_sample(job, cfg),
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(cfg)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

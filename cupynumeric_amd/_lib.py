@@ -51,12 +51,15 @@ PROTOTYPES: dict[str, tuple] = {
     "cpn_last_hip_error": (c_int, []),
     "cpn_set_lds_row_limit": (c_int64, [c_int64]),
     "cpn_dtype_size": (c_uint64, [c_int]),
+    "cpn_key_order_bits": (c_uint64, [c_int, c_uint64]),
     "cpn_local_sort_temp_bytes": (c_uint64, [c_int, c_uint64, c_uint64, c_int, c_int, c_int]),
     "cpn_local_sort": (
         c_int,
         [c_int, c_void_p, c_void_p, c_void_p, c_uint64, c_uint64, c_int64, c_int, c_void_p, c_uint64, c_void_p],
     ),
     "cpn_local_sort_check": (c_int, [c_void_p, c_void_p]),
+    "cpn_profile_enable": (c_int, [c_int]),
+    "cpn_profile_collect": (c_int, [c_void_p, c_uint64, c_void_p, c_int]),
     "cpn_swapaxes_copy": (c_int, [c_int, c_void_p, c_void_p, ctypes.POINTER(c_int64), c_int, c_int, c_int, c_void_p]),
 }
 
@@ -92,6 +95,17 @@ def load() -> ctypes.CDLL:
         fn.argtypes = argtypes
     _lib = lib
     return lib
+
+
+def profile_collect(max_records: int = 65536) -> list[tuple[str, float]]:
+    """(label, milliseconds) of every kernel launch recorded since the last collect."""
+    lib = load()
+    stride = 32
+    labels = ctypes.create_string_buffer(stride * max_records)
+    ms = (ctypes.c_float * max_records)()
+    n = lib.cpn_profile_collect(labels, stride, ms, max_records)
+    raw = labels.raw
+    return [(raw[i * stride : (i + 1) * stride].split(b"\0", 1)[0].decode(), float(ms[i])) for i in range(n)]
 
 
 def status_string(status: int) -> str:

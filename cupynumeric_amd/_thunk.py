@@ -52,6 +52,8 @@ class Storage:
         return int(self.device().data_ptr())
 
     def to_numpy(self, shape: tuple[int, ...], dtype: np.dtype) -> np.ndarray:
+        if 0 in shape:
+            return np.empty(shape, dtype=dtype)  # nothing to fetch; works without a device
         if self._dev is None and self._host is not None:
             return np.array(self._host, dtype=dtype).reshape(shape)
         return runtime.download(self.device(), shape, dtype)

@@ -23,6 +23,7 @@ LIB_PATH = PKG_DIR / "libcpnsort.so"
 SOURCES = [
     "sort_api.hip",
     "swapaxes.hip",
+    "profile.hip",
     "sort_keys8.hip",
     "sort_keys16.hip",
     "sort_keys32.hip",

@@ -90,6 +90,28 @@ int64_t cpn_set_lds_row_limit(int64_t limit)
 
 uint64_t cpn_dtype_size(int dtype) { return static_cast<uint64_t>(cpn::key_kind(dtype).bytes); }
 
+uint64_t cpn_key_order_bits(int dtype, uint64_t raw_bits)
+{
+  const cpn::KeyKind k = cpn::key_kind(dtype);
+  if (k.bytes == 0 || k.codec < 0) {
+    return 0;
+  }
+  switch (k.bytes * 4 + k.codec) {
+    case 1 * 4 + cpn::CODEC_UNSIGNED: return cpn::ordered_bits<cpn::CODEC_UNSIGNED, uint8_t>(static_cast<uint8_t>(raw_bits));
+    case 1 * 4 + cpn::CODEC_SIGNED: return cpn::ordered_bits<cpn::CODEC_SIGNED, uint8_t>(static_cast<uint8_t>(raw_bits));
+    case 2 * 4 + cpn::CODEC_UNSIGNED: return cpn::ordered_bits<cpn::CODEC_UNSIGNED, uint16_t>(static_cast<uint16_t>(raw_bits));
+    case 2 * 4 + cpn::CODEC_SIGNED: return cpn::ordered_bits<cpn::CODEC_SIGNED, uint16_t>(static_cast<uint16_t>(raw_bits));
+    case 2 * 4 + cpn::CODEC_FLOAT: return cpn::ordered_bits<cpn::CODEC_FLOAT, uint16_t>(static_cast<uint16_t>(raw_bits));
+    case 4 * 4 + cpn::CODEC_UNSIGNED: return cpn::ordered_bits<cpn::CODEC_UNSIGNED, uint32_t>(static_cast<uint32_t>(raw_bits));
+    case 4 * 4 + cpn::CODEC_SIGNED: return cpn::ordered_bits<cpn::CODEC_SIGNED, uint32_t>(static_cast<uint32_t>(raw_bits));
+    case 4 * 4 + cpn::CODEC_FLOAT: return cpn::ordered_bits<cpn::CODEC_FLOAT, uint32_t>(static_cast<uint32_t>(raw_bits));
+    case 8 * 4 + cpn::CODEC_UNSIGNED: return cpn::ordered_bits<cpn::CODEC_UNSIGNED, uint64_t>(raw_bits);
+    case 8 * 4 + cpn::CODEC_SIGNED: return cpn::ordered_bits<cpn::CODEC_SIGNED, uint64_t>(raw_bits);
+    case 8 * 4 + cpn::CODEC_FLOAT: return cpn::ordered_bits<cpn::CODEC_FLOAT, uint64_t>(raw_bits);
+    default: return 0;
+  }
+}
+
 uint64_t cpn_local_sort_temp_bytes(int dtype, uint64_t volume, uint64_t sort_dim_size, int want_values,
                                    int want_indices, int in_place)
 {

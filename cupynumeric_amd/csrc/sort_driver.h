@@ -11,6 +11,7 @@
 #include "../../include/cpn_sort.h"
 #include "lds_row_sort.h"
 #include "onesweep.h"
+#include "profile.h"
 
 namespace cpn {
 
@@ -147,8 +148,11 @@ inline int launch_zero_fill(void* p, uint64_t bytes, hipStream_t stream)
   if (blocks == 0) {
     return CPN_OK;
   }
-  hipLaunchKernelGGL(zero_fill_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, stream,
-                     static_cast<uint4*>(p), n_vec);
+  {
+    ProfileScope prof("zero_fill", stream);
+    hipLaunchKernelGGL(zero_fill_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, stream,
+                       static_cast<uint4*>(p), n_vec);
+  }
   CPN_HIP_TRY(hipGetLastError());
   return CPN_OK;
 }
@@ -158,10 +162,13 @@ template <typename KeyT, int CODEC, bool HAS_IDX, int BLOCK, int ITEMS>
 inline int launch_lds_rows(const SortRequest& r)
 {
   const uint64_t rows = r.volume / r.seg;
-  hipLaunchKernelGGL((lds_row_sort_kernel<KeyT, CODEC, HAS_IDX, BLOCK, ITEMS>),
-                     dim3(static_cast<uint32_t>(rows)), dim3(BLOCK), 0, r.stream,
-                     static_cast<const KeyT*>(r.values_in), static_cast<KeyT*>(r.values_out), r.indices_out,
-                     static_cast<uint32_t>(r.seg), r.index_offset);
+  {
+    ProfileScope prof("lds_row_sort", r.stream);
+    hipLaunchKernelGGL((lds_row_sort_kernel<KeyT, CODEC, HAS_IDX, BLOCK, ITEMS>),
+                       dim3(static_cast<uint32_t>(rows)), dim3(BLOCK), 0, r.stream,
+                       static_cast<const KeyT*>(r.values_in), static_cast<KeyT*>(r.values_out), r.indices_out,
+                       static_cast<uint32_t>(r.seg), r.index_offset);
+  }
   CPN_HIP_TRY(hipGetLastError());
   return CPN_OK;
 }
@@ -229,12 +236,18 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
     if (grid >= (1ull << 31)) {
       return CPN_ERR_UNSUPPORTED;
     }
-    hipLaunchKernelGGL((histogram_kernel<KeyT, CODEC, OffT>), dim3(static_cast<uint32_t>(grid)),
-                       dim3(HIST_BLOCK), 0, r.stream, static_cast<const KeyT*>(r.values_in), hist, r.seg,
-                       static_cast<uint32_t>(bpr), chunk);
+    {
+      ProfileScope prof("histogram", r.stream);
+      hipLaunchKernelGGL((histogram_kernel<KeyT, CODEC, OffT>), dim3(static_cast<uint32_t>(grid)),
+                         dim3(HIST_BLOCK), 0, r.stream, static_cast<const KeyT*>(r.values_in), hist, r.seg,
+                         static_cast<uint32_t>(bpr), chunk);
+    }
     CPN_HIP_TRY(hipGetLastError());
-    hipLaunchKernelGGL((histogram_scan_kernel<OffT>), dim3(static_cast<uint32_t>(L.rows * PASSES)),
-                       dim3(RADIX), 0, r.stream, hist);
+    {
+      ProfileScope prof("histogram_scan", r.stream);
+      hipLaunchKernelGGL((histogram_scan_kernel<OffT>), dim3(static_cast<uint32_t>(L.rows * PASSES)),
+                         dim3(RADIX), 0, r.stream, hist);
+    }
     CPN_HIP_TRY(hipGetLastError());
   }
 
@@ -277,8 +290,11 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
     a.num_tiles       = static_cast<uint32_t>(L.num_tiles);
     a.shift           = p * RADIX_BITS;
     a.idx_final       = last ? 1 : 0;
-    hipLaunchKernelGGL((onesweep_kernel<KeyT, CODEC, BIG, HAS_IDX, BLOCK, ITEMS>),
-                       dim3(static_cast<uint32_t>(L.num_tiles)), dim3(BLOCK), 0, r.stream, a);
+    {
+      ProfileScope prof("onesweep", r.stream);
+      hipLaunchKernelGGL((onesweep_kernel<KeyT, CODEC, BIG, HAS_IDX, BLOCK, ITEMS>),
+                         dim3(static_cast<uint32_t>(L.num_tiles)), dim3(BLOCK), 0, r.stream, a);
+    }
     CPN_HIP_TRY(hipGetLastError());
     key_src = key_dst;
     idx_src = idx_dst;

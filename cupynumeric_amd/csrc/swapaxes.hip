@@ -100,6 +100,7 @@ static int swapaxes_typed(const void* in, void* out, uint64_t P, uint64_t A, uin
     if (tiles_a >= (1ull << 31) || tiles_b >= (1ull << 31) || grid >= (1ull << 31)) {
       return CPN_ERR_UNSUPPORTED;
     }
+    ProfileScope prof("transpose_last", stream);
     hipLaunchKernelGGL((transpose_last_kernel<T, TS>), dim3(static_cast<uint32_t>(grid)), dim3(256), 0, stream,
                        static_cast<const T*>(in), static_cast<T*>(out), A, M, B, static_cast<uint32_t>(tiles_a),
                        static_cast<uint32_t>(tiles_b));
@@ -108,6 +109,7 @@ static int swapaxes_typed(const void* in, void* out, uint64_t P, uint64_t A, uin
     if (grid > 65536) {
       grid = 65536;
     }
+    ProfileScope prof("swapaxes_generic", stream);
     hipLaunchKernelGGL((swapaxes_generic_kernel<T>), dim3(static_cast<uint32_t>(grid)), dim3(256), 0, stream,
                        static_cast<const T*>(in), static_cast<T*>(out), A, M, B, Q, total);
   }

@@ -83,6 +83,16 @@ int64_t cpn_set_lds_row_limit(int64_t limit);
 uint64_t cpn_dtype_size(int dtype);
 
 /*
+ * Host-side image of the key transform the kernels apply before extracting radix digits:
+ * the unsigned integer (of the element's width) whose natural order is the sort order of
+ * the element with raw bit pattern `raw_bits`.  Pure host arithmetic, for tests and
+ * debugging.  Stands where the reference relies on cub's radix key traits
+ * (src/cupynumeric/sort/cub_sort.cuh:60-71); unlike those it maps every NaN to the maximum
+ * and -0.0 to the key of +0.0.  Returns 0 for unknown or unsupported codes.
+ */
+uint64_t cpn_key_order_bits(int dtype, uint64_t raw_bits);
+
+/*
  * Workspace size, in bytes, that cpn_local_sort needs for this request.  Pure host
  * arithmetic (no HIP call); returns 0 when the request itself is invalid.  Replaces the
  * size query of cub::DeviceRadixSort (src/cupynumeric/sort/cub_sort.cuh:56-63).
@@ -135,6 +145,20 @@ int cpn_local_sort_check(const void* temp, void* stream);
  */
 int cpn_swapaxes_copy(int elem_bytes, const void* in, void* out, const int64_t* shape, int ndim,
                       int axis_a, int axis_b, void* stream);
+
+/*
+ * Per-launch timing.  cpn_profile_enable(1) makes every kernel launch of the library record
+ * a pair of HIP events on the stream it is launched on; it returns the previous setting.
+ * cpn_profile_collect waits for the recorded events, writes up to `max_records` entries --
+ * a NUL-terminated label ("histogram", "onesweep", "lds_row_sort", "transpose_last", ...) of
+ * at most label_stride-1 characters at labels + i*label_stride, and the launch duration in
+ * milliseconds at milliseconds[i], in launch order -- returns how many it wrote and forgets
+ * all records (also those it had no room for).  Off by default; meant for benchmarks.  The
+ * reference's counterpart is the Legate profiler range around each API call
+ * (cupynumeric/_utils/profiling.py:37-73).
+ */
+int cpn_profile_enable(int on);
+int cpn_profile_collect(char* labels, uint64_t label_stride, float* milliseconds, int max_records);
 
 #ifdef __cplusplus
 }

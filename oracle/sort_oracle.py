@@ -1,0 +1,142 @@
+"""TEST INFRASTRUCTURE -- CPU oracle for the sort path.  Not part of the product: only tests/,
+`__graft_entry__.smoke()` and `bench.py`'s `cpu_baseline` leg may import this module.
+
+Two layers, mirroring the reference:
+
+* `local_sort` calls the C restatement (`sort_oracle.c`) of `SortImplBodyCpu` /
+  `thrust_local_sort_inplace` (`src/cupynumeric/sort/sort_cpu.inl:52-85,937-1074`): rows of the
+  last axis, stable, NumPy ordering, indices `i % seg + offset`.
+* `sort` / `argsort` restate the Python side: `cupynumeric/_module/ssc_sorting.py:29-121` (result
+  shape and dtype), `DeferredArray.sort` (`cupynumeric/_thunk/deferred.py:5453-5474`: kind -> stable
+  flag, `order` -> NotImplementedError, axis range -> ValueError) and the axis dispatch of
+  `cupynumeric/_thunk/_sort.py:37-136` (flatten / last axis / swap-sort-swap), with NumPy doing the
+  `swapaxes` copies.
+
+Deviation kept on purpose (same as the product): results are always stable.
+"""
+from __future__ import annotations
+
+import ctypes
+import subprocess
+from pathlib import Path
+
+import numpy as np
+from numpy.exceptions import AxisError
+from numpy.lib.array_utils import normalize_axis_index
+
+HERE = Path(__file__).resolve().parent
+LIB_PATH = HERE / "_build" / "libcpnoracle.so"
+
+# same codes as enum cpn_dtype (include/cpn_sort.h); complex is outside the oracle
+DTYPE_CODES = {
+    np.dtype(np.bool_): 0,
+    np.dtype(np.int8): 1,
+    np.dtype(np.int16): 2,
+    np.dtype(np.int32): 3,
+    np.dtype(np.int64): 4,
+    np.dtype(np.uint8): 5,
+    np.dtype(np.uint16): 6,
+    np.dtype(np.uint32): 7,
+    np.dtype(np.uint64): 8,
+    np.dtype(np.float16): 9,
+    np.dtype(np.float32): 10,
+    np.dtype(np.float64): 11,
+}
+
+_lib = None
+
+
+def build(force: bool = False) -> Path:
+    """Compile sort_oracle.c with gcc (see Makefile)."""
+    if force or not LIB_PATH.exists() or LIB_PATH.stat().st_mtime < (HERE / "sort_oracle.c").stat().st_mtime:
+        subprocess.run(["make", "-C", str(HERE), "-B" if force else "-s"], check=True, capture_output=True)
+    return LIB_PATH
+
+
+def load() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not LIB_PATH.exists():
+            build()
+        lib = ctypes.CDLL(str(LIB_PATH))
+        lib.cpn_oracle_local_sort.restype = ctypes.c_int
+        lib.cpn_oracle_local_sort.argtypes = [
+            ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+            ctypes.c_uint64, ctypes.c_uint64, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+        ]
+        lib.cpn_oracle_max_threads.restype = ctypes.c_int
+        _lib = lib
+    return _lib
+
+
+def max_threads() -> int:
+    return int(load().cpn_oracle_max_threads())
+
+
+def local_sort(x: np.ndarray, argsort: bool, stable: bool = True, offset: int = 0, threads: int = 1):
+    """Sort the rows (last axis) of a C-contiguous array.  Returns sorted values, or int64 row
+    positions when `argsort`."""
+    x = np.ascontiguousarray(x)
+    if x.dtype not in DTYPE_CODES:
+        raise TypeError(f"cuPyNumeric does not support dtype={x.dtype}")
+    values = np.empty_like(x)
+    indices = np.empty(x.shape, dtype=np.int64) if argsort else None
+    seg = x.shape[-1] if x.ndim > 0 else 1
+    if x.size:
+        rc = load().cpn_oracle_local_sort(
+            DTYPE_CODES[x.dtype],
+            x.ctypes.data,
+            values.ctypes.data,
+            indices.ctypes.data if argsort else None,
+            x.size,
+            seg,
+            offset,
+            int(stable),
+            threads,
+        )
+        if rc != 0:
+            raise RuntimeError(f"cpn_oracle_local_sort failed: {rc}")
+    return indices if argsort else values
+
+
+def _sort_deferred(x: np.ndarray, argsort: bool, axis, stable: bool, threads: int) -> np.ndarray:
+    # cupynumeric/_thunk/_sort.py:110-136
+    if x.ndim == 0:
+        if axis is not None:
+            raise AxisError(axis, x.ndim)
+        return np.zeros(1, dtype=np.int64) if argsort else x.copy()
+    if axis is None and x.ndim > 1:
+        return _sort_deferred(x.reshape(-1), argsort, -1, stable, threads)  # sort_flattened :37-47
+    computed_axis = 0 if axis is None else normalize_axis_index(axis, x.ndim)
+    if computed_axis == x.ndim - 1:
+        return local_sort(x, argsort, stable, 0, threads)  # sort_task :79-107
+    # sort_swapped :50-76
+    swapped_copy = np.ascontiguousarray(np.swapaxes(x, computed_axis, x.ndim - 1))
+    res = local_sort(swapped_copy, argsort, stable, 0, threads)
+    return np.ascontiguousarray(np.swapaxes(res, x.ndim - 1, computed_axis))
+
+
+def _thunk_sort(x: np.ndarray, argsort: bool, axis, kind: str, order, threads: int) -> np.ndarray:
+    # cupynumeric/_thunk/deferred.py:5453-5474
+    stable = kind == "stable"
+    if order is not None:
+        raise NotImplementedError(
+            "cuPyNumeric does not support sorting with 'order' as ndarray only supports numeric values"
+        )
+    if axis is not None and (axis >= x.ndim or axis < -x.ndim):
+        raise ValueError("invalid axis")
+    return _sort_deferred(x, argsort, axis, stable, threads)
+
+
+def sort(a, axis=-1, kind="quicksort", order=None, threads: int = 1) -> np.ndarray:
+    x = np.asarray(a)
+    if x.dtype not in DTYPE_CODES:
+        raise TypeError(f"cuPyNumeric does not support dtype={x.dtype}")
+    return _thunk_sort(x, False, axis, kind, order, threads)
+
+
+def argsort(a, axis=-1, kind="quicksort", order=None, threads: int = 1) -> np.ndarray:
+    x = np.asarray(a)
+    if x.dtype not in DTYPE_CODES:
+        raise TypeError(f"cuPyNumeric does not support dtype={x.dtype}")
+    return _thunk_sort(x, True, axis, kind, order, threads)

@@ -1,0 +1,199 @@
+"""CPU-only checks of the host side: the C-ABI library loads and exports every symbol the header
+declares, pure-host entry points behave, the Python layer validates arguments like the
+reference, and the product has no CPU fallback."""
+from __future__ import annotations
+
+import re
+from pathlib import Path
+
+import numpy as np
+import pytest
+from conftest import ALL_REAL_DTYPES, ROOT, make_input
+
+import cupynumeric_amd as num
+from cupynumeric_amd import _lib
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return _lib.load()
+
+
+def test_every_declared_symbol_is_exported(lib):
+    header = (ROOT / "include" / "cpn_sort.h").read_text()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(cpn_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations found in include/cpn_sort.h"
+    assert declared == set(_lib.PROTOTYPES), "ctypes prototypes and header differ"
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared but not exported"
+
+
+def test_dtype_codes_match_header():
+    header = (ROOT / "include" / "cpn_sort.h").read_text()
+    codes = dict(re.findall(r"CPN_([A-Z0-9]+)\s*=\s*(\d+)", header))
+    names = {"BOOL": np.bool_, "INT8": np.int8, "INT16": np.int16, "INT32": np.int32, "INT64": np.int64,
+             "UINT8": np.uint8, "UINT16": np.uint16, "UINT32": np.uint32, "UINT64": np.uint64,
+             "FLOAT16": np.float16, "FLOAT32": np.float32, "FLOAT64": np.float64,
+             "COMPLEX64": np.complex64, "COMPLEX128": np.complex128}
+    for name, np_type in names.items():
+        assert _lib.DTYPE_CODES[np.dtype(np_type)] == int(codes[name])
+
+
+def test_version_status_strings_and_sizes(lib):
+    assert lib.cpn_sort_version() >= 1
+    assert lib.cpn_status_string(0) == b"ok"
+    for status in range(-8, 0):
+        assert lib.cpn_status_string(status) not in (b"ok", b"unknown status")
+    assert lib.cpn_status_string(-99) == b"unknown status"
+    for dt, code in _lib.DTYPE_CODES.items():
+        assert lib.cpn_dtype_size(code) == dt.itemsize
+    assert lib.cpn_dtype_size(99) == 0
+
+
+def test_argument_validation_without_a_device(lib):
+    # every check below fails before the first HIP call
+    sort = lib.cpn_local_sort
+    assert sort(99, 16, 16, None, 4, 4, 0, 1, 256, 256, None) == _lib.CPN_ERR_DTYPE
+    assert sort(3, None, None, None, 0, 0, 0, 1, None, 0, None) == _lib.CPN_OK  # volume 0: no-op
+    assert sort(3, 16, 32, None, 10, 3, 0, 1, 256, 256, None) == _lib.CPN_ERR_SHAPE  # 3 does not divide 10
+    assert sort(3, 16, 32, None, 10, 0, 0, 1, 256, 256, None) == _lib.CPN_ERR_SHAPE
+    assert sort(3, None, 32, None, 4, 4, 0, 1, 256, 256, None) == _lib.CPN_ERR_NULL
+    assert sort(3, 16, None, None, 4, 4, 0, 1, 256, 256, None) == _lib.CPN_ERR_NULL  # no output at all
+    assert sort(3, 18, 32, None, 4, 4, 0, 1, 256, 256, None) == _lib.CPN_ERR_ALIGN
+    assert sort(3, 16, None, 36, 4, 4, 0, 1, 256, 256, None) == _lib.CPN_ERR_ALIGN  # int64 out misaligned
+    assert sort(3, 16, 32, None, 4, 4, 0, 1, None, 0, None) == _lib.CPN_ERR_TEMP
+    assert sort(3, 16, 32, None, 4, 4, 0, 1, 256, 16, None) == _lib.CPN_ERR_TEMP  # too small
+    assert sort(3, 16, 32, None, 4, 4, 0, 1, 264, 4096, None) == _lib.CPN_ERR_TEMP  # misaligned
+    assert sort(12, 16, 32, None, 4, 4, 0, 1, 256, 256, None) == _lib.CPN_ERR_UNSUPPORTED  # complex64
+    assert lib.cpn_local_sort_check(None, None) == _lib.CPN_ERR_NULL
+    swap = lib.cpn_swapaxes_copy
+    import ctypes
+
+    shape = (ctypes.c_int64 * 2)(3, 4)
+    assert swap(4, 16, 64, shape, 2, 0, 2, None) == _lib.CPN_ERR_SHAPE
+    assert swap(3, 16, 64, shape, 2, 0, 1, None) == _lib.CPN_ERR_SHAPE
+    assert swap(4, None, 64, shape, 2, 0, 1, None) == _lib.CPN_ERR_NULL
+    assert swap(4, 18, 64, shape, 2, 0, 1, None) == _lib.CPN_ERR_ALIGN
+    empty = (ctypes.c_int64 * 2)(0, 4)
+    assert swap(4, None, None, empty, 2, 0, 1, None) == _lib.CPN_OK
+
+
+def test_temp_bytes_layout(lib):
+    tb = lib.cpn_local_sort_temp_bytes
+    f32, i64, u8, f16 = 10, 4, 5, 9
+    assert tb(99, 100, 100, 1, 0, 0) == 0
+    assert tb(f32, 100, 7, 1, 0, 0) == 0  # 7 does not divide 100
+    assert tb(f32, 0, 0, 1, 0, 0) == 256
+    assert tb(f32, 1 << 20, 1024, 1, 1, 0) == 256  # rows that fit LDS need only the status header
+    n = 1 << 24
+    tiles = n // 8192
+    fixed = 256 + 4 * 256 * 4 + 4 * tiles * 256 * 4
+    assert tb(f32, n, n, 1, 0, 0) == fixed + 4 * n  # one key buffer
+    assert tb(f32, n, n, 1, 0, 1) == fixed + 4 * n  # in place, even pass count: same
+    assert tb(f32, n, n, 0, 1, 0) == fixed + 2 * 4 * n + 4 * n  # index-only: two key buffers + narrow indices
+    assert tb(f32, n, n, 1, 1, 0) == fixed + 4 * n + 4 * n
+    # 8-bit keys take one pass: no key buffer unless sorting in place
+    t8 = 256 + 256 * 4 + tiles * 256 * 4
+    assert tb(u8, n, n, 1, 0, 0) == t8
+    assert tb(u8, n, n, 1, 0, 1) == t8 + n
+    assert tb(u8, n, n, 0, 1, 0) == t8
+    # monotone in the request
+    assert tb(i64, n, n, 0, 1, 0) > tb(f32, n, n, 0, 1, 0) > tb(f16, n, n, 0, 1, 0)
+    # the row-length switch moves work to the global path
+    prev = lib.cpn_set_lds_row_limit(0)
+    try:
+        assert tb(f32, 1 << 20, 1024, 1, 1, 0) > 256
+    finally:
+        lib.cpn_set_lds_row_limit(prev)
+    assert tb(f32, 1 << 20, 1024, 1, 1, 0) == 256
+
+
+@pytest.mark.parametrize("dtype", ALL_REAL_DTYPES)
+def test_key_transform_orders_like_numpy(lib, dtype):
+    """Sorting by the library's key transform (a stable integer sort) must reproduce NumPy's
+    stable argsort: pins NaN-last, -0 == +0 and the signed/unsigned flips on the host."""
+    dt = np.dtype(dtype)
+    code = _lib.DTYPE_CODES[dt]
+    ub = {1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[dt.itemsize]
+    if dt.itemsize <= 2:
+        raw = np.arange(1 << (8 * dt.itemsize), dtype=np.uint32).astype(ub)  # every bit pattern
+        if dt.kind == "b":
+            raw = np.array([0, 1], dtype=ub)
+        raw = np.random.default_rng(0).permutation(raw)
+    else:
+        raw = make_input(dtype, (20000,), seed=3).view(ub)
+    x = raw.view(dt)
+    keys = np.array([lib.cpn_key_order_bits(code, int(b)) for b in raw], dtype=np.uint64)
+    assert np.array_equal(np.argsort(keys, kind="stable"), np.argsort(x, kind="stable"))
+    assert int(keys.max()) < (1 << (8 * dt.itemsize)) or dt.itemsize == 8
+
+
+# ---- Python layer: the reference's observable behaviour, no GPU needed ----------------------------
+def test_python_validation_before_any_device_work():
+    a = num.array(np.arange(6, dtype=np.int32).reshape(2, 3))
+    # cupynumeric/_thunk/deferred.py:5471-5472, tests/integration/test_sort.py:67-70
+    for axis in (2, -3):
+        with pytest.raises(ValueError, match="invalid axis"):
+            num.sort(a, axis=axis)
+        with pytest.raises(ValueError, match="invalid axis"):
+            num.argsort(a, axis=axis)
+        with pytest.raises(ValueError, match="invalid axis"):
+            a.sort(axis=axis)
+    with pytest.raises(ValueError):
+        num.sort([-1, 0, 1, 2, 10], axis=2)
+    # cupynumeric/_thunk/deferred.py:5466-5470
+    with pytest.raises(NotImplementedError, match="does not support sorting with 'order'"):
+        num.sort(a, order="x")
+    # cupynumeric/_utils/array.py:64-68, tests/integration/test_sort.py:185-192
+    with pytest.raises(TypeError, match="cuPyNumeric does not support dtype="):
+        num.sort(np.array(["a", "b", "c"]))
+    with pytest.raises(TypeError, match="cuPyNumeric does not support dtype="):
+        num.array(np.array(["a"]))
+    # 0-D with an axis: the ValueError of the thunk pre-empts AxisError
+    # (tests/integration/test_sort.py:249-264)
+    with pytest.raises(ValueError):
+        num.sort(num.array(np.int32(3)), axis=0)
+
+
+def test_result_metadata_of_empty_inputs():
+    # tests/integration/test_sort.py:60-65: no device work is needed for empty arrays
+    for arr in ([], [[]], [[], []]):
+        res = num.sort(arr)
+        assert np.array_equal(res, np.sort(arr))
+        idx = num.argsort(arr)
+        assert np.array_equal(idx, np.argsort(arr))
+        assert idx.dtype == np.int64
+    for shape in [(0,), (0, 1), (1, 0), (1, 0, 0), (1, 1, 0), (1, 0, 1)]:
+        x = np.zeros(shape, dtype=np.int32)
+        for axis in range(-len(shape) + 1, len(shape)):
+            assert num.sort(x, axis=axis).shape == shape
+            assert num.argsort(x, axis=axis).shape == shape
+        assert num.sort(x, axis=None).shape == (0,)
+
+
+def test_no_cpu_fallback():
+    """Without a HIP device the sort must fail loudly instead of computing on the host."""
+    import torch
+
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        num.sort(np.array([3, 1, 2], dtype=np.int32))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        num.argsort(np.array([[3.0, 1.0], [2.0, 0.0]]), axis=0)
+
+
+def test_product_does_not_reach_the_oracle():
+    """Nothing under cupynumeric_amd/ may import or load the CPU oracle."""
+    for path in (ROOT / "cupynumeric_amd").rglob("*"):
+        if path.suffix in (".py", ".h", ".hip"):
+            text = path.read_text()
+            assert "oracle" not in text.lower(), f"{path} mentions the oracle"
+
+
+def test_missing_library_is_an_error(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "libcpnsort.so")
+    with pytest.raises(_lib.NativeLibraryError, match="no CPU fallback"):
+        _lib.load()

@@ -1,0 +1,153 @@
+"""Pins the CPU oracle (oracle/sort_oracle.py + sort_oracle.c) before anything is checked
+against it: the reference's golden vectors, NumPy's independent stable sort, closed forms and a
+brute-force insertion sort on adversarial float alphabets.  CPU only."""
+from __future__ import annotations
+
+import itertools
+
+import numpy as np
+import pytest
+from conftest import ALL_REAL_DTYPES, assert_same_bits, make_input
+
+from oracle import sort_oracle as oracle
+
+
+# ---- golden vectors of the reference's own tests ------------------------------------------------
+def test_reference_golden_vectors(reference_vectors):
+    assert len(reference_vectors) == 300
+    for case in reference_vectors:
+        x = np.array(case["input"], dtype=case["dtype"]).reshape(case["shape"])
+        # kinds the reference runs the case with (tests/cpp/integration/test_argsort.cc:221-224)
+        kinds = ["mergesort", "stable"] if case["stable_only"] else ["quicksort", "mergesort", "heapsort", "stable"]
+        for kind in kinds:
+            if case["op"] == "sort":
+                got = oracle.sort(x, axis=case["axis"], kind=kind)
+                want = np.array(case["expect"], dtype=case["dtype"]).reshape(case["shape"])
+            else:
+                got = oracle.argsort(x, axis=case["axis"], kind=kind)
+                want = np.array(case["expect"], dtype=np.int64).reshape(case["shape"])
+            assert_same_bits(got, want, f"{case['where']} shape={case['shape']} axis={case['axis']} kind={kind}")
+
+
+def test_reference_large_reversed():
+    # tests/cpp/integration/test_argsort.cc:379-410: 10 000 descending values -> N-1-j
+    count = 10000
+    want = count - 1 - np.arange(count, dtype=np.int64)
+    assert np.array_equal(oracle.argsort(np.array([count - i for i in range(count)], dtype=np.int32)), want)
+    assert np.array_equal(oracle.argsort(np.array([count * 1.1 - i for i in range(count)], dtype=np.float64)), want)
+
+
+@pytest.mark.parametrize("shape", [(0,), (0, 1), (1, 0), (1, 0, 0), (1, 1, 0), (1, 0, 1)])
+def test_reference_empty(shape):
+    # tests/cpp/integration/test_argsort.cc:412-433, test_sort.cc:574-594
+    x = np.zeros(shape, dtype=np.int32)
+    for axis in range(-len(shape) + 1, len(shape)):
+        assert oracle.sort(x, axis=axis).shape == shape
+        assert oracle.argsort(x, axis=axis).shape == shape
+        assert oracle.argsort(x, axis=axis).dtype == np.int64
+
+
+@pytest.mark.parametrize("shape", [(1,), (1, 1), (1, 1, 1)])
+def test_reference_single_item(shape):
+    # tests/cpp/integration/test_argsort.cc:435-455, test_sort.cc:596-615
+    x = np.full(shape, 12, dtype=np.int32)
+    for axis in range(-len(shape) + 1, len(shape)):
+        assert np.array_equal(oracle.sort(x, axis=axis), x)
+        assert np.array_equal(oracle.argsort(x, axis=axis), np.zeros(shape, dtype=np.int64))
+
+
+def test_reference_negative():
+    # tests/cpp/integration/test_argsort.cc:457-467 (invalid axis); Python side raises ValueError
+    # (cupynumeric/_thunk/deferred.py:5471-5472, tests/integration/test_sort.py:67-70)
+    x = np.zeros((2, 3), dtype=np.int32)
+    for axis in (2, -3):
+        with pytest.raises(ValueError):
+            oracle.argsort(x, axis=axis)
+        with pytest.raises(ValueError):
+            oracle.sort(x, axis=axis)
+    with pytest.raises(NotImplementedError):
+        oracle.sort(x, order="a")
+    with pytest.raises(TypeError, match="cuPyNumeric does not support dtype="):
+        oracle.sort(np.array(["a", "b"]))
+
+
+# ---- NumPy's own stable sort as an independent implementation ------------------------------------
+@pytest.mark.parametrize("dtype", ALL_REAL_DTYPES)
+@pytest.mark.parametrize("threads", [1, 4])
+def test_against_numpy_1d(dtype, threads):
+    for n in (1, 2, 3, 17, 24, 25, 1000, 70001):
+        x = make_input(dtype, (n,), seed=n)
+        assert np.array_equal(oracle.argsort(x, kind="stable", threads=threads), np.argsort(x, kind="stable"))
+        assert_same_bits(oracle.sort(x, kind="stable", threads=threads), np.sort(x, kind="stable"), f"{dtype} n={n}")
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.float32, np.float16, np.float64, np.uint8])
+def test_against_numpy_axes(dtype):
+    for shape in [(5, 5), (7, 1, 9), (3, 4, 5, 6), (33, 65)]:
+        x = make_input(dtype, shape, seed=len(shape))
+        for axis in list(range(-len(shape), len(shape))) + [None]:
+            assert np.array_equal(oracle.argsort(x, axis=axis, kind="stable"), np.argsort(x, axis=axis, kind="stable"))
+            assert_same_bits(oracle.sort(x, axis=axis), np.sort(x, axis=axis, kind="stable"), f"{shape} axis={axis}")
+
+
+def test_parallel_segment_matches_serial():
+    x = make_input(np.float32, (3, 200000), seed=5)
+    assert np.array_equal(oracle.argsort(x, threads=1), oracle.argsort(x, threads=oracle.max_threads()))
+
+
+# ---- closed forms ------------------------------------------------------------------------------
+def test_closed_forms():
+    n = 5003
+    iota = np.arange(n, dtype=np.int64)
+    assert np.array_equal(oracle.argsort(np.full(n, 7, dtype=np.int16)), iota)  # all equal -> identity
+    assert np.array_equal(oracle.argsort(iota.astype(np.float32)), iota)  # sorted -> identity
+    assert np.array_equal(oracle.argsort(-iota), iota[::-1])  # reversed distinct
+    perm = np.random.default_rng(1).permutation(n)
+    inv = np.empty(n, dtype=np.int64)
+    inv[perm] = iota
+    assert np.array_equal(oracle.argsort(perm.astype(np.uint32)), inv)  # argsort of a permutation = inverse
+    # row-relative indices: every row of an N-D argsort is a permutation of 0..seg-1
+    idx = oracle.argsort(make_input(np.int8, (11, 300), seed=2))
+    assert np.array_equal(np.sort(idx, axis=-1), np.broadcast_to(np.arange(300), (11, 300)))
+
+
+# ---- brute force over an adversarial float alphabet --------------------------------------------
+def numpy_rule_less(a: float, b: float) -> bool:
+    """a sorts strictly before b: a < b, or b is NaN and a is not."""
+    return bool(a < b or (b != b and a == a))
+
+
+def insertion_argsort(x: np.ndarray) -> list[int]:
+    order: list[int] = []
+    for i, v in enumerate(x):
+        j = len(order)
+        while j > 0 and numpy_rule_less(float(v), float(x[order[j - 1]])):
+            j -= 1
+        order.insert(j, i)
+    return order
+
+
+@pytest.mark.parametrize("dtype,ubits", [(np.float16, np.uint16), (np.float32, np.uint32), (np.float64, np.uint64)])
+def test_bruteforce_float_alphabet(dtype, ubits):
+    dt = np.dtype(dtype)
+    nan = np.array(np.nan, dtype=dt).view(ubits)
+    sign = ubits(1) << ubits(dt.itemsize * 8 - 1)
+    alphabet_bits = [
+        nan, nan | sign, nan | ubits(1),  # +NaN, -NaN, NaN with payload
+        np.array(-np.inf, dtype=dt).view(ubits), np.array(np.inf, dtype=dt).view(ubits),
+        np.array(-1.0, dtype=dt).view(ubits), np.array(1.0, dtype=dt).view(ubits),
+        sign, ubits(0),  # -0.0, +0.0
+        ubits(1), sign | ubits(1),  # smallest subnormals
+    ]
+    alphabet = np.array(alphabet_bits, dtype=ubits).view(dt)
+    # all length-3 words over the alphabet, plus a long random word
+    for word in itertools.product(range(len(alphabet)), repeat=3):
+        x = alphabet[list(word)]
+        got = oracle.argsort(x, kind="stable")
+        assert got.tolist() == insertion_argsort(x), (dtype, word)
+        assert_same_bits(oracle.sort(x), x[got])
+    rng = np.random.default_rng(7)
+    x = alphabet[rng.integers(0, len(alphabet), 400)]
+    got = oracle.argsort(x, kind="stable")
+    assert got.tolist() == insertion_argsort(x)
+    assert_same_bits(oracle.sort(x), x[got])

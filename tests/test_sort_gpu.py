@@ -1,0 +1,282 @@
+"""GPU parity tests: the HIP sort path (through the C ABI and through the Python API on top of
+it) against the CPU oracle, the reference's golden vectors and NumPy.  Integer, byte and index
+results must be bit-exact; float values are compared by bit pattern as well."""
+from __future__ import annotations
+
+import ctypes
+
+import numpy as np
+import pytest
+from conftest import ALL_REAL_DTYPES, assert_same_bits, make_input
+
+import cupynumeric_amd as num
+from cupynumeric_amd import _lib
+from oracle import sort_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return _lib.load()
+
+
+@pytest.fixture(scope="module")
+def torch_cuda():
+    import torch
+
+    assert torch.cuda.is_available(), "these tests need a HIP device"
+    return torch
+
+
+@pytest.fixture()
+def global_path(lib):
+    """Send every row, however short, down the global onesweep path."""
+    prev = lib.cpn_set_lds_row_limit(0)
+    yield
+    lib.cpn_set_lds_row_limit(prev)
+
+
+def abi_sort(lib, torch, x: np.ndarray, want_values=True, want_indices=False, in_place=False, offset=0):
+    """Call cpn_local_sort directly on torch-owned device buffers; returns (values, indices)."""
+    x = np.ascontiguousarray(x)
+    dev = torch.device("cuda")
+    seg = x.shape[-1]
+    volume = x.size
+    code = _lib.DTYPE_CODES[x.dtype]
+    d_in = torch.from_numpy(x.reshape(-1).view(np.uint8).copy()).to(dev)
+    d_val = d_in if in_place else (torch.zeros_like(d_in) if want_values else None)
+    d_idx = torch.full((volume,), -7, dtype=torch.int64, device=dev) if want_indices else None
+    tb = lib.cpn_local_sort_temp_bytes(code, volume, seg, int(want_values), int(want_indices), int(in_place))
+    assert tb >= 256
+    temp = torch.empty(tb, dtype=torch.uint8, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rc = lib.cpn_local_sort(
+        code, d_in.data_ptr(), d_val.data_ptr() if want_values else None,
+        d_idx.data_ptr() if want_indices else None, volume, seg, offset, 1, temp.data_ptr(), tb, stream,
+    )
+    assert rc == 0, _lib.status_string(rc)
+    assert lib.cpn_local_sort_check(temp.data_ptr(), stream) == 0
+    vals = d_val.cpu().numpy().view(x.dtype).reshape(x.shape) if want_values else None
+    idx = d_idx.cpu().numpy().reshape(x.shape) if want_indices else None
+    if not in_place:  # the input must not be touched
+        assert np.array_equal(d_in.cpu().numpy(), x.reshape(-1).view(np.uint8))
+    return vals, idx
+
+
+def check_rows(lib, torch, x, what):
+    want_v = oracle.local_sort(x, argsort=False)
+    want_i = oracle.local_sort(x, argsort=True)
+    v, _ = abi_sort(lib, torch, x, want_values=True, want_indices=False)
+    assert_same_bits(v, want_v, f"{what} sort")
+    _, i = abi_sort(lib, torch, x, want_values=False, want_indices=True)
+    assert_same_bits(i, want_i, f"{what} argsort")
+    return want_v, want_i
+
+
+# ---- golden vectors of the reference, through the public API ------------------------------------
+def test_reference_golden_vectors(reference_vectors):
+    for case in reference_vectors:
+        x = np.array(case["input"], dtype=case["dtype"]).reshape(case["shape"])
+        a = num.array(x)
+        kinds = ["mergesort", "stable"] if case["stable_only"] else ["quicksort", "mergesort", "heapsort", "stable"]
+        for kind in kinds:
+            where = f"{case['where']} shape={case['shape']} axis={case['axis']} kind={kind}"
+            if case["op"] == "sort":
+                want = np.array(case["expect"], dtype=case["dtype"]).reshape(case["shape"])
+                assert_same_bits(np.asarray(num.sort(a, axis=case["axis"], kind=kind)), want, where)
+            else:
+                want = np.array(case["expect"], dtype=np.int64).reshape(case["shape"])
+                assert_same_bits(np.asarray(num.argsort(a, axis=case["axis"], kind=kind)), want, where)
+                assert_same_bits(np.asarray(a.argsort(axis=case["axis"], kind=kind)), want, where)
+
+
+def test_reference_large_reversed():
+    # tests/cpp/integration/test_argsort.cc:379-410
+    count = 10000
+    want = count - 1 - np.arange(count, dtype=np.int64)
+    for x in (np.array([count - i for i in range(count)], dtype=np.int32),
+              np.array([count * 1.1 - i for i in range(count)], dtype=np.float64)):
+        for kind in ("quicksort", "mergesort", "heapsort", "stable"):
+            assert np.array_equal(np.asarray(num.argsort(x, axis=0, kind=kind)), want)
+
+
+# ---- the reference's integration tests, case for case --------------------------------------------
+DIM = 5
+SIZES = [(0,), (1), (DIM), (0, 1), (1, 0), (1, 1), (1, DIM), (DIM, 1), (DIM, DIM), (1, 0, 0), (1, 1, 0),
+         (1, 0, 1), (1, 1, 1), (DIM, 1, 1), (1, DIM, 1), (1, 1, DIM), (DIM, DIM, DIM)]
+SORT_TYPES = ["quicksort", "mergesort", "heapsort", "stable"]
+
+
+@pytest.mark.parametrize("size", SIZES)
+def test_integration_sort_and_argsort(size):
+    # tests/integration/test_sort.py:84-125, test_argsort.py (same structure); duplicates are
+    # present, so every kind is held to the stable result
+    rng = np.random.default_rng(hash(str(size)) & 0xFFFF)
+    arr_np = rng.integers(-100, 100, size)
+    arr_num = num.array(arr_np)
+    for kind in SORT_TYPES:
+        for axis in range(-arr_np.ndim + 1, arr_np.ndim):
+            assert np.array_equal(num.sort(arr_num, axis=axis, kind=kind), np.sort(arr_np, axis=axis, kind="stable"))
+            assert np.array_equal(num.sort(arr_num, axis=axis, kind=kind), oracle.sort(arr_np, axis=axis, kind=kind))
+            assert np.array_equal(
+                num.argsort(arr_num, axis=axis, kind=kind), np.argsort(arr_np, axis=axis, kind="stable")
+            )
+            assert np.array_equal(
+                arr_num.argsort(axis=axis, kind=kind), oracle.argsort(arr_np, axis=axis, kind=kind)
+            )
+            in_place = num.array(arr_np)
+            in_place.sort(axis=axis, kind=kind)
+            assert np.array_equal(in_place, np.sort(arr_np, axis=axis, kind="stable"))
+
+
+@pytest.mark.parametrize("size", [s for s in SIZES if not isinstance(s, int)] + [(DIM,)])
+def test_integration_axis_none(size):
+    # tests/integration/test_sort.py:194-225
+    arr_np = np.random.default_rng(3).integers(-100, 100, size)
+    arr_num = num.array(arr_np)
+    res = num.sort(arr_num, axis=None)
+    assert res.shape == (arr_np.size,)
+    assert np.array_equal(res, np.sort(arr_np, axis=None, kind="stable"))
+    idx = num.argsort(arr_num, axis=None, kind="stable")
+    assert idx.shape == (arr_np.size,)
+    assert np.array_equal(idx, np.argsort(arr_np, axis=None, kind="stable"))
+
+
+def test_random_module_and_flatten():
+    a = num.random.randint(-100, 100, (4, 6))
+    flat = a.flatten()
+    assert flat.shape == (24,)
+    assert np.array_equal(num.sort(flat), np.sort(np.asarray(a).reshape(-1), kind="stable"))
+
+
+# ---- per-row LDS path: every dtype, lengths around every workgroup-shape boundary -------------------
+LDS_LENGTHS = [1, 2, 3, 63, 64, 65, 255, 256, 257, 1000, 1023, 1024, 1025, 4095, 4096, 4097, 8191, 8192]
+
+
+@pytest.mark.parametrize("dtype", ALL_REAL_DTYPES)
+def test_lds_rows_all_dtypes(lib, torch_cuda, dtype):
+    for seg in LDS_LENGTHS:
+        for rows in (1, 3):
+            x = make_input(dtype, (rows, seg), seed=seg * 7 + rows)
+            check_rows(lib, torch_cuda, x, f"{np.dtype(dtype)} rows={rows} seg={seg}")
+
+
+def test_lds_many_short_rows(lib, torch_cuda):
+    for dtype, shape in [(np.float64, (3000, 37)), (np.int8, (5000, 5)), (np.float16, (700, 401)), (np.uint32, (129, 1024))]:
+        check_rows(lib, torch_cuda, make_input(dtype, shape, seed=11), f"{np.dtype(dtype)} {shape}")
+
+
+# ---- global onesweep path ---------------------------------------------------------------------------
+GLOBAL_LENGTHS = [1, 2, 100, 4095, 4096, 4097, 8191, 8192, 8193, 3 * 8192 + 5, 100003]
+
+
+@pytest.mark.parametrize("dtype", ALL_REAL_DTYPES)
+def test_global_path_all_dtypes(lib, torch_cuda, global_path, dtype):
+    for seg in GLOBAL_LENGTHS:
+        x = make_input(dtype, (seg,), seed=seg)
+        check_rows(lib, torch_cuda, x, f"{np.dtype(dtype)} seg={seg} (global)")
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.float32, np.float64, np.uint8, np.float16])
+def test_global_path_batched_rows(lib, torch_cuda, global_path, dtype):
+    # rows shorter than, equal to and longer than a tile; the look-back must stop at row starts
+    for shape in [(50, 129), (7, 4096), (5, 8192), (3, 8193), (4, 20011), (300, 1)]:
+        check_rows(lib, torch_cuda, make_input(dtype, shape, seed=shape[0]), f"{np.dtype(dtype)} {shape} (global)")
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.float32, np.int64, np.float64, np.float16, np.uint8])
+def test_global_path_default_dispatch(lib, torch_cuda, dtype):
+    # long rows take the global path without any override
+    for shape in [(1 << 20,), (3, 70001), (2, 8193)]:
+        check_rows(lib, torch_cuda, make_input(dtype, shape, seed=5), f"{np.dtype(dtype)} {shape}")
+
+
+@pytest.mark.parametrize("path", ["lds", "global"])
+@pytest.mark.parametrize("dtype", [np.uint8, np.int16, np.float32, np.int64])
+def test_outputs_in_place_and_offset(lib, torch_cuda, path, dtype):
+    prev = lib.cpn_set_lds_row_limit(0 if path == "global" else -1)
+    try:
+        for shape in [(4, 3000), (2, 9001)]:
+            x = make_input(dtype, shape, seed=9)
+            want_v = oracle.local_sort(x, argsort=False)
+            want_i = oracle.local_sort(x, argsort=True, offset=1000)
+            v, i = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=True, offset=1000)
+            assert_same_bits(v, want_v, f"values+indices {shape}")
+            assert_same_bits(i, want_i, f"values+indices {shape}")
+            v, _ = abi_sort(lib, torch_cuda, x, want_values=True, in_place=True)
+            assert_same_bits(v, want_v, f"in place {shape}")
+            v, i = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=True, in_place=True, offset=-5)
+            assert_same_bits(v, want_v, f"in place + indices {shape}")
+            assert_same_bits(i, want_i - 1005, f"in place + indices {shape}")
+    finally:
+        lib.cpn_set_lds_row_limit(prev)
+
+
+# ---- adversarial key distributions ------------------------------------------------------------------
+@pytest.mark.parametrize("path", ["lds", "global"])
+def test_skewed_and_degenerate_keys(lib, torch_cuda, path):
+    prev = lib.cpn_set_lds_row_limit(0 if path == "global" else -1)
+    try:
+        n = 8192 if path == "lds" else 200001
+        rng = np.random.default_rng(4)
+        iota = np.arange(n, dtype=np.int64)
+        cases = {
+            "all equal": np.full(n, -3, dtype=np.int32),
+            "sorted": iota.astype(np.int64),
+            "reversed": (-iota).astype(np.int64),
+            "16 distinct int64": rng.integers(-(2**63), 2**63 - 1, 16, dtype=np.int64)[rng.integers(0, 16, n)],
+            "two values": rng.integers(0, 2, n).astype(np.uint16) * np.uint16(40000),
+            "all NaN": np.full(n, np.nan, dtype=np.float32),
+            "NaN and zeros": rng.choice(np.array([np.nan, 0.0, -0.0], dtype=np.float64), n),
+            "bool": rng.integers(0, 2, n).astype(np.bool_),
+        }
+        for name, x in cases.items():
+            _, want_i = check_rows(lib, torch_cuda, x, f"{name} ({path})")
+            if name in ("all equal", "sorted", "all NaN"):
+                assert np.array_equal(want_i, iota)
+            if name == "reversed":
+                assert np.array_equal(want_i, iota[::-1])
+        perm = rng.permutation(n)
+        inv = np.empty(n, dtype=np.int64)
+        inv[perm] = iota
+        _, i = abi_sort(lib, torch_cuda, perm.astype(np.uint32), want_values=False, want_indices=True)
+        assert np.array_equal(i, inv)  # argsort of a permutation is its inverse
+    finally:
+        lib.cpn_set_lds_row_limit(prev)
+
+
+# ---- swapaxes copy ------------------------------------------------------------------------------------
+@pytest.mark.parametrize("elem", [np.uint8, np.float16, np.int32, np.float64, np.complex128])
+def test_swapaxes_copy(lib, torch_cuda, elem):
+    torch = torch_cuda
+    shapes = [((3, 4), 0, 1), ((65, 130), 0, 1), ((64, 64), 1, 0), ((5, 6, 7), 0, 2), ((5, 6, 7), 1, 2), ((5, 6, 7), 0, 1),
+              ((2, 3, 4, 5), 1, 3), ((2, 3, 4, 5), 0, 2), ((1, 12, 1), 1, 2), ((7, 1), 0, 1), ((300, 3), 0, 1),
+              ((4, 5), 1, 1), ((2, 2, 1, 1, 2, 1, 2), 0, 6)]
+    rng = np.random.default_rng(0)
+    for shape, a, b in shapes:
+        x = rng.integers(0, 255, int(np.prod(shape)) * np.dtype(elem).itemsize, dtype=np.uint8).view(elem).reshape(shape)
+        d_in = torch.from_numpy(x.reshape(-1).view(np.uint8).copy()).cuda()
+        d_out = torch.zeros_like(d_in)
+        c_shape = (ctypes.c_int64 * len(shape))(*shape)
+        rc = lib.cpn_swapaxes_copy(np.dtype(elem).itemsize, d_in.data_ptr(), d_out.data_ptr(), c_shape, len(shape), a, b,
+                                   ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0
+        want = np.ascontiguousarray(np.swapaxes(x, a, b))
+        got = d_out.cpu().numpy().view(elem).reshape(want.shape)
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (shape, a, b)
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.float16, np.float64, np.uint8])
+def test_sort_along_other_axes(dtype):
+    for shape in [(100, 70), (5, 6, 7), (65, 130), (2, 3, 4, 5), (1000, 3), (3, 9000)]:
+        x = make_input(dtype, shape, seed=len(shape))
+        a = num.array(x)
+        for axis in range(len(shape)):
+            assert_same_bits(np.asarray(num.sort(a, axis=axis)), oracle.sort(x, axis=axis), f"{shape} axis={axis}")
+            assert_same_bits(np.asarray(num.argsort(a, axis=axis)), oracle.argsort(x, axis=axis), f"{shape} axis={axis}")
+
+
+def test_unsupported_complex_is_reported():
+    with pytest.raises(NotImplementedError):
+        num.sort(np.array([1 + 2j, 0.5 - 1j], dtype=np.complex64))
