@@ -124,10 +124,13 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
     }
     __syncthreads();
     uint32_t rnk[ITEMS];
+    uint32_t dpk[(ITEMS + 3) / 4];  // the digits, four per register
 #pragma unroll
     for (int i = 0; i < ITEMS; ++i) {
       const bool valid = full || (woff + i * WAVE < seg);
-      rnk[i]           = wave_match_rank(radix_digit<CODEC, KeyT>(key[i], shift), valid, wctr);
+      const uint32_t d = radix_digit<CODEC, KeyT>(key[i], shift);
+      dpk[i / 4]       = (i % 4 == 0) ? d : (dpk[i / 4] | (d << (8 * (i % 4))));
+      rnk[i]           = wave_match_rank(d, valid, wctr);
     }
     __syncthreads();
     // exclusive scan over (digit, wave) in digit-major order
@@ -167,7 +170,7 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
 #pragma unroll
     for (int i = 0; i < ITEMS; ++i) {
       if (full || (woff + i * WAVE < seg)) {
-        const uint32_t d   = radix_digit<CODEC, KeyT>(key[i], shift);
+        const uint32_t d   = (dpk[i / 4] >> (8 * (i % 4))) & 0xFFu;
         const uint32_t pos = wctr[d] + rnk[i];
         s_keys[pos]        = key[i];
         if constexpr (HAS_IDX) {

@@ -49,6 +49,12 @@ struct DescBits {
 // that every wave exits even if a predecessor never publishes.
 constexpr uint32_t LOOKBACK_SPIN_LIMIT = 1u << 22;
 
+// Predecessor descriptors each look-back round reads at once.
+#ifndef CPN_LOOKBACK_WINDOW
+#define CPN_LOOKBACK_WINDOW 4
+#endif
+constexpr int LOOKBACK_WINDOW = CPN_LOOKBACK_WINDOW;
+
 // Status word values written by kernels into the workspace header.
 constexpr uint32_t DEVICE_ERR_LOOKBACK = 1u;
 
@@ -200,14 +206,17 @@ __global__ __launch_bounds__(BLOCK) void onesweep_kernel(const SweepArgs<BIG> a)
   using OffT = typename RowWidth<BIG>::off_t;
   using DB   = DescBits<OffT>;
   static_assert(BLOCK >= RADIX, "one thread per digit is needed for the look-back");
+  static_assert(ITEMS % 4 == 0, "digits are cached four to a register");
   constexpr int WAVES      = BLOCK / WAVE;
   constexpr int TILE       = BLOCK * ITEMS;
   constexpr int WTILE      = ITEMS * WAVE;  // keys of one wave, contiguous in the tile
   constexpr int STAGE_ELEM = (HAS_IDX && sizeof(OffT) > sizeof(KeyT)) ? sizeof(OffT) : sizeof(KeyT);
+  static_assert(TILE <= 65536, "positions inside a tile are kept in 16 bits");
 
   __shared__ __align__(16) unsigned char s_stage[TILE * STAGE_ELEM];
+  __shared__ uint8_t s_dig[TILE];  // digit of the key at each sorted position of the tile
   __shared__ uint32_t s_ctr[WAVES * RADIX];
-  __shared__ uint64_t s_gbase[RADIX];
+  __shared__ OffT s_gbase[RADIX];
   __shared__ uint32_t s_wsum[RADIX / WAVE];
   __shared__ uint32_t s_tile;
 
@@ -252,8 +261,164 @@ __global__ __launch_bounds__(BLOCK) void onesweep_kernel(const SweepArgs<BIG> a)
       key[i]           = (o < count) ? kin[o] : static_cast<KeyT>(0);
     }
   }
-  OffT idx[HAS_IDX ? ITEMS : 1];
+
+  // ---- digits, and the tile's digit counts per wave before any ranking ("early counts"):
+  //      the aggregate can be published, and the look-back can start, while the keys are ranked
+  uint32_t dpk[ITEMS / 4];  // the digits, four per register
+  uint32_t* wctr = s_ctr + wave * RADIX;
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t d = radix_digit<CODEC, KeyT>(key[i], a.shift);
+    dpk[i / 4]       = (i % 4 == 0) ? d : (dpk[i / 4] | (d << (8 * (i % 4))));
+    if (full || (woff + i * WAVE < count)) {
+      atomicAdd(&wctr[d], 1u);
+    }
+  }
+  __syncthreads();
+
+  // ---- per digit: start of every wave's keys, tile total, publish, first look-back reads ----
+  uint32_t dsum = 0, dincl = 0;
+  OffT window[LOOKBACK_WINDOW];
+  OffT* my_desc     = a.desc + static_cast<uint64_t>(tile) * RADIX + tid;
+  const uint32_t t0 = tile - trow;  // first tile of the row, always published INCLUSIVE
+  if (tid < RADIX) {
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      const uint32_t c       = s_ctr[w * RADIX + tid];
+      s_ctr[w * RADIX + tid] = dsum;
+      dsum += c;
+    }
+    const OffT first = (trow == 0) ? DB::INCLUSIVE : DB::AGGREGATE;
+    __hip_atomic_store(my_desc, static_cast<OffT>(first | dsum), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (trow != 0) {
+#pragma unroll
+      for (int j = 0; j < LOOKBACK_WINDOW; ++j) {
+        // tiles before the row start are replaced by the row's first tile (the sum stops there)
+        const uint32_t t = (tile - 1 >= t0 + j) ? tile - 1 - j : t0;
+        window[j] = __hip_atomic_load(a.desc + static_cast<uint64_t>(t) * RADIX + tid, __ATOMIC_RELAXED,
+                                      __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    dincl = wave_inclusive_scan(dsum, lane);
+    if (lane == WAVE - 1) {
+      s_wsum[wave] = dincl;
+    }
+  }
+  __syncthreads();
+  uint32_t dexcl = 0;  // start of this digit's keys in the sorted tile
+  if (tid < RADIX) {
+    dexcl = dincl - dsum;
+    for (int w = 0; w < wave; ++w) {
+      dexcl += s_wsum[w];
+    }
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      s_ctr[w * RADIX + tid] += dexcl;
+    }
+  }
+  __syncthreads();
+
+  // ---- rank inside the wave and scatter into LDS: the counters already hold each wave's
+  //      first position per digit, so the rank is the final position in the sorted tile ----
+  KeyT* s_keys = reinterpret_cast<KeyT*>(s_stage);
+  uint32_t pos2[ITEMS / 2];  // positions in the sorted tile, two per register
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const bool valid   = full || (woff + i * WAVE < count);
+    const uint32_t d   = (dpk[i / 4] >> (8 * (i % 4))) & 0xFFu;
+    const uint32_t pos = wave_match_rank(d, valid, wctr);
+    if (valid) {
+      s_keys[pos] = key[i];
+      s_dig[pos]  = static_cast<uint8_t>(d);
+    }
+    pos2[i / 2] = (i % 2 == 0) ? (pos & 0xFFFFu) : (pos2[i / 2] | (pos << 16));
+  }
+
+  // ---- decoupled look-back over the earlier tiles of this row ----
+  // A descriptor written on another XCD is only visible through memory-side accesses, so
+  // one poll costs a full memory round trip.  The first window of predecessors was requested
+  // before the ranking phase; its answers are summed front to back until the first
+  // inclusive one, further windows follow only if none was.
+  if (tid < RADIX) {
+    OffT before = 0;
+    if (trow != 0) {
+      uint32_t hi = tile - 1;  // nearest predecessor not yet accounted for
+      bool done   = false;
+      bool failed = false;
+      while (true) {
+#pragma unroll
+        for (int j = 0; j < LOOKBACK_WINDOW; ++j) {
+          if (!done) {
+            OffT w = window[j];
+            if ((w & DB::STATUS) == 0) {
+              const uint32_t t = (hi >= t0 + j) ? hi - j : t0;
+              const OffT* dp   = a.desc + static_cast<uint64_t>(t) * RADIX + tid;
+              uint32_t spins   = 0;
+              do {
+                if (++spins >= LOOKBACK_SPIN_LIMIT) {
+                  failed = true;
+                  break;
+                }
+                if ((spins & 255u) == 0 &&
+                    __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
+                  failed = true;  // another tile already gave up: drain quickly
+                  break;
+                }
+                __builtin_amdgcn_s_sleep(4);
+                w = __hip_atomic_load(dp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+              } while ((w & DB::STATUS) == 0);
+            }
+            if (failed) {
+              done = true;
+            } else {
+              before += (w & DB::VALUE);
+              if ((w & DB::INCLUSIVE) != 0) {
+                done = true;
+              }
+            }
+          }
+        }
+        if (done) {
+          break;
+        }
+        hi = (hi >= t0 + LOOKBACK_WINDOW) ? hi - LOOKBACK_WINDOW : t0;
+#pragma unroll
+        for (int j = 0; j < LOOKBACK_WINDOW; ++j) {
+          const uint32_t t = (hi >= t0 + j) ? hi - j : t0;
+          window[j] = __hip_atomic_load(a.desc + static_cast<uint64_t>(t) * RADIX + tid, __ATOMIC_RELAXED,
+                                        __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+      if (failed) {
+        __hip_atomic_fetch_or(a.status, DEVICE_ERR_LOOKBACK, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      __hip_atomic_store(my_desc, static_cast<OffT>(DB::INCLUSIVE | (before + dsum)), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+    }
+    // offset inside the row of local sorted position 0 for this digit (unsigned wrap is fine)
+    s_gbase[tid] = a.hist_excl[row * a.hist_row_stride + tid] + before - static_cast<OffT>(dexcl);
+  }
+  __syncthreads();
+
+  // ---- coalesced runs from LDS to HBM ----
+  OffT goff[ITEMS];  // offset in the row of the element at sorted position tid + k*BLOCK
+  KeyT* kout = (a.keys_out != nullptr) ? static_cast<KeyT*>(a.keys_out) + row_base : nullptr;
+#pragma unroll
+  for (int k = 0; k < ITEMS; ++k) {
+    const uint32_t p = tid + k * BLOCK;
+    if (full || p < count) {
+      goff[k] = s_gbase[s_dig[p]] + p;
+      if (kout != nullptr) {
+        kout[goff[k]] = s_keys[p];
+      }
+    } else {
+      goff[k] = 0;
+    }
+  }
   if constexpr (HAS_IDX) {
+    // the payload takes the same route: row positions from the previous pass (or synthesised
+    // by the first pass) go through the same LDS slots as the keys did
+    OffT idx[ITEMS];
     if (a.idx_in != nullptr) {
       const OffT* iin = a.idx_in + row_base + tile_off;
 #pragma unroll
@@ -267,142 +432,31 @@ __global__ __launch_bounds__(BLOCK) void onesweep_kernel(const SweepArgs<BIG> a)
         idx[i] = static_cast<OffT>(tile_off + woff + i * WAVE);
       }
     }
-  }
-
-  // ---- rank inside the wave, count digits per wave ----
-  uint32_t rnk[ITEMS];
-  uint32_t* wctr = s_ctr + wave * RADIX;
-#pragma unroll
-  for (int i = 0; i < ITEMS; ++i) {
-    const bool valid = full || (woff + i * WAVE < count);
-    rnk[i]           = wave_match_rank(radix_digit<CODEC, KeyT>(key[i], a.shift), valid, wctr);
-  }
-  __syncthreads();
-
-  // ---- per digit: offsets of the waves, tile total, publish, scan over digits ----
-  uint32_t dsum = 0, dincl = 0;
-  OffT* my_desc = a.desc + static_cast<uint64_t>(tile) * RADIX + tid;
-  if (tid < RADIX) {
-#pragma unroll
-    for (int w = 0; w < WAVES; ++w) {
-      const uint32_t c       = s_ctr[w * RADIX + tid];
-      s_ctr[w * RADIX + tid] = dsum;
-      dsum += c;
-    }
-    const OffT first = (trow == 0) ? DB::INCLUSIVE : DB::AGGREGATE;
-    __hip_atomic_store(my_desc, static_cast<OffT>(first | dsum), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    dincl = wave_inclusive_scan(dsum, lane);
-    if (lane == WAVE - 1) {
-      s_wsum[wave] = dincl;
-    }
-  }
-  __syncthreads();
-  if (tid < RADIX) {
-    uint32_t dexcl = dincl - dsum;
-    for (int w = 0; w < wave; ++w) {
-      dexcl += s_wsum[w];
-    }
-    // ---- decoupled look-back over the earlier tiles of this row ----
-    OffT before = 0;
-    if (trow != 0) {
-      uint32_t t        = tile - 1;
-      const uint32_t t0 = tile - trow;  // first tile of the row, always INCLUSIVE
-      bool failed       = false;
-      while (true) {
-        const OffT* dp = a.desc + static_cast<uint64_t>(t) * RADIX + tid;
-        OffT v         = __hip_atomic_load(dp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        uint32_t spins = 0;
-        while ((v & DB::STATUS) == 0) {
-          if (++spins >= LOOKBACK_SPIN_LIMIT) {
-            failed = true;
-            break;
-          }
-          if ((spins & 1023u) == 0 &&
-              __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
-            failed = true;  // another tile already gave up: drain quickly
-            break;
-          }
-          __builtin_amdgcn_s_sleep(2);
-          v = __hip_atomic_load(dp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        if (failed) {
-          break;
-        }
-        before += (v & DB::VALUE);
-        if ((v & DB::INCLUSIVE) != 0 || t == t0) {
-          break;
-        }
-        --t;
-      }
-      if (failed) {
-        __hip_atomic_fetch_or(a.status, DEVICE_ERR_LOOKBACK, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-      __hip_atomic_store(my_desc, static_cast<OffT>(DB::INCLUSIVE | (before + dsum)), __ATOMIC_RELAXED,
-                         __HIP_MEMORY_SCOPE_AGENT);
-    }
-    // global element offset of local sorted position 0 for this digit (unsigned wrap is fine)
-    s_gbase[tid] = row_base + static_cast<uint64_t>(a.hist_excl[row * a.hist_row_stride + tid]) +
-                   static_cast<uint64_t>(before) - static_cast<uint64_t>(dexcl);
-#pragma unroll
-    for (int w = 0; w < WAVES; ++w) {
-      s_ctr[w * RADIX + tid] += dexcl;
-    }
-  }
-  __syncthreads();
-
-  // ---- local scatter into LDS, then coalesced runs to HBM ----
-  KeyT* s_keys = reinterpret_cast<KeyT*>(s_stage);
-#pragma unroll
-  for (int i = 0; i < ITEMS; ++i) {
-    if (full || (woff + i * WAVE < count)) {
-      const uint32_t d   = radix_digit<CODEC, KeyT>(key[i], a.shift);
-      const uint32_t pos = wctr[d] + rnk[i];
-      rnk[i]             = pos;
-      s_keys[pos]        = key[i];
-    }
-  }
-  __syncthreads();
-  uint32_t dig[ITEMS];
-  KeyT* kout = static_cast<KeyT*>(a.keys_out);
-#pragma unroll
-  for (int k = 0; k < ITEMS; ++k) {
-    const uint32_t p = tid + k * BLOCK;
-    if (full || p < count) {
-      const KeyT kk = s_keys[p];
-      dig[k]        = radix_digit<CODEC, KeyT>(kk, a.shift);
-      if (kout != nullptr) {
-        kout[s_gbase[dig[k]] + p] = kk;
-      }
-    } else {
-      dig[k] = 0;
-    }
-  }
-  if constexpr (HAS_IDX) {
     __syncthreads();
     OffT* s_idx = reinterpret_cast<OffT*>(s_stage);
 #pragma unroll
     for (int i = 0; i < ITEMS; ++i) {
       if (full || (woff + i * WAVE < count)) {
-        s_idx[rnk[i]] = idx[i];
+        s_idx[(pos2[i / 2] >> (16 * (i % 2))) & 0xFFFFu] = idx[i];
       }
     }
     __syncthreads();
     if (a.idx_final) {
-      int64_t* iout = static_cast<int64_t*>(a.idx_out);
+      int64_t* iout = static_cast<int64_t*>(a.idx_out) + row_base;
 #pragma unroll
       for (int k = 0; k < ITEMS; ++k) {
         const uint32_t p = tid + k * BLOCK;
         if (full || p < count) {
-          iout[s_gbase[dig[k]] + p] = static_cast<int64_t>(s_idx[p]) + a.index_offset;
+          iout[goff[k]] = static_cast<int64_t>(s_idx[p]) + a.index_offset;
         }
       }
     } else {
-      OffT* iout = static_cast<OffT*>(a.idx_out);
+      OffT* iout = static_cast<OffT*>(a.idx_out) + row_base;
 #pragma unroll
       for (int k = 0; k < ITEMS; ++k) {
         const uint32_t p = tid + k * BLOCK;
         if (full || p < count) {
-          iout[s_gbase[dig[k]] + p] = s_idx[p];
+          iout[goff[k]] = s_idx[p];
         }
       }
     }

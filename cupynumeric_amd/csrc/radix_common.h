@@ -31,20 +31,28 @@ __device__ __forceinline__ uint32_t lanes_below(uint64_t mask)
 //
 // Returns the number of keys with the same digit that precede this key in the wave
 // (earlier rounds + lower lanes of this round) and advances the counter.  Eight ballots
-// build the mask of lanes holding the same digit; the highest such lane updates the
-// counter after every peer has read it (LDS operations of one wave execute in order).
+// build the mask of lanes holding the same digit: for every digit bit, a lane accumulates
+// the lanes whose bit differs from its own (ballot XOR own bit broadcast over 32 bits).
+// The highest lane of each group updates the counter after every member has read it (LDS
+// operations of one wave execute in order).
 __device__ __forceinline__ uint32_t wave_match_rank(uint32_t digit, bool valid, uint32_t* wctr)
 {
-  uint64_t peers = __builtin_amdgcn_ballot_w64(valid);
+  const uint64_t vmask = __builtin_amdgcn_ballot_w64(valid);
+  uint32_t mis_lo = 0, mis_hi = 0;
 #pragma unroll
   for (int b = 0; b < RADIX_BITS; ++b) {
-    const bool bit     = (digit >> b) & 1u;
-    const uint64_t bal = __builtin_amdgcn_ballot_w64(bit);
-    peers &= bit ? bal : ~bal;
+    int32_t own = __builtin_amdgcn_sbfe(static_cast<int32_t>(digit), b, 1);  // 0 or -1
+    asm volatile("" : "+v"(own));  // keep the compare on `own` (one v_cmp) instead of a re-derived bit test
+    const uint64_t bal = __builtin_amdgcn_ballot_w64(own != 0);
+    // mis |= bal ^ own, one three-input bit operation per half (truth table 0xF6 = a | (b ^ c))
+    mis_lo = __builtin_amdgcn_bitop3_b32(mis_lo, static_cast<uint32_t>(bal), static_cast<uint32_t>(own), 0xF6);
+    mis_hi = __builtin_amdgcn_bitop3_b32(mis_hi, static_cast<uint32_t>(bal >> 32), static_cast<uint32_t>(own), 0xF6);
   }
-  const uint32_t lower = lanes_below(peers);
-  const uint32_t total = static_cast<uint32_t>(__builtin_popcountll(peers));
-  const uint32_t old   = wctr[digit];
+  const uint32_t peers_lo = static_cast<uint32_t>(vmask) & ~mis_lo;
+  const uint32_t peers_hi = static_cast<uint32_t>(vmask >> 32) & ~mis_hi;
+  const uint32_t lower    = __builtin_amdgcn_mbcnt_hi(peers_hi, __builtin_amdgcn_mbcnt_lo(peers_lo, 0u));
+  const uint32_t total    = static_cast<uint32_t>(__builtin_popcount(peers_lo) + __builtin_popcount(peers_hi));
+  const uint32_t old      = wctr[digit];
   __builtin_amdgcn_wave_barrier();
   if (valid && lower + 1 == total) {
     wctr[digit] = old + total;

@@ -35,11 +35,20 @@ constexpr uint64_t BIG_ROW_ELEMENTS = 1ull << 30;
 
 __host__ __device__ constexpr uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
 
-// Tile shape of the global sort per key width.
-__host__ __device__ constexpr int global_block(int /*key_bytes*/) { return 512; }
+// Tile shape of the global sort per key width (the macros allow A/B builds of other shapes).
+#ifndef CPN_GLOBAL_BLOCK
+#define CPN_GLOBAL_BLOCK 512
+#endif
+#ifndef CPN_GLOBAL_ITEMS
+#define CPN_GLOBAL_ITEMS 16
+#endif
+__host__ __device__ constexpr int global_block(int /*key_bytes*/) { return CPN_GLOBAL_BLOCK; }
 // (64-bit keys or 64-bit row positions halve the items per thread so that the LDS staging
 // area stays at 32 KiB)
-__host__ __device__ constexpr int global_items(int key_bytes, bool big) { return (key_bytes == 8 || big) ? 8 : 16; }
+__host__ __device__ constexpr int global_items(int key_bytes, bool big)
+{
+  return (key_bytes == 8 || big) ? CPN_GLOBAL_ITEMS / 2 : CPN_GLOBAL_ITEMS;
+}
 __host__ __device__ constexpr int global_tile(int key_bytes, bool big)
 {
   return global_block(key_bytes) * global_items(key_bytes, big);
