@@ -200,8 +200,12 @@ struct SweepArgs {
   int idx_final;           // idx_out is the caller's int64 array
 };
 
+#ifndef CPN_ONESWEEP_WAVES_PER_EU
+#define CPN_ONESWEEP_WAVES_PER_EU 6
+#endif
 template <typename KeyT, int CODEC, bool BIG, bool HAS_IDX, int BLOCK, int ITEMS>
-__global__ __launch_bounds__(BLOCK) void onesweep_kernel(const SweepArgs<BIG> a)
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(CPN_ONESWEEP_WAVES_PER_EU)))
+void onesweep_kernel(const SweepArgs<BIG> a)
 {
   using OffT = typename RowWidth<BIG>::off_t;
   using DB   = DescBits<OffT>;
@@ -262,21 +266,25 @@ __global__ __launch_bounds__(BLOCK) void onesweep_kernel(const SweepArgs<BIG> a)
     }
   }
 
-  // ---- digits, and the tile's digit counts per wave before any ranking ("early counts"):
-  //      the aggregate can be published, and the look-back can start, while the keys are ranked
-  uint32_t dpk[ITEMS / 4];  // the digits, four per register
+  // ---- rank inside the wave (counters run from zero), count digits per wave ----
+  uint32_t dpk[ITEMS / 4];   // the digits, four per register
+  uint32_t rnk2[ITEMS / 2];  // rank among the wave's keys of the same digit, two per register
   uint32_t* wctr = s_ctr + wave * RADIX;
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
+    const bool valid = full || (woff + i * WAVE < count);
     const uint32_t d = radix_digit<CODEC, KeyT>(key[i], a.shift);
     dpk[i / 4]       = (i % 4 == 0) ? d : (dpk[i / 4] | (d << (8 * (i % 4))));
-    if (full || (woff + i * WAVE < count)) {
-      atomicAdd(&wctr[d], 1u);
-    }
+    const uint32_t r = wave_match_rank(d, valid, wctr) & 0xFFFFu;
+    rnk2[i / 2]      = (i % 2 == 0) ? r : (rnk2[i / 2] | (r << 16));
+    // the packed registers are opaque to the optimiser, which would otherwise keep every
+    // digit and rank alive in a register of its own until the scatter phase
+    asm volatile("" : "+v"(dpk[i / 4]), "+v"(rnk2[i / 2]));
   }
   __syncthreads();
 
-  // ---- per digit: start of every wave's keys, tile total, publish, first look-back reads ----
+  // ---- per digit: start of every wave's keys, tile total, publish, first look-back reads:
+  //      the answers travel while the tile is scattered into LDS ----
   uint32_t dsum = 0, dincl = 0;
   OffT window[LOOKBACK_WINDOW];
   OffT* my_desc     = a.desc + static_cast<uint64_t>(tile) * RADIX + tid;
@@ -318,26 +326,24 @@ __global__ __launch_bounds__(BLOCK) void onesweep_kernel(const SweepArgs<BIG> a)
   }
   __syncthreads();
 
-  // ---- rank inside the wave and scatter into LDS: the counters already hold each wave's
-  //      first position per digit, so the rank is the final position in the sorted tile ----
+  // ---- scatter into LDS: counter = first position of this wave's keys with that digit ----
   KeyT* s_keys = reinterpret_cast<KeyT*>(s_stage);
   uint32_t pos2[ITEMS / 2];  // positions in the sorted tile, two per register
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
-    const bool valid   = full || (woff + i * WAVE < count);
     const uint32_t d   = (dpk[i / 4] >> (8 * (i % 4))) & 0xFFu;
-    const uint32_t pos = wave_match_rank(d, valid, wctr);
-    if (valid) {
+    const uint32_t pos = (wctr[d] + ((rnk2[i / 2] >> (16 * (i % 2))) & 0xFFFFu)) & 0xFFFFu;
+    if (full || (woff + i * WAVE < count)) {
       s_keys[pos] = key[i];
       s_dig[pos]  = static_cast<uint8_t>(d);
     }
-    pos2[i / 2] = (i % 2 == 0) ? (pos & 0xFFFFu) : (pos2[i / 2] | (pos << 16));
+    pos2[i / 2] = (i % 2 == 0) ? pos : (pos2[i / 2] | (pos << 16));
   }
 
   // ---- decoupled look-back over the earlier tiles of this row ----
   // A descriptor written on another XCD is only visible through memory-side accesses, so
   // one poll costs a full memory round trip.  The first window of predecessors was requested
-  // before the ranking phase; its answers are summed front to back until the first
+  // before the scatter phase; its answers are summed front to back until the first
   // inclusive one, further windows follow only if none was.
   if (tid < RADIX) {
     OffT before = 0;
@@ -400,19 +406,16 @@ __global__ __launch_bounds__(BLOCK) void onesweep_kernel(const SweepArgs<BIG> a)
   }
   __syncthreads();
 
-  // ---- coalesced runs from LDS to HBM ----
-  OffT goff[ITEMS];  // offset in the row of the element at sorted position tid + k*BLOCK
-  KeyT* kout = (a.keys_out != nullptr) ? static_cast<KeyT*>(a.keys_out) + row_base : nullptr;
+  // ---- coalesced runs from LDS to HBM: the element at sorted position p of the tile goes
+  //      to row offset s_gbase[digit] + p ----
+  if (a.keys_out != nullptr) {
+    KeyT* kout = static_cast<KeyT*>(a.keys_out) + row_base;
 #pragma unroll
-  for (int k = 0; k < ITEMS; ++k) {
-    const uint32_t p = tid + k * BLOCK;
-    if (full || p < count) {
-      goff[k] = s_gbase[s_dig[p]] + p;
-      if (kout != nullptr) {
-        kout[goff[k]] = s_keys[p];
+    for (int k = 0; k < ITEMS; ++k) {
+      const uint32_t p = tid + k * BLOCK;
+      if (full || p < count) {
+        kout[s_gbase[s_dig[p]] + p] = s_keys[p];
       }
-    } else {
-      goff[k] = 0;
     }
   }
   if constexpr (HAS_IDX) {
@@ -447,7 +450,7 @@ __global__ __launch_bounds__(BLOCK) void onesweep_kernel(const SweepArgs<BIG> a)
       for (int k = 0; k < ITEMS; ++k) {
         const uint32_t p = tid + k * BLOCK;
         if (full || p < count) {
-          iout[goff[k]] = static_cast<int64_t>(s_idx[p]) + a.index_offset;
+          iout[s_gbase[s_dig[p]] + p] = static_cast<int64_t>(s_idx[p]) + a.index_offset;
         }
       }
     } else {
@@ -456,7 +459,7 @@ __global__ __launch_bounds__(BLOCK) void onesweep_kernel(const SweepArgs<BIG> a)
       for (int k = 0; k < ITEMS; ++k) {
         const uint32_t p = tid + k * BLOCK;
         if (full || p < count) {
-          iout[goff[k]] = s_idx[p];
+          iout[s_gbase[s_dig[p]] + p] = s_idx[p];
         }
       }
     }
