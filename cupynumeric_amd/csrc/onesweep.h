@@ -201,7 +201,7 @@ struct SweepArgs {
 };
 
 #ifndef CPN_ONESWEEP_WAVES_PER_EU
-#define CPN_ONESWEEP_WAVES_PER_EU 6
+#define CPN_ONESWEEP_WAVES_PER_EU 4
 #endif
 template <typename KeyT, int CODEC, bool BIG, bool HAS_IDX, int BLOCK, int ITEMS>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(CPN_ONESWEEP_WAVES_PER_EU)))
@@ -218,7 +218,6 @@ void onesweep_kernel(const SweepArgs<BIG> a)
   static_assert(TILE <= 65536, "positions inside a tile are kept in 16 bits");
 
   __shared__ __align__(16) unsigned char s_stage[TILE * STAGE_ELEM];
-  __shared__ uint8_t s_dig[TILE];  // digit of the key at each sorted position of the tile
   __shared__ uint32_t s_ctr[WAVES * RADIX];
   __shared__ OffT s_gbase[RADIX];
   __shared__ uint32_t s_wsum[RADIX / WAVE];
@@ -335,7 +334,6 @@ void onesweep_kernel(const SweepArgs<BIG> a)
     const uint32_t pos = (wctr[d] + ((rnk2[i / 2] >> (16 * (i % 2))) & 0xFFFFu)) & 0xFFFFu;
     if (full || (woff + i * WAVE < count)) {
       s_keys[pos] = key[i];
-      s_dig[pos]  = static_cast<uint8_t>(d);
     }
     pos2[i / 2] = (i % 2 == 0) ? pos : (pos2[i / 2] | (pos << 16));
   }
@@ -407,20 +405,28 @@ void onesweep_kernel(const SweepArgs<BIG> a)
   __syncthreads();
 
   // ---- coalesced runs from LDS to HBM: the element at sorted position p of the tile goes
-  //      to row offset s_gbase[digit] + p ----
-  if (a.keys_out != nullptr) {
-    KeyT* kout = static_cast<KeyT*>(a.keys_out) + row_base;
+  //      to row offset s_gbase[its digit] + p.  The digits of this thread's output positions
+  //      are kept (four per register) for the payload, which goes the same way. ----
+  uint32_t dq[ITEMS / 4];
+  {
+    KeyT* kout = (a.keys_out != nullptr) ? static_cast<KeyT*>(a.keys_out) + row_base : nullptr;
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
       const uint32_t p = tid + k * BLOCK;
+      uint32_t d       = 0;
       if (full || p < count) {
-        kout[s_gbase[s_dig[p]] + p] = s_keys[p];
+        const KeyT kk = s_keys[p];
+        d             = radix_digit<CODEC, KeyT>(kk, a.shift);
+        if (kout != nullptr) {
+          kout[s_gbase[d] + p] = kk;
+        }
       }
+      dq[k / 4] = (k % 4 == 0) ? d : (dq[k / 4] | (d << (8 * (k % 4))));
+      asm volatile("" : "+v"(dq[k / 4]));
     }
   }
   if constexpr (HAS_IDX) {
-    // the payload takes the same route: row positions from the previous pass (or synthesised
-    // by the first pass) go through the same LDS slots as the keys did
+    // row positions from the previous pass, or synthesised by the first pass
     OffT idx[ITEMS];
     if (a.idx_in != nullptr) {
       const OffT* iin = a.idx_in + row_base + tile_off;
@@ -450,7 +456,8 @@ void onesweep_kernel(const SweepArgs<BIG> a)
       for (int k = 0; k < ITEMS; ++k) {
         const uint32_t p = tid + k * BLOCK;
         if (full || p < count) {
-          iout[s_gbase[s_dig[p]] + p] = static_cast<int64_t>(s_idx[p]) + a.index_offset;
+          const uint32_t d       = (dq[k / 4] >> (8 * (k % 4))) & 0xFFu;
+          iout[s_gbase[d] + p] = static_cast<int64_t>(s_idx[p]) + a.index_offset;
         }
       }
     } else {
@@ -459,7 +466,8 @@ void onesweep_kernel(const SweepArgs<BIG> a)
       for (int k = 0; k < ITEMS; ++k) {
         const uint32_t p = tid + k * BLOCK;
         if (full || p < count) {
-          iout[s_gbase[s_dig[p]] + p] = s_idx[p];
+          const uint32_t d       = (dq[k / 4] >> (8 * (k % 4))) & 0xFFu;
+          iout[s_gbase[d] + p] = s_idx[p];
         }
       }
     }

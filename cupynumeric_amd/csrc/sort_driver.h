@@ -40,11 +40,11 @@ __host__ __device__ constexpr uint64_t align_up(uint64_t v, uint64_t a) { return
 #define CPN_GLOBAL_BLOCK 512
 #endif
 #ifndef CPN_GLOBAL_ITEMS
-#define CPN_GLOBAL_ITEMS 16
+#define CPN_GLOBAL_ITEMS 32
 #endif
 __host__ __device__ constexpr int global_block(int /*key_bytes*/) { return CPN_GLOBAL_BLOCK; }
 // (64-bit keys or 64-bit row positions halve the items per thread so that the LDS staging
-// area stays at 32 KiB)
+// area stays at 64 KiB: two workgroups of 512 threads fit in a CU's 160 KiB)
 __host__ __device__ constexpr int global_items(int key_bytes, bool big)
 {
   return (key_bytes == 8 || big) ? CPN_GLOBAL_ITEMS / 2 : CPN_GLOBAL_ITEMS;
