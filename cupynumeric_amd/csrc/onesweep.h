@@ -203,75 +203,62 @@ struct SweepArgs {
 #ifndef CPN_ONESWEEP_WAVES_PER_EU
 #define CPN_ONESWEEP_WAVES_PER_EU 4
 #endif
-template <typename KeyT, int CODEC, bool BIG, bool HAS_IDX, int BLOCK, int ITEMS>
-__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(CPN_ONESWEEP_WAVES_PER_EU)))
-void onesweep_kernel(const SweepArgs<BIG> a)
+
+// Shared-memory view of one onesweep workgroup.
+template <typename KeyT, typename OffT, int WAVES, int TILE, int STAGE_ELEM>
+struct SweepShared {
+  alignas(16) unsigned char stage[TILE * STAGE_ELEM];  // sorted tile: keys, then the payload
+  uint32_t ctr[WAVES * RADIX];                         // per wave and digit: count, then first position
+  OffT gbase[RADIX];                                   // per digit: row offset of sorted position 0
+  uint32_t wsum[RADIX / WAVE];
+  uint32_t tile;
+};
+
+// The work on one tile.  FULL is true for tiles of exactly TILE keys: every bounds test
+// folds away and the body is straight-line code, which lets the compiler batch the LDS and
+// HBM accesses of a phase instead of waiting on each one.
+template <typename KeyT, int CODEC, bool BIG, bool HAS_IDX, int BLOCK, int ITEMS, bool FULL>
+__device__ __forceinline__ void onesweep_tile(
+  const SweepArgs<BIG>& a,
+  SweepShared<KeyT, typename RowWidth<BIG>::off_t, BLOCK / WAVE, BLOCK * ITEMS,
+              ((HAS_IDX && sizeof(typename RowWidth<BIG>::off_t) > sizeof(KeyT)) ? sizeof(typename RowWidth<BIG>::off_t)
+                                                                                : sizeof(KeyT))>& sh,
+  const uint32_t tile,
+  const uint64_t row,
+  const uint32_t trow,
+  const uint32_t count)
 {
   using OffT = typename RowWidth<BIG>::off_t;
   using DB   = DescBits<OffT>;
-  static_assert(BLOCK >= RADIX, "one thread per digit is needed for the look-back");
-  static_assert(ITEMS % 4 == 0, "digits are cached four to a register");
-  constexpr int WAVES      = BLOCK / WAVE;
-  constexpr int TILE       = BLOCK * ITEMS;
-  constexpr int WTILE      = ITEMS * WAVE;  // keys of one wave, contiguous in the tile
-  constexpr int STAGE_ELEM = (HAS_IDX && sizeof(OffT) > sizeof(KeyT)) ? sizeof(OffT) : sizeof(KeyT);
-  static_assert(TILE <= 65536, "positions inside a tile are kept in 16 bits");
+  constexpr int WAVES = BLOCK / WAVE;
+  constexpr int TILE  = BLOCK * ITEMS;
+  constexpr int WTILE = ITEMS * WAVE;  // keys of one wave, contiguous in the tile
 
-  __shared__ __align__(16) unsigned char s_stage[TILE * STAGE_ELEM];
-  __shared__ uint32_t s_ctr[WAVES * RADIX];
-  __shared__ OffT s_gbase[RADIX];
-  __shared__ uint32_t s_wsum[RADIX / WAVE];
-  __shared__ uint32_t s_tile;
-
-  const int tid  = threadIdx.x;
-  const int lane = tid & (WAVE - 1);
-  const int wave = tid / WAVE;
-
-  // Tiles are handed out in launch order of the workgroups that are actually running, so
-  // every tile a look-back waits for belongs to a resident workgroup.
-  if (tid == 0) {
-    s_tile = __hip_atomic_fetch_add(a.ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-  for (int j = tid; j < WAVES * RADIX; j += BLOCK) {
-    s_ctr[j] = 0;
-  }
-  __syncthreads();
-  const uint32_t tile = s_tile;
-  if (tile >= a.num_tiles) {
-    return;  // uniform per block; cannot happen when grid == num_tiles
-  }
-  const uint64_t row      = tile / a.tiles_per_row;
-  const uint32_t trow     = tile - static_cast<uint32_t>(row * a.tiles_per_row);
+  const int tid           = threadIdx.x;
+  const int lane          = tid & (WAVE - 1);
+  const int wave          = tid / WAVE;
+  const uint32_t woff     = wave * WTILE + lane;
   const uint64_t row_base = row * a.seg;
   const uint64_t tile_off = static_cast<uint64_t>(trow) * TILE;
-  const uint64_t remain   = a.seg - tile_off;
-  const uint32_t count    = remain < static_cast<uint64_t>(TILE) ? static_cast<uint32_t>(remain) : TILE;
-  const bool full         = (count == TILE);
-  const uint32_t woff     = wave * WTILE + lane;
+  uint32_t* wctr          = sh.ctr + wave * RADIX;
+  KeyT* s_keys            = reinterpret_cast<KeyT*>(sh.stage);
+  OffT* s_idx             = reinterpret_cast<OffT*>(sh.stage);
 
   // ---- load: item i of lane l is element  wave*WTILE + i*64 + l  of the tile ----
   const KeyT* kin = static_cast<const KeyT*>(a.keys_in) + row_base + tile_off;
   KeyT key[ITEMS];
-  if (full) {
 #pragma unroll
-    for (int i = 0; i < ITEMS; ++i) {
-      key[i] = kin[woff + i * WAVE];
-    }
-  } else {
-#pragma unroll
-    for (int i = 0; i < ITEMS; ++i) {
-      const uint32_t o = woff + i * WAVE;
-      key[i]           = (o < count) ? kin[o] : static_cast<KeyT>(0);
-    }
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t o = woff + i * WAVE;
+    key[i]           = (FULL || o < count) ? kin[o] : static_cast<KeyT>(0);
   }
 
   // ---- rank inside the wave (counters run from zero), count digits per wave ----
   uint32_t dpk[ITEMS / 4];   // the digits, four per register
   uint32_t rnk2[ITEMS / 2];  // rank among the wave's keys of the same digit, two per register
-  uint32_t* wctr = s_ctr + wave * RADIX;
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
-    const bool valid = full || (woff + i * WAVE < count);
+    const bool valid = FULL || (woff + i * WAVE < count);
     const uint32_t d = radix_digit<CODEC, KeyT>(key[i], a.shift);
     dpk[i / 4]       = (i % 4 == 0) ? d : (dpk[i / 4] | (d << (8 * (i % 4))));
     const uint32_t r = wave_match_rank(d, valid, wctr) & 0xFFFFu;
@@ -291,8 +278,8 @@ void onesweep_kernel(const SweepArgs<BIG> a)
   if (tid < RADIX) {
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) {
-      const uint32_t c       = s_ctr[w * RADIX + tid];
-      s_ctr[w * RADIX + tid] = dsum;
+      const uint32_t c        = sh.ctr[w * RADIX + tid];
+      sh.ctr[w * RADIX + tid] = dsum;
       dsum += c;
     }
     const OffT first = (trow == 0) ? DB::INCLUSIVE : DB::AGGREGATE;
@@ -308,7 +295,7 @@ void onesweep_kernel(const SweepArgs<BIG> a)
     }
     dincl = wave_inclusive_scan(dsum, lane);
     if (lane == WAVE - 1) {
-      s_wsum[wave] = dincl;
+      sh.wsum[wave] = dincl;
     }
   }
   __syncthreads();
@@ -316,23 +303,22 @@ void onesweep_kernel(const SweepArgs<BIG> a)
   if (tid < RADIX) {
     dexcl = dincl - dsum;
     for (int w = 0; w < wave; ++w) {
-      dexcl += s_wsum[w];
+      dexcl += sh.wsum[w];
     }
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) {
-      s_ctr[w * RADIX + tid] += dexcl;
+      sh.ctr[w * RADIX + tid] += dexcl;
     }
   }
   __syncthreads();
 
   // ---- scatter into LDS: counter = first position of this wave's keys with that digit ----
-  KeyT* s_keys = reinterpret_cast<KeyT*>(s_stage);
   uint32_t pos2[ITEMS / 2];  // positions in the sorted tile, two per register
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t d   = (dpk[i / 4] >> (8 * (i % 4))) & 0xFFu;
     const uint32_t pos = (wctr[d] + ((rnk2[i / 2] >> (16 * (i % 2))) & 0xFFFFu)) & 0xFFFFu;
-    if (full || (woff + i * WAVE < count)) {
+    if (FULL || (woff + i * WAVE < count)) {
       s_keys[pos] = key[i];
     }
     pos2[i / 2] = (i % 2 == 0) ? pos : (pos2[i / 2] | (pos << 16));
@@ -400,29 +386,35 @@ void onesweep_kernel(const SweepArgs<BIG> a)
                          __HIP_MEMORY_SCOPE_AGENT);
     }
     // offset inside the row of local sorted position 0 for this digit (unsigned wrap is fine)
-    s_gbase[tid] = a.hist_excl[row * a.hist_row_stride + tid] + before - static_cast<OffT>(dexcl);
+    sh.gbase[tid] = a.hist_excl[row * a.hist_row_stride + tid] + before - static_cast<OffT>(dexcl);
   }
   __syncthreads();
 
   // ---- coalesced runs from LDS to HBM: the element at sorted position p of the tile goes
-  //      to row offset s_gbase[its digit] + p.  The digits of this thread's output positions
+  //      to row offset gbase[its digit] + p.  The digits of this thread's output positions
   //      are kept (four per register) for the payload, which goes the same way. ----
   uint32_t dq[ITEMS / 4];
   {
-    KeyT* kout = (a.keys_out != nullptr) ? static_cast<KeyT*>(a.keys_out) + row_base : nullptr;
+    KeyT kk[ITEMS];
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
       const uint32_t p = tid + k * BLOCK;
-      uint32_t d       = 0;
-      if (full || p < count) {
-        const KeyT kk = s_keys[p];
-        d             = radix_digit<CODEC, KeyT>(kk, a.shift);
-        if (kout != nullptr) {
-          kout[s_gbase[d] + p] = kk;
+      kk[k]            = (FULL || p < count) ? s_keys[p] : static_cast<KeyT>(0);
+    }
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+      const uint32_t d = radix_digit<CODEC, KeyT>(kk[k], a.shift);
+      dq[k / 4]        = (k % 4 == 0) ? d : (dq[k / 4] | (d << (8 * (k % 4))));
+    }
+    if (a.keys_out != nullptr) {
+      KeyT* kout = static_cast<KeyT*>(a.keys_out) + row_base;
+#pragma unroll
+      for (int k = 0; k < ITEMS; ++k) {
+        const uint32_t p = tid + k * BLOCK;
+        if (FULL || p < count) {
+          kout[sh.gbase[(dq[k / 4] >> (8 * (k % 4))) & 0xFFu] + p] = kk[k];
         }
       }
-      dq[k / 4] = (k % 4 == 0) ? d : (dq[k / 4] | (d << (8 * (k % 4))));
-      asm volatile("" : "+v"(dq[k / 4]));
     }
   }
   if constexpr (HAS_IDX) {
@@ -433,7 +425,7 @@ void onesweep_kernel(const SweepArgs<BIG> a)
 #pragma unroll
       for (int i = 0; i < ITEMS; ++i) {
         const uint32_t o = woff + i * WAVE;
-        idx[i]           = (full || o < count) ? iin[o] : static_cast<OffT>(0);
+        idx[i]           = (FULL || o < count) ? iin[o] : static_cast<OffT>(0);
       }
     } else {
 #pragma unroll
@@ -442,10 +434,9 @@ void onesweep_kernel(const SweepArgs<BIG> a)
       }
     }
     __syncthreads();
-    OffT* s_idx = reinterpret_cast<OffT*>(s_stage);
 #pragma unroll
     for (int i = 0; i < ITEMS; ++i) {
-      if (full || (woff + i * WAVE < count)) {
+      if (FULL || (woff + i * WAVE < count)) {
         s_idx[(pos2[i / 2] >> (16 * (i % 2))) & 0xFFFFu] = idx[i];
       }
     }
@@ -455,9 +446,8 @@ void onesweep_kernel(const SweepArgs<BIG> a)
 #pragma unroll
       for (int k = 0; k < ITEMS; ++k) {
         const uint32_t p = tid + k * BLOCK;
-        if (full || p < count) {
-          const uint32_t d       = (dq[k / 4] >> (8 * (k % 4))) & 0xFFu;
-          iout[s_gbase[d] + p] = static_cast<int64_t>(s_idx[p]) + a.index_offset;
+        if (FULL || p < count) {
+          iout[sh.gbase[(dq[k / 4] >> (8 * (k % 4))) & 0xFFu] + p] = static_cast<int64_t>(s_idx[p]) + a.index_offset;
         }
       }
     } else {
@@ -465,12 +455,49 @@ void onesweep_kernel(const SweepArgs<BIG> a)
 #pragma unroll
       for (int k = 0; k < ITEMS; ++k) {
         const uint32_t p = tid + k * BLOCK;
-        if (full || p < count) {
-          const uint32_t d       = (dq[k / 4] >> (8 * (k % 4))) & 0xFFu;
-          iout[s_gbase[d] + p] = s_idx[p];
+        if (FULL || p < count) {
+          iout[sh.gbase[(dq[k / 4] >> (8 * (k % 4))) & 0xFFu] + p] = s_idx[p];
         }
       }
     }
+  }
+}
+
+template <typename KeyT, int CODEC, bool BIG, bool HAS_IDX, int BLOCK, int ITEMS>
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(CPN_ONESWEEP_WAVES_PER_EU)))
+void onesweep_kernel(const SweepArgs<BIG> a)
+{
+  using OffT = typename RowWidth<BIG>::off_t;
+  static_assert(BLOCK >= RADIX, "one thread per digit is needed for the look-back");
+  static_assert(ITEMS % 4 == 0, "digits are cached four to a register");
+  constexpr int WAVES      = BLOCK / WAVE;
+  constexpr int TILE       = BLOCK * ITEMS;
+  constexpr int STAGE_ELEM = (HAS_IDX && sizeof(OffT) > sizeof(KeyT)) ? sizeof(OffT) : sizeof(KeyT);
+  static_assert(TILE <= 65536, "positions inside a tile are kept in 16 bits");
+
+  __shared__ SweepShared<KeyT, OffT, WAVES, TILE, STAGE_ELEM> sh;
+
+  const int tid = threadIdx.x;
+  // Tiles are handed out in launch order of the workgroups that are actually running, so
+  // every tile a look-back waits for belongs to a resident workgroup.
+  if (tid == 0) {
+    sh.tile = __hip_atomic_fetch_add(a.ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  for (int j = tid; j < WAVES * RADIX; j += BLOCK) {
+    sh.ctr[j] = 0;
+  }
+  __syncthreads();
+  const uint32_t tile = sh.tile;
+  if (tile >= a.num_tiles) {
+    return;  // uniform per block; cannot happen when grid == num_tiles
+  }
+  const uint64_t row    = tile / a.tiles_per_row;
+  const uint32_t trow   = tile - static_cast<uint32_t>(row * a.tiles_per_row);
+  const uint64_t remain = a.seg - static_cast<uint64_t>(trow) * TILE;
+  if (remain >= static_cast<uint64_t>(TILE)) {
+    onesweep_tile<KeyT, CODEC, BIG, HAS_IDX, BLOCK, ITEMS, true>(a, sh, tile, row, trow, TILE);
+  } else {
+    onesweep_tile<KeyT, CODEC, BIG, HAS_IDX, BLOCK, ITEMS, false>(a, sh, tile, row, trow, static_cast<uint32_t>(remain));
   }
 }
 
