@@ -217,7 +217,12 @@ struct SweepShared {
 // The work on one tile.  FULL is true for tiles of exactly TILE keys: every bounds test
 // folds away and the body is straight-line code, which lets the compiler batch the LDS and
 // HBM accesses of a phase instead of waiting on each one.
-template <typename KeyT, int CODEC, bool BIG, bool HAS_IDX, int BLOCK, int ITEMS, bool FULL>
+//
+// XFORM (index-only sorts): the keys are replaced by their order-preserving unsigned image
+// as soon as they are loaded and are written out that way, so that the later passes, which
+// then run with the identity codec, do not pay for the key transform again.  The values
+// themselves are never returned in that case.
+template <typename KeyT, int CODEC, bool XFORM, bool BIG, bool HAS_IDX, int BLOCK, int ITEMS, bool FULL>
 __device__ __forceinline__ void onesweep_tile(
   const SweepArgs<BIG>& a,
   SweepShared<KeyT, typename RowWidth<BIG>::off_t, BLOCK / WAVE, BLOCK * ITEMS,
@@ -233,6 +238,7 @@ __device__ __forceinline__ void onesweep_tile(
   constexpr int WAVES = BLOCK / WAVE;
   constexpr int TILE  = BLOCK * ITEMS;
   constexpr int WTILE = ITEMS * WAVE;  // keys of one wave, contiguous in the tile
+  constexpr int DCODEC = XFORM ? static_cast<int>(CODEC_UNSIGNED) : CODEC;  // codec at digit extraction
 
   const int tid           = threadIdx.x;
   const int lane          = tid & (WAVE - 1);
@@ -251,6 +257,9 @@ __device__ __forceinline__ void onesweep_tile(
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t o = woff + i * WAVE;
     key[i]           = (FULL || o < count) ? kin[o] : static_cast<KeyT>(0);
+    if constexpr (XFORM) {
+      key[i] = ordered_bits<CODEC, KeyT>(key[i]);
+    }
   }
 
   // ---- rank inside the wave (counters run from zero), count digits per wave ----
@@ -259,7 +268,7 @@ __device__ __forceinline__ void onesweep_tile(
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const bool valid = FULL || (woff + i * WAVE < count);
-    const uint32_t d = radix_digit<CODEC, KeyT>(key[i], a.shift);
+    const uint32_t d = radix_digit<DCODEC, KeyT>(key[i], a.shift);
     dpk[i / 4]       = (i % 4 == 0) ? d : (dpk[i / 4] | (d << (8 * (i % 4))));
     const uint32_t r = wave_match_rank(d, valid, wctr) & 0xFFFFu;
     rnk2[i / 2]      = (i % 2 == 0) ? r : (rnk2[i / 2] | (r << 16));
@@ -403,7 +412,7 @@ __device__ __forceinline__ void onesweep_tile(
     }
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
-      const uint32_t d = radix_digit<CODEC, KeyT>(kk[k], a.shift);
+      const uint32_t d = radix_digit<DCODEC, KeyT>(kk[k], a.shift);
       dq[k / 4]        = (k % 4 == 0) ? d : (dq[k / 4] | (d << (8 * (k % 4))));
     }
     if (a.keys_out != nullptr) {
@@ -463,7 +472,7 @@ __device__ __forceinline__ void onesweep_tile(
   }
 }
 
-template <typename KeyT, int CODEC, bool BIG, bool HAS_IDX, int BLOCK, int ITEMS>
+template <typename KeyT, int CODEC, bool XFORM, bool BIG, bool HAS_IDX, int BLOCK, int ITEMS>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(CPN_ONESWEEP_WAVES_PER_EU)))
 void onesweep_kernel(const SweepArgs<BIG> a)
 {
@@ -495,9 +504,9 @@ void onesweep_kernel(const SweepArgs<BIG> a)
   const uint32_t trow   = tile - static_cast<uint32_t>(row * a.tiles_per_row);
   const uint64_t remain = a.seg - static_cast<uint64_t>(trow) * TILE;
   if (remain >= static_cast<uint64_t>(TILE)) {
-    onesweep_tile<KeyT, CODEC, BIG, HAS_IDX, BLOCK, ITEMS, true>(a, sh, tile, row, trow, TILE);
+    onesweep_tile<KeyT, CODEC, XFORM, BIG, HAS_IDX, BLOCK, ITEMS, true>(a, sh, tile, row, trow, TILE);
   } else {
-    onesweep_tile<KeyT, CODEC, BIG, HAS_IDX, BLOCK, ITEMS, false>(a, sh, tile, row, trow, static_cast<uint32_t>(remain));
+    onesweep_tile<KeyT, CODEC, XFORM, BIG, HAS_IDX, BLOCK, ITEMS, false>(a, sh, tile, row, trow, static_cast<uint32_t>(remain));
   }
 }
 

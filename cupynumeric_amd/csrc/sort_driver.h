@@ -268,6 +268,11 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
   void* idx1 = L.off_idx ? ws + L.off_idx : nullptr;
   void* idxX = r.indices_out;  // the int64 output doubles as a narrow scratch array
 
+  // Index-only sorts never return the keys: the first pass stores their order-preserving
+  // unsigned image in the workspace and the later passes run with the identity codec.
+  constexpr bool CAN_ORDER_KEYS = HAS_IDX && CODEC != CODEC_UNSIGNED && PASSES >= 2;
+  const bool ordered_keys       = CAN_ORDER_KEYS && !want_vals;
+
   const void* key_src = r.values_in;
   const void* idx_src = nullptr;
   for (int p = 0; p < PASSES; ++p) {
@@ -301,8 +306,24 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
     a.idx_final       = last ? 1 : 0;
     {
       ProfileScope prof("onesweep", r.stream);
-      hipLaunchKernelGGL((onesweep_kernel<KeyT, CODEC, BIG, HAS_IDX, BLOCK, ITEMS>),
-                         dim3(static_cast<uint32_t>(L.num_tiles)), dim3(BLOCK), 0, r.stream, a);
+      const dim3 grid(static_cast<uint32_t>(L.num_tiles));
+      bool launched = false;
+      if constexpr (CAN_ORDER_KEYS) {
+        if (ordered_keys) {
+          if (p == 0) {
+            hipLaunchKernelGGL((onesweep_kernel<KeyT, CODEC, true, BIG, HAS_IDX, BLOCK, ITEMS>), grid, dim3(BLOCK), 0,
+                               r.stream, a);
+          } else {
+            hipLaunchKernelGGL((onesweep_kernel<KeyT, CODEC_UNSIGNED, false, BIG, HAS_IDX, BLOCK, ITEMS>), grid,
+                               dim3(BLOCK), 0, r.stream, a);
+          }
+          launched = true;
+        }
+      }
+      if (!launched) {
+        hipLaunchKernelGGL((onesweep_kernel<KeyT, CODEC, false, BIG, HAS_IDX, BLOCK, ITEMS>), grid, dim3(BLOCK), 0,
+                           r.stream, a);
+      }
     }
     CPN_HIP_TRY(hipGetLastError());
     key_src = key_dst;
