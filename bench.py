@@ -34,10 +34,10 @@ if str(ROOT) not in sys.path:
 
 HBM_PEAK_BYTES_PER_S = 8.0e12  # MI355X HBM3E
 
-# HBM bytes per onesweep launch of the default workload, from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE runs scaled by a copy kernel of known size (profiles/onesweep_c2_traffic.txt).
-# None until that measurement exists for the workload being run.
-MEASURED_TRAFFIC_BYTES = {}
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# of this file scaled by a plain copy of known size (profiles/onesweep_c2_traffic.txt).  Keyed by
+# (config, keys); workloads without such a measurement report null.
+MEASURED_TRAFFIC_BYTES = {("c2", 1 << 28): 4.519e9}
 
 
 # -------------------------------------------------------------------------------------------------
@@ -247,6 +247,9 @@ def main() -> None:
     ap.add_argument("--log2n", type=int, default=None, help="shrink a 1-D workload to 2^L keys")
     ap.add_argument("--rows", type=int, default=None, help="shrink a 2-D workload to this many rows")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 1 GiB device copy, the known-size kernel that "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build sorts on one GPU; --gpus must be 1 (no multi-GPU sample sort is built)")
@@ -256,6 +259,14 @@ def main() -> None:
     torch = job.torch
     lib = job.lib
     from cupynumeric_amd import _lib
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0").normal_()
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)  # reads 1 GiB, writes 1 GiB (shows up as the runtime's copyBuffer kernel)
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         job.step()
