@@ -87,7 +87,7 @@ def test_temp_bytes_layout(lib):
     assert tb(f32, 0, 0, 1, 0, 0) == 256
     assert tb(f32, 1 << 20, 1024, 1, 1, 0) == 256  # rows that fit LDS need only the status header
     n = 1 << 24
-    tiles = n // 8192
+    tiles = n // 16384  # 512 threads x 32 keys per tile for keys of up to 4 bytes
     fixed = 256 + 4 * 256 * 4 + 4 * tiles * 256 * 4
     assert tb(f32, n, n, 1, 0, 0) == fixed + 4 * n  # one key buffer
     assert tb(f32, n, n, 1, 0, 1) == fixed + 4 * n  # in place, even pass count: same
