@@ -168,7 +168,7 @@ def test_lds_many_short_rows(lib, torch_cuda):
 
 
 # ---- global onesweep path ---------------------------------------------------------------------------
-GLOBAL_LENGTHS = [1, 2, 100, 4095, 4096, 4097, 8191, 8192, 8193, 3 * 8192 + 5, 100003]
+GLOBAL_LENGTHS = [1, 2, 100, 4097, 8191, 8192, 8193, 16383, 16384, 16385, 3 * 16384 + 5, 100003]
 
 
 @pytest.mark.parametrize("dtype", ALL_REAL_DTYPES)
@@ -181,14 +181,14 @@ def test_global_path_all_dtypes(lib, torch_cuda, global_path, dtype):
 @pytest.mark.parametrize("dtype", [np.int32, np.float32, np.float64, np.uint8, np.float16])
 def test_global_path_batched_rows(lib, torch_cuda, global_path, dtype):
     # rows shorter than, equal to and longer than a tile; the look-back must stop at row starts
-    for shape in [(50, 129), (7, 4096), (5, 8192), (3, 8193), (4, 20011), (300, 1)]:
+    for shape in [(50, 129), (7, 4096), (5, 8192), (3, 8193), (5, 16384), (3, 16385), (4, 40011), (300, 1)]:
         check_rows(lib, torch_cuda, make_input(dtype, shape, seed=shape[0]), f"{np.dtype(dtype)} {shape} (global)")
 
 
 @pytest.mark.parametrize("dtype", [np.int32, np.float32, np.int64, np.float64, np.float16, np.uint8])
 def test_global_path_default_dispatch(lib, torch_cuda, dtype):
     # long rows take the global path without any override
-    for shape in [(1 << 20,), (3, 70001), (2, 8193)]:
+    for shape in [(1 << 20,), (3, 70001), (2, 8193), (2, 16385)]:
         check_rows(lib, torch_cuda, make_input(dtype, shape, seed=5), f"{np.dtype(dtype)} {shape}")
 
 
