@@ -28,6 +28,7 @@ SOURCES = [
     "sort_keys16.hip",
     "sort_keys32.hip",
     "sort_keys64.hip",
+    "sort_keys128.hip",
 ]
 
 HIPCC_FLAGS = [

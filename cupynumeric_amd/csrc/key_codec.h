@@ -15,7 +15,14 @@ namespace cpn {
 enum Codec : int {
   CODEC_UNSIGNED = 0,  // bool, uint8/16/32/64: identity
   CODEC_SIGNED   = 1,  // int8/16/32/64: flip the sign bit
-  CODEC_FLOAT    = 2   // float16/32/64: NaN -> all ones, -0 -> +0, then sign-magnitude flip
+  CODEC_FLOAT    = 2,  // float16/32/64: NaN -> all ones, -0 -> +0, then sign-magnitude flip
+  CODEC_COMPLEX  = 3   // complex64/128: (class, primary, secondary) of two float keys, see KeyTraits
+};
+
+// Raw bits of a complex128 element: real part in `lo`, imaginary part in `hi`.
+struct alignas(16) U128 {
+  uint64_t lo;
+  uint64_t hi;
 };
 
 template <typename U>
@@ -69,5 +76,90 @@ __host__ __device__ __forceinline__ uint32_t radix_digit(U raw, int shift)
 {
   return static_cast<uint32_t>(ordered_bits<CODEC, U>(raw) >> shift) & 0xFFu;
 }
+
+// What the sort kernels need to know about a key type: how many 8-bit passes sort it, the
+// digit of a pass, and the key as 64-bit words whose bytes are those digits (word p/8, byte
+// p%8), from which a row finds the passes on which all its keys agree.
+template <int CODEC, typename U>
+struct KeyTraits {
+  static constexpr int PASSES = sizeof(U);
+  static constexpr int NWORDS = 1;
+  static __host__ __device__ __forceinline__ uint32_t digit(U raw, int pass)
+  {
+    return radix_digit<CODEC, U>(raw, pass * 8);
+  }
+  static __host__ __device__ __forceinline__ void words(U raw, uint64_t (&w)[NWORDS])
+  {
+    w[0] = static_cast<uint64_t>(ordered_bits<CODEC, U>(raw));
+  }
+};
+
+// NumPy orders complex numbers by (real, imag) with NaNs last in this sense
+// (numpy/_core/src/npysort/npysort_common.h, CFLOAT_LT): first every element without NaN,
+// by real then imaginary part; then those whose imaginary part only is NaN, by real part;
+// then those whose real part is NaN, by imaginary part; last those with two NaNs.  As a radix
+// key: class (0..3) most significant, then a primary and a secondary float key
+//   class 0: (real, imag)   class 1: (real, -)   class 2: (imag, -)   class 3: (-, -)
+// so a complex key of 2w bits sorts in 2w/8 + 1 passes.  The reference sorts complex values
+// with thrust and `less<complex>` (src/cupynumeric/sort/thrust_sort.h:129-145).
+template <typename F>  // F = unsigned type of one component
+struct ComplexOrder {
+  F primary;
+  F secondary;
+  uint32_t cls;
+};
+template <typename F>
+__host__ __device__ __forceinline__ ComplexOrder<F> complex_order(F real_bits, F imag_bits)
+{
+  constexpr F nan_key = static_cast<F>(~static_cast<F>(0));
+  const F r           = ordered_bits<CODEC_FLOAT, F>(real_bits);
+  const F i           = ordered_bits<CODEC_FLOAT, F>(imag_bits);
+  const bool rn       = (r == nan_key);
+  const bool in       = (i == nan_key);
+  ComplexOrder<F> o;
+  o.cls       = (rn ? 2u : 0u) + (in ? 1u : 0u);
+  o.primary   = rn ? (in ? static_cast<F>(0) : i) : r;
+  o.secondary = (rn || in) ? static_cast<F>(0) : i;
+  return o;
+}
+
+template <>
+struct KeyTraits<CODEC_COMPLEX, uint64_t> {  // complex64: real in the low, imag in the high 32 bits
+  static constexpr int PASSES = 9;
+  static constexpr int NWORDS = 2;
+  static __host__ __device__ __forceinline__ void words(uint64_t raw, uint64_t (&w)[NWORDS])
+  {
+    const ComplexOrder<uint32_t> o =
+      complex_order<uint32_t>(static_cast<uint32_t>(raw), static_cast<uint32_t>(raw >> 32));
+    w[0] = (static_cast<uint64_t>(o.primary) << 32) | o.secondary;
+    w[1] = o.cls;
+  }
+  static __host__ __device__ __forceinline__ uint32_t digit(uint64_t raw, int pass)
+  {
+    uint64_t w[NWORDS];
+    words(raw, w);
+    return pass < 8 ? static_cast<uint32_t>(w[0] >> (pass * 8)) & 0xFFu : static_cast<uint32_t>(w[1]);
+  }
+};
+
+template <>
+struct KeyTraits<CODEC_COMPLEX, U128> {  // complex128
+  static constexpr int PASSES = 17;
+  static constexpr int NWORDS = 3;
+  static __host__ __device__ __forceinline__ void words(U128 raw, uint64_t (&w)[NWORDS])
+  {
+    const ComplexOrder<uint64_t> o = complex_order<uint64_t>(raw.lo, raw.hi);
+    w[0]                           = o.secondary;
+    w[1]                           = o.primary;
+    w[2]                           = o.cls;
+  }
+  static __host__ __device__ __forceinline__ uint32_t digit(U128 raw, int pass)
+  {
+    uint64_t w[NWORDS];
+    words(raw, w);
+    const uint64_t v = pass < 8 ? w[0] : (pass < 16 ? w[1] : w[2]);
+    return static_cast<uint32_t>(v >> ((pass & 7) * 8)) & 0xFFu;
+  }
+};
 
 }  // namespace cpn

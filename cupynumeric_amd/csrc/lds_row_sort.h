@@ -37,15 +37,7 @@ __device__ __forceinline__ T wave_reduce_or(T v)
   return v;
 }
 
-// Register type used for shuffles of a key (sub-word keys travel as 32 bits).
-template <typename KeyT>
-struct ShuffleWord {
-  using type = uint32_t;
-};
-template <>
-struct ShuffleWord<uint64_t> {
-  using type = unsigned long long;
-};
+using SkipWord = unsigned long long;  // a key's digits, eight to a word, as shuffled across the wave
 
 template <typename KeyT, int CODEC, bool HAS_IDX, int BLOCK, int ITEMS>
 __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in,
@@ -57,9 +49,11 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
   constexpr int WAVES  = BLOCK / WAVE;
   constexpr int TILE   = BLOCK * ITEMS;
   constexpr int WTILE  = ITEMS * WAVE;
-  constexpr int PASSES = sizeof(KeyT);
+  using KT             = KeyTraits<CODEC, KeyT>;
+  constexpr int PASSES = KT::PASSES;
+  constexpr int NW     = KT::NWORDS;
   using DT             = DigitThreads<BLOCK>;
-  using SW             = typename ShuffleWord<KeyT>::type;
+  using SW             = SkipWord;
   using IdxS           = uint16_t;  // row position while staged in LDS
   static_assert(TILE <= 65536, "row positions are staged as 16 bits");
 
@@ -67,7 +61,7 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
   __shared__ IdxS s_idx[HAS_IDX ? TILE : 1];
   __shared__ uint32_t s_ctr[WAVES * RADIX];
   __shared__ uint32_t s_wsum[DT::WAVES];
-  __shared__ SW s_red[2 * WAVES];
+  __shared__ SW s_red[2 * WAVES * NW];
 
   const int tid       = threadIdx.x;
   const int lane      = tid & (WAVE - 1);
@@ -78,45 +72,64 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
 
   KeyT key[ITEMS];
   uint32_t idx[HAS_IDX ? ITEMS : 1];
-  SW all_and = ~static_cast<SW>(0), all_or = 0;
+  SW all_and[NW], all_or[NW];
+#pragma unroll
+  for (int n = 0; n < NW; ++n) {
+    all_and[n] = ~static_cast<SW>(0);
+    all_or[n]  = 0;
+  }
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t o = woff + i * WAVE;
     if (full || o < seg) {
-      key[i]     = keys_in[base + o];
-      const SW v = static_cast<SW>(ordered_bits<CODEC, KeyT>(key[i]));
-      all_and &= v;
-      all_or |= v;
+      key[i] = keys_in[base + o];
+      uint64_t w[NW];
+      KT::words(key[i], w);
+#pragma unroll
+      for (int n = 0; n < NW; ++n) {
+        all_and[n] &= w[n];
+        all_or[n] |= w[n];
+      }
     } else {
-      key[i] = static_cast<KeyT>(0);
+      key[i] = KeyT{};
     }
     if constexpr (HAS_IDX) {
       idx[i] = o;
     }
   }
   // bits on which the keys of the row differ
-  all_and = wave_reduce_and(all_and);
-  all_or  = wave_reduce_or(all_or);
-  if (lane == 0) {
-    s_red[2 * wave]     = all_and;
-    s_red[2 * wave + 1] = all_or;
+#pragma unroll
+  for (int n = 0; n < NW; ++n) {
+    all_and[n] = wave_reduce_and(all_and[n]);
+    all_or[n]  = wave_reduce_or(all_or[n]);
+    if (lane == 0) {
+      s_red[(2 * wave) * NW + n]     = all_and[n];
+      s_red[(2 * wave + 1) * NW + n] = all_or[n];
+    }
   }
   __syncthreads();
-  SW varying;
-  {
-    SW a = s_red[0], o = s_red[1];
+  SW varying[NW];
+#pragma unroll
+  for (int n = 0; n < NW; ++n) {
+    SW a = s_red[n], o = s_red[NW + n];
 #pragma unroll
     for (int w = 1; w < WAVES; ++w) {
-      a &= s_red[2 * w];
-      o |= s_red[2 * w + 1];
+      a &= s_red[(2 * w) * NW + n];
+      o |= s_red[(2 * w + 1) * NW + n];
     }
-    varying = a ^ o;
+    varying[n] = a ^ o;
+  }
+  uint32_t active = 0;  // bit p: the keys of the row differ in digit p
+#pragma unroll
+  for (int p = 0; p < PASSES; ++p) {
+    if (((varying[p / 8] >> ((p % 8) * RADIX_BITS)) & 0xFFu) != 0) {
+      active |= 1u << p;
+    }
   }
 
   uint32_t* wctr = s_ctr + wave * RADIX;
   for (int pass = 0; pass < PASSES; ++pass) {
-    const int shift = pass * RADIX_BITS;
-    if (((varying >> shift) & 0xFFu) == 0) {
+    if (((active >> pass) & 1u) == 0) {
       continue;  // uniform for the block
     }
     for (int j = tid; j < WAVES * RADIX; j += BLOCK) {
@@ -128,7 +141,7 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
 #pragma unroll
     for (int i = 0; i < ITEMS; ++i) {
       const bool valid = full || (woff + i * WAVE < seg);
-      const uint32_t d = radix_digit<CODEC, KeyT>(key[i], shift);
+      const uint32_t d = KT::digit(key[i], pass);
       dpk[i / 4]       = (i % 4 == 0) ? d : (dpk[i / 4] | (d << (8 * (i % 4))));
       rnk[i]           = wave_match_rank(d, valid, wctr);
     }

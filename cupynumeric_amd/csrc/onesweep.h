@@ -78,17 +78,20 @@ constexpr int HIST_BLOCK = 256;
 // queueing on one address.
 // Measured on 2^28 float32 keys: 1 copy 0.51 ms, 2: 0.37, 4: 0.30, 8: 0.27 ms (= the read rate of
 // a plain reduction on the same device).  64-bit keys have twice the histograms: 4 copies keep
-// the block at 32 KiB of LDS.
-__host__ __device__ constexpr int hist_copies(int key_bytes) { return key_bytes == 8 ? 4 : 8; }
+// the block at 32 KiB of LDS
+// (complex keys: 9 passes x 4 copies, 17 passes x 2 copies).
+__host__ __device__ constexpr int hist_copies(int passes) { return passes <= 4 ? 8 : (passes <= 9 ? 4 : 2); }
 
 template <typename KeyT, int CODEC, int PASSES>
 __device__ __forceinline__ void hist_accumulate(uint32_t* s_hist, KeyT raw, uint32_t copy)
 {
-  constexpr int HIST_COPIES = hist_copies(sizeof(KeyT));
-  const KeyT o              = ordered_bits<CODEC, KeyT>(raw);
+  using KT                  = KeyTraits<CODEC, KeyT>;
+  constexpr int HIST_COPIES = hist_copies(PASSES);
+  uint64_t w[KT::NWORDS];
+  KT::words(raw, w);
 #pragma unroll
   for (int p = 0; p < PASSES; ++p) {
-    const uint32_t d = static_cast<uint32_t>(o >> (p * RADIX_BITS)) & 0xFFu;
+    const uint32_t d = static_cast<uint32_t>(w[p / 8] >> ((p % 8) * RADIX_BITS)) & 0xFFu;
     atomicAdd(&s_hist[(p * RADIX + d) * HIST_COPIES + copy], 1u);
   }
 }
@@ -102,9 +105,9 @@ __global__ __launch_bounds__(HIST_BLOCK) void histogram_kernel(const KeyT* __res
                                                                  uint32_t blocks_per_row,
                                                                  uint64_t chunk)
 {
-  constexpr int PASSES      = sizeof(KeyT);
+  constexpr int PASSES      = KeyTraits<CODEC, KeyT>::PASSES;
   constexpr int VEC         = 16 / sizeof(KeyT);
-  constexpr int HIST_COPIES = hist_copies(sizeof(KeyT));
+  constexpr int HIST_COPIES = hist_copies(PASSES);
   __shared__ uint32_t s_hist[PASSES * RADIX * HIST_COPIES];
 
   const int tid        = threadIdx.x;
@@ -224,7 +227,7 @@ struct SweepArgs {
   int64_t index_offset;
   uint32_t tiles_per_row;
   uint32_t num_tiles;
-  int shift;               // bit position of this pass's digit
+  int pass;                // which 8-bit digit this pass sorts by
   int idx_final;           // idx_out is the caller's int64 array
 };
 
@@ -284,7 +287,7 @@ __device__ __forceinline__ void onesweep_tile(
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t o = woff + i * WAVE;
-    key[i]           = (FULL || o < count) ? kin[o] : static_cast<KeyT>(0);
+    key[i]           = (FULL || o < count) ? kin[o] : KeyT{};
     if constexpr (XFORM) {
       key[i] = ordered_bits<CODEC, KeyT>(key[i]);
     }
@@ -296,7 +299,7 @@ __device__ __forceinline__ void onesweep_tile(
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const bool valid = FULL || (woff + i * WAVE < count);
-    const uint32_t d = radix_digit<DCODEC, KeyT>(key[i], a.shift);
+    const uint32_t d = KeyTraits<DCODEC, KeyT>::digit(key[i], a.pass);
     dpk[i / 4]       = (i % 4 == 0) ? d : (dpk[i / 4] | (d << (8 * (i % 4))));
     const uint32_t r = wave_match_rank(d, valid, wctr) & 0xFFFFu;
     rnk2[i / 2]      = (i % 2 == 0) ? r : (rnk2[i / 2] | (r << 16));
@@ -436,11 +439,11 @@ __device__ __forceinline__ void onesweep_tile(
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
       const uint32_t p = tid + k * BLOCK;
-      kk[k]            = (FULL || p < count) ? s_keys[p] : static_cast<KeyT>(0);
+      kk[k]            = (FULL || p < count) ? s_keys[p] : KeyT{};
     }
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
-      const uint32_t d = radix_digit<DCODEC, KeyT>(kk[k], a.shift);
+      const uint32_t d = KeyTraits<DCODEC, KeyT>::digit(kk[k], a.pass);
       dq[k / 4]        = (k % 4 == 0) ? d : (dq[k / 4] | (d << (8 * (k % 4))));
     }
     if (a.keys_out != nullptr) {

@@ -53,8 +53,8 @@ static KeyKind key_kind(int dtype)
     case CPN_FLOAT16: return {2, CODEC_FLOAT};
     case CPN_FLOAT32: return {4, CODEC_FLOAT};
     case CPN_FLOAT64: return {8, CODEC_FLOAT};
-    case CPN_COMPLEX64: return {8, -1};
-    case CPN_COMPLEX128: return {16, -1};
+    case CPN_COMPLEX64: return {8, CODEC_COMPLEX};
+    case CPN_COMPLEX128: return {16, CODEC_COMPLEX};
     default: return {0, -1};
   }
 }
@@ -93,8 +93,8 @@ uint64_t cpn_dtype_size(int dtype) { return static_cast<uint64_t>(cpn::key_kind(
 uint64_t cpn_key_order_bits(int dtype, uint64_t raw_bits)
 {
   const cpn::KeyKind k = cpn::key_kind(dtype);
-  if (k.bytes == 0 || k.codec < 0) {
-    return 0;
+  if (k.bytes == 0 || k.codec < 0 || k.codec == cpn::CODEC_COMPLEX) {
+    return 0;  // complex keys are wider than 64 bits
   }
   switch (k.bytes * 4 + k.codec) {
     case 1 * 4 + cpn::CODEC_UNSIGNED: return cpn::ordered_bits<cpn::CODEC_UNSIGNED, uint8_t>(static_cast<uint8_t>(raw_bits));
@@ -125,7 +125,7 @@ uint64_t cpn_local_sort_temp_bytes(int dtype, uint64_t volume, uint64_t sort_dim
   if (sort_dim_size == 0 || volume % sort_dim_size != 0) {
     return 0;
   }
-  return cpn::workspace_bytes(k.bytes, volume, sort_dim_size, want_values != 0, want_indices != 0, in_place != 0);
+  return cpn::workspace_bytes(k.bytes, cpn::key_passes(k.bytes, k.codec), volume, sort_dim_size, want_values != 0, want_indices != 0, in_place != 0);
 }
 
 int cpn_local_sort(int dtype, const void* values_in, void* values_out, int64_t* indices_out, uint64_t volume,
@@ -169,6 +169,7 @@ int cpn_local_sort(int dtype, const void* values_in, void* values_out, int64_t* 
     case 2: return cpn::sort_keys16(k.codec, r);
     case 4: return cpn::sort_keys32(k.codec, r);
     case 8: return cpn::sort_keys64(k.codec, r);
+    case 16: return cpn::sort_keys128(k.codec, r);
     default: return CPN_ERR_UNSUPPORTED;
   }
 }

@@ -47,7 +47,7 @@ __host__ __device__ constexpr int global_block(int /*key_bytes*/) { return CPN_G
 // area stays at 64 KiB: two workgroups of 512 threads fit in a CU's 160 KiB)
 __host__ __device__ constexpr int global_items(int key_bytes, bool big)
 {
-  return (key_bytes == 8 || big) ? CPN_GLOBAL_ITEMS / 2 : CPN_GLOBAL_ITEMS;
+  return key_bytes == 16 ? CPN_GLOBAL_ITEMS / 4 : ((key_bytes == 8 || big) ? CPN_GLOBAL_ITEMS / 2 : CPN_GLOBAL_ITEMS);
 }
 __host__ __device__ constexpr int global_tile(int key_bytes, bool big)
 {
@@ -55,7 +55,15 @@ __host__ __device__ constexpr int global_tile(int key_bytes, bool big)
 }
 
 // Longest row the LDS kernel can take, per key width (keeps static LDS below 64 KiB).
-__host__ __device__ constexpr uint64_t lds_row_capacity(int key_bytes) { return key_bytes == 8 ? 4096 : 8192; }
+__host__ __device__ constexpr uint64_t lds_row_capacity(int key_bytes)
+{
+  return key_bytes == 16 ? 2048 : (key_bytes == 8 ? 4096 : 8192);
+}
+// Radix passes of a key: one per byte, plus the NaN-class pass of complex keys.
+__host__ __device__ constexpr int key_passes(int key_bytes, int codec)
+{
+  return codec == CODEC_COMPLEX ? key_bytes + 1 : key_bytes;
+}
 
 // Row length up to which the LDS kernel is used.  Equals lds_row_capacity unless the
 // environment variable CPN_SORT_LDS_ROW_LIMIT or cpn_set_lds_row_limit lowers it, e.g. to 0
@@ -90,12 +98,12 @@ struct GlobalLayout {
   bool valid;
 };
 
-inline GlobalLayout global_layout(int key_bytes, uint64_t volume, uint64_t seg, bool want_values,
+inline GlobalLayout global_layout(int key_bytes, int passes, uint64_t volume, uint64_t seg, bool want_values,
                                   bool want_indices, bool in_place)
 {
   GlobalLayout L{};
   L.big           = seg >= BIG_ROW_ELEMENTS;
-  L.passes        = key_bytes;
+  L.passes        = passes;
   L.rows          = volume / seg;
   const uint64_t tile = static_cast<uint64_t>(global_tile(key_bytes, L.big));
   const uint64_t tpr  = (seg + tile - 1) / tile;
@@ -137,13 +145,13 @@ inline GlobalLayout global_layout(int key_bytes, uint64_t volume, uint64_t seg, 
   return L;
 }
 
-inline uint64_t workspace_bytes(int key_bytes, uint64_t volume, uint64_t seg, bool want_values,
+inline uint64_t workspace_bytes(int key_bytes, int passes, uint64_t volume, uint64_t seg, bool want_values,
                                 bool want_indices, bool in_place)
 {
   if (volume == 0 || seg <= lds_row_limit(key_bytes)) {
     return HEADER_BYTES;
   }
-  const GlobalLayout L = global_layout(key_bytes, volume, seg, want_values, want_indices, in_place);
+  const GlobalLayout L = global_layout(key_bytes, passes, volume, seg, want_values, want_indices, in_place);
   return L.valid ? L.total : 0;
 }
 
@@ -195,13 +203,17 @@ inline int sort_rows_in_lds(const SortRequest& r)
     return launch_lds_rows<KeyT, CODEC, HAS_IDX, 64, 4>(r);
   } else if (r.seg <= 1024) {
     return launch_lds_rows<KeyT, CODEC, HAS_IDX, 256, 4>(r);
-  } else if (r.seg <= 4096) {
-    return launch_lds_rows<KeyT, CODEC, HAS_IDX, 256, 16>(r);
+  }
+  if constexpr (sizeof(KeyT) == 16) {
+    return launch_lds_rows<KeyT, CODEC, HAS_IDX, 256, 8>(r);  // up to lds_row_capacity(16) == 2048
   } else {
+    if (r.seg <= 4096) {
+      return launch_lds_rows<KeyT, CODEC, HAS_IDX, 256, 16>(r);
+    }
     if constexpr (sizeof(KeyT) < 8) {
       return launch_lds_rows<KeyT, CODEC, HAS_IDX, 512, 16>(r);
     } else {
-      return CPN_ERR_UNSUPPORTED;  // not reached: lds_row_limit(8) == 4096
+      return CPN_ERR_UNSUPPORTED;  // not reached: lds_row_capacity(8) == 4096
     }
   }
 }
@@ -214,7 +226,7 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
   constexpr int KB     = sizeof(KeyT);
   constexpr int BLOCK  = global_block(KB);
   constexpr int ITEMS  = global_items(KB, BIG);
-  constexpr int PASSES = KB;
+  constexpr int PASSES = KeyTraits<CODEC, KeyT>::PASSES;
   unsigned char* ws    = static_cast<unsigned char*>(r.temp);
   const bool in_place  = (r.values_out == r.values_in);
   const bool want_vals = (r.values_out != nullptr);
@@ -270,7 +282,7 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
 
   // Index-only sorts never return the keys: the first pass stores their order-preserving
   // unsigned image in the workspace and the later passes run with the identity codec.
-  constexpr bool CAN_ORDER_KEYS = HAS_IDX && CODEC != CODEC_UNSIGNED && PASSES >= 2;
+  constexpr bool CAN_ORDER_KEYS = HAS_IDX && (CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT) && PASSES >= 2;
   const bool ordered_keys       = CAN_ORDER_KEYS && !want_vals;
 
   const void* key_src = r.values_in;
@@ -302,7 +314,7 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
     a.index_offset    = r.index_offset;
     a.tiles_per_row   = L.tiles_per_row;
     a.num_tiles       = static_cast<uint32_t>(L.num_tiles);
-    a.shift           = p * RADIX_BITS;
+    a.pass            = p;
     a.idx_final       = last ? 1 : 0;
     {
       ProfileScope prof("onesweep", r.stream);
@@ -338,10 +350,11 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
 template <typename KeyT, int CODEC>
 int sort_typed(const SortRequest& r)
 {
-  constexpr int KB    = sizeof(KeyT);
-  const bool has_idx  = (r.indices_out != nullptr);
-  const bool in_place = (r.values_out == r.values_in);
-  const uint64_t need = workspace_bytes(KB, r.volume, r.seg, r.values_out != nullptr, has_idx, in_place);
+  constexpr int KB     = sizeof(KeyT);
+  constexpr int PASSES = KeyTraits<CODEC, KeyT>::PASSES;
+  const bool has_idx   = (r.indices_out != nullptr);
+  const bool in_place  = (r.values_out == r.values_in);
+  const uint64_t need  = workspace_bytes(KB, PASSES, r.volume, r.seg, r.values_out != nullptr, has_idx, in_place);
   if (need == 0) {
     return CPN_ERR_UNSUPPORTED;
   }
@@ -355,7 +368,7 @@ int sort_typed(const SortRequest& r)
     }
     return has_idx ? sort_rows_in_lds<KeyT, CODEC, true>(r) : sort_rows_in_lds<KeyT, CODEC, false>(r);
   }
-  const GlobalLayout L = global_layout(KB, r.volume, r.seg, r.values_out != nullptr, has_idx, in_place);
+  const GlobalLayout L = global_layout(KB, PASSES, r.volume, r.seg, r.values_out != nullptr, has_idx, in_place);
   if (L.big) {
     return has_idx ? sort_global<KeyT, CODEC, true, true>(r, L) : sort_global<KeyT, CODEC, true, false>(r, L);
   }
@@ -367,5 +380,6 @@ int sort_keys8(int codec, const SortRequest& r);
 int sort_keys16(int codec, const SortRequest& r);
 int sort_keys32(int codec, const SortRequest& r);
 int sort_keys64(int codec, const SortRequest& r);
+int sort_keys128(int codec, const SortRequest& r);
 
 }  // namespace cpn

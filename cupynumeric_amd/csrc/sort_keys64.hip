@@ -11,6 +11,7 @@ int sort_keys64(int codec, const SortRequest& r)
     case CODEC_UNSIGNED: return sort_typed<uint64_t, CODEC_UNSIGNED>(r);
     case CODEC_SIGNED: return sort_typed<uint64_t, CODEC_SIGNED>(r);
     case CODEC_FLOAT: return sort_typed<uint64_t, CODEC_FLOAT>(r);
+    case CODEC_COMPLEX: return sort_typed<uint64_t, CODEC_COMPLEX>(r);  // complex64
     default: return CPN_ERR_DTYPE;
   }
 }

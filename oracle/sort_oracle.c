@@ -16,7 +16,8 @@
  *
  * thrust itself (CCCL, pulled in through Legate; not under /root/reference) is not restated:
  * the per-segment sort is a textbook stable merge sort.  Its comparison is NumPy's order --
- * integers by value, floats ascending with every NaN last and -0.0 == +0.0 -- which is the
+ * integers by value, floats ascending with every NaN last and -0.0 == +0.0, complex numbers by
+ * (real, imag) with NaNs last -- which is the
  * ordering contract of this build; thrust's own treatment of NaN (unordered under `less`,
  * bit-pattern order under its host radix sort) is deliberately not reproduced.  Unstable
  * kinds are served by the same stable sort (any stable result is a valid unstable one).
@@ -35,7 +36,7 @@
 #endif
 
 /* element type codes: same values as enum cpn_dtype in include/cpn_sort.h */
-enum { T_BOOL, T_I8, T_I16, T_I32, T_I64, T_U8, T_U16, T_U32, T_U64, T_F16, T_F32, T_F64 };
+enum { T_BOOL, T_I8, T_I16, T_I32, T_I64, T_U8, T_U16, T_U32, T_U64, T_F16, T_F32, T_F64, T_C64, T_C128 };
 
 /* ---- NumPy's "less" for floating point: a < b, or b is NaN and a is not ---------------- */
 static inline int less_f32(float a, float b) { return a < b || (b != b && a == a); }
@@ -69,6 +70,31 @@ static inline float half_to_float(uint16_t h)
   return f;
 }
 static inline int less_f16(uint16_t a, uint16_t b) { return less_f32(half_to_float(a), half_to_float(b)); }
+
+/*
+ * Complex numbers: NumPy's order (numpy/_core/src/npysort/npysort_common.h, CFLOAT_LT /
+ * CDOUBLE_LT), restated branch for branch: lexicographic on (real, imag) with NaNs last.  The
+ * reference compares complex values with thrust and `less` on legate::Complex
+ * (src/cupynumeric/sort/thrust_sort.h:129-145), which agrees on NaN-free data (the only data
+ * its tests feed, tests/cpp/integration/test_sort.cc:98-134).
+ */
+typedef struct { float re, im; } c64_t;
+typedef struct { double re, im; } c128_t;
+#define DEFINE_CLT(NAME, T)                                                            \
+  static inline int NAME(T a, T b)                                                     \
+  {                                                                                    \
+    if (a.re < b.re) {                                                                 \
+      return a.im == a.im || b.im != b.im;                                             \
+    } else if (a.re > b.re) {                                                          \
+      return b.im != b.im && a.im == a.im;                                             \
+    } else if (a.re == b.re || (a.re != a.re && b.re != b.re)) {                       \
+      return a.im < b.im || (b.im != b.im && a.im == a.im);                            \
+    } else {                                                                           \
+      return b.re != b.re;                                                             \
+    }                                                                                  \
+  }
+DEFINE_CLT(less_c64, c64_t)
+DEFINE_CLT(less_c128, c128_t)
 
 #define LESS_INT(a, b) ((a) < (b))
 
@@ -218,6 +244,8 @@ DEFINE_SORT(s_i64, int64_t, LESS_INT)
 DEFINE_SORT(s_f16, uint16_t, less_f16)
 DEFINE_SORT(s_f32, float, less_f32)
 DEFINE_SORT(s_f64, double, less_f64)
+DEFINE_SORT(s_c64, c64_t, less_c64)
+DEFINE_SORT(s_c128, c128_t, less_c128)
 
 static size_t elem_size(int dtype)
 {
@@ -225,7 +253,8 @@ static size_t elem_size(int dtype)
     case T_BOOL: case T_I8: case T_U8: return 1;
     case T_I16: case T_U16: case T_F16: return 2;
     case T_I32: case T_U32: case T_F32: return 4;
-    case T_I64: case T_U64: case T_F64: return 8;
+    case T_I64: case T_U64: case T_F64: case T_C64: return 8;
+    case T_C128: return 16;
     default: return 0;
   }
 }
@@ -272,6 +301,8 @@ int cpn_oracle_local_sort(int dtype, const void* input, void* values, int64_t* i
     case T_F16: return s_f16_local_sort_inplace((uint16_t*)values, indices, volume, seg, threads);
     case T_F32: return s_f32_local_sort_inplace((float*)values, indices, volume, seg, threads);
     case T_F64: return s_f64_local_sort_inplace((double*)values, indices, volume, seg, threads);
+    case T_C64: return s_c64_local_sort_inplace((c64_t*)values, indices, volume, seg, threads);
+    case T_C128: return s_c128_local_sort_inplace((c128_t*)values, indices, volume, seg, threads);
     default: return -2;
   }
 }

@@ -27,7 +27,7 @@ from numpy.lib.array_utils import normalize_axis_index
 HERE = Path(__file__).resolve().parent
 LIB_PATH = HERE / "_build" / "libcpnoracle.so"
 
-# same codes as enum cpn_dtype (include/cpn_sort.h); complex is outside the oracle
+# same codes as enum cpn_dtype (include/cpn_sort.h)
 DTYPE_CODES = {
     np.dtype(np.bool_): 0,
     np.dtype(np.int8): 1,
@@ -41,6 +41,8 @@ DTYPE_CODES = {
     np.dtype(np.float16): 9,
     np.dtype(np.float32): 10,
     np.dtype(np.float64): 11,
+    np.dtype(np.complex64): 12,
+    np.dtype(np.complex128): 13,
 }
 
 _lib = None

@@ -28,6 +28,8 @@ def reference_vectors():
 def bits(a: np.ndarray) -> np.ndarray:
     """Unsigned-integer view of an array, so that NaN payloads and zero signs are compared."""
     a = np.ascontiguousarray(a)
+    if a.dtype.itemsize == 16:  # complex128: two words per element
+        return a.reshape(-1).view(np.uint64)
     return a.view({1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[a.dtype.itemsize])
 
 
@@ -39,12 +41,27 @@ def assert_same_bits(got: np.ndarray, want: np.ndarray, what: str = "") -> None:
     if got.size == 0:
         return
     if not np.array_equal(bits(got), bits(want)):
-        bad = np.flatnonzero(bits(got).reshape(-1) != bits(want).reshape(-1))
+        bad = np.flatnonzero(bits(got).reshape(-1) != bits(want).reshape(-1)) // (2 if got.dtype.itemsize == 16 else 1)
         raise AssertionError(
             f"{what}: {bad.size} of {got.size} elements differ, first at flat index {bad[0]}: "
             f"got {got.reshape(-1)[bad[0]]!r}, want {want.reshape(-1)[bad[0]]!r}"
         )
 
+
+def case_array(values, dtype, shape=None) -> np.ndarray:
+    """Array of a golden-vector case; complex values are stored as [real, imag] pairs."""
+    dt = np.dtype(dtype)
+    if dt.kind == "c" :
+        pairs = np.array(values, dtype=np.float64).reshape(-1, 2)
+        out = np.empty(len(pairs), dtype=dt)
+        out.real = pairs[:, 0]
+        out.imag = pairs[:, 1]
+    else:
+        out = np.array(values, dtype=dt)
+    return out if shape is None else out.reshape(shape)
+
+
+COMPLEX_DTYPES = [np.complex64, np.complex128]
 
 ALL_REAL_DTYPES = [
     np.bool_, np.int8, np.int16, np.int32, np.int64,
@@ -59,6 +76,17 @@ def make_input(dtype, shape, seed: int, special: bool = True, duplicates: bool =
     rng = np.random.default_rng(seed)
     dt = np.dtype(dtype)
     n = int(np.prod(shape, dtype=np.int64))
+    if dt.kind == "c":
+        # few distinct real parts so that the imaginary part decides often; specials in both parts
+        part = np.float32 if dt == np.complex64 else np.float64
+        re = make_input(part, (n,), seed * 2 + 1, special)
+        im = make_input(part, (n,), seed * 2 + 2, special)
+        if n:
+            re = np.where(rng.random(n) < 0.6, np.round(re * 2) / 2, re).astype(part)
+        x = np.empty(n, dtype=dt)
+        x.real = re
+        x.imag = im
+        return x.reshape(shape)
     if dt.kind == "f":
         x = rng.standard_normal(n).astype(dt)
         if special and n:

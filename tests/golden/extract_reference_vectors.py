@@ -9,8 +9,8 @@ expected outputs in
     tests/cpp/integration/test_argsort.cc  (12-element :26-60, 4-D..7-D :62-204, inputs :282-377)
 The reference is read as text, never imported, built or run.  Cases the reference generates by
 formula (10 000 reversed elements :379-410, empty :412-433, single item :435-455) are restated as
-formulas in tests/test_oracle.py instead of being stored.  Complex inputs are left out (complex
-sorting is not built yet).
+formulas in tests/test_oracle.py instead of being stored.  Complex values are stored as
+[real, imag] pairs (test_sort.cc:98-134,557-571, test_argsort.cc:298-311,330-344).
 """
 from __future__ import annotations
 
@@ -41,6 +41,21 @@ def parse_expect_table(body: str) -> list[dict[str, list[float]]]:
     init = body[body.index("= {") + 2 : body.rindex("};") + 1]
     nested = json.loads(init.replace("{", "[").replace("}", "]"))
     return [{str(axis): vals for axis, vals in per_shape} for per_shape in nested]
+
+
+COMPLEX = re.compile(r"legate::Complex<float>\(\s*([-0-9.eE]+)\s*,\s*([-0-9.eE]+)\s*\)")
+
+
+def decomplex(text: str) -> str:
+    """`legate::Complex<float>(a, b)` -> `{a, b}` so that the generic brace parser applies."""
+    return COMPLEX.sub(lambda m: "{" + m.group(1) + "," + m.group(2) + "}", text)
+
+
+def parse_complex_array(text: str, decl: str) -> list[list[float]]:
+    i = text.index(decl)
+    j = text.index("{", i)
+    k = text.index("};", j)
+    return [[float(a), float(b)] for a, b in COMPLEX.findall(text[j:k])]
 
 
 def parse_shapes(text: str, anchor: str) -> list[list[int]]:
@@ -92,14 +107,22 @@ def main() -> None:
     add("sort", "float64", parse_array(body, "in_array2"), shapes12,
         parse_expect_table(function_body(sort_cc, "get_expect_result_double")), False, "test_sort.cc:62-96,552")
 
+    add("sort", "complex64", parse_complex_array(body, "in_array3"), shapes12,
+        parse_expect_table(decomplex(function_body(sort_cc, "get_expect_result_complex"))), False,
+        "test_sort.cc:98-134,557")
+
     # argsort: test_argsort.cc
     table12 = parse_expect_table(function_body(argsort_cc, "get_argsort_expect_result"))
     body = argsort_cc[argsort_cc.index("void argsort_basic_axis()") :]
     add("argsort", "int32", parse_array(body, "in_array1"), shapes12, table12, False, "test_argsort.cc:26-60,290")
     add("argsort", "float64", parse_array(body, "in_array2"), shapes12, table12, False, "test_argsort.cc:26-60,294")
+    add("argsort", "complex64", parse_complex_array(body, "in_array3"), shapes12, table12, False,
+        "test_argsort.cc:26-60,298")
     body = argsort_cc[argsort_cc.index("void argsort_basic_axis_stable()") :]
     add("argsort", "int32", parse_array(body, "in_array1"), shapes12, table12, True, "test_argsort.cc:26-60,321")
     add("argsort", "float64", parse_array(body, "in_array2"), shapes12, table12, True, "test_argsort.cc:26-60,326")
+    add("argsort", "complex64", parse_complex_array(body, "in_array3"), shapes12, table12, True,
+        "test_argsort.cc:26-60,330")
 
     body = argsort_cc[argsort_cc.index("void argsort_basic_axis_max_dim()") :]
     data16 = parse_array(body, "in_array")

@@ -65,7 +65,7 @@ def test_argument_validation_without_a_device(lib):
     assert sort(3, 16, 32, None, 4, 4, 0, 1, None, 0, None) == _lib.CPN_ERR_TEMP
     assert sort(3, 16, 32, None, 4, 4, 0, 1, 256, 16, None) == _lib.CPN_ERR_TEMP  # too small
     assert sort(3, 16, 32, None, 4, 4, 0, 1, 264, 4096, None) == _lib.CPN_ERR_TEMP  # misaligned
-    assert sort(12, 16, 32, None, 4, 4, 0, 1, 256, 256, None) == _lib.CPN_ERR_UNSUPPORTED  # complex64
+    assert sort(13, 24, 32, None, 4, 4, 0, 1, 256, 256, None) == _lib.CPN_ERR_ALIGN  # complex128 needs 16-byte alignment
     assert lib.cpn_local_sort_check(None, None) == _lib.CPN_ERR_NULL
     swap = lib.cpn_swapaxes_copy
     import ctypes
@@ -100,6 +100,10 @@ def test_temp_bytes_layout(lib):
     assert tb(u8, n, n, 0, 1, 0) == t8
     # monotone in the request
     assert tb(i64, n, n, 0, 1, 0) > tb(f32, n, n, 0, 1, 0) > tb(f16, n, n, 0, 1, 0)
+    # complex keys take one more pass (the NaN class) than their bytes
+    c64, c128 = 12, 13
+    assert tb(c64, n, n, 1, 0, 0) == 256 + 9 * 256 * 4 + 9 * (n // 8192) * 256 * 4 + 8 * n
+    assert tb(c128, n, n, 1, 0, 0) == 256 + 17 * 256 * 4 + 17 * (n // 4096) * 256 * 4 + 16 * n
     # the row-length switch moves work to the global path
     prev = lib.cpn_set_lds_row_limit(0)
     try:

@@ -7,22 +7,22 @@ import itertools
 
 import numpy as np
 import pytest
-from conftest import ALL_REAL_DTYPES, assert_same_bits, make_input
+from conftest import ALL_REAL_DTYPES, COMPLEX_DTYPES, assert_same_bits, case_array, make_input
 
 from oracle import sort_oracle as oracle
 
 
 # ---- golden vectors of the reference's own tests ------------------------------------------------
 def test_reference_golden_vectors(reference_vectors):
-    assert len(reference_vectors) == 300
+    assert len(reference_vectors) == 390
     for case in reference_vectors:
-        x = np.array(case["input"], dtype=case["dtype"]).reshape(case["shape"])
+        x = case_array(case["input"], case["dtype"], case["shape"])
         # kinds the reference runs the case with (tests/cpp/integration/test_argsort.cc:221-224)
         kinds = ["mergesort", "stable"] if case["stable_only"] else ["quicksort", "mergesort", "heapsort", "stable"]
         for kind in kinds:
             if case["op"] == "sort":
                 got = oracle.sort(x, axis=case["axis"], kind=kind)
-                want = np.array(case["expect"], dtype=case["dtype"]).reshape(case["shape"])
+                want = case_array(case["expect"], case["dtype"], case["shape"])
             else:
                 got = oracle.argsort(x, axis=case["axis"], kind=kind)
                 want = np.array(case["expect"], dtype=np.int64).reshape(case["shape"])
@@ -72,7 +72,7 @@ def test_reference_negative():
 
 
 # ---- NumPy's own stable sort as an independent implementation ------------------------------------
-@pytest.mark.parametrize("dtype", ALL_REAL_DTYPES)
+@pytest.mark.parametrize("dtype", ALL_REAL_DTYPES + COMPLEX_DTYPES)
 @pytest.mark.parametrize("threads", [1, 4])
 def test_against_numpy_1d(dtype, threads):
     for n in (1, 2, 3, 17, 24, 25, 1000, 70001):
@@ -81,7 +81,7 @@ def test_against_numpy_1d(dtype, threads):
         assert_same_bits(oracle.sort(x, kind="stable", threads=threads), np.sort(x, kind="stable"), f"{dtype} n={n}")
 
 
-@pytest.mark.parametrize("dtype", [np.int32, np.float32, np.float16, np.float64, np.uint8])
+@pytest.mark.parametrize("dtype", [np.int32, np.float32, np.float16, np.float64, np.uint8, np.complex64])
 def test_against_numpy_axes(dtype):
     for shape in [(5, 5), (7, 1, 9), (3, 4, 5, 6), (33, 65)]:
         x = make_input(dtype, shape, seed=len(shape))
@@ -151,3 +151,40 @@ def test_bruteforce_float_alphabet(dtype, ubits):
     got = oracle.argsort(x, kind="stable")
     assert got.tolist() == insertion_argsort(x)
     assert_same_bits(oracle.sort(x), x[got])
+
+
+# ---- complex: brute force with NumPy's rule written from its definition ----------------------------
+def complex_rule_less(a: complex, b: complex) -> bool:
+    """a sorts strictly before b: classes (no NaN) < (imag NaN) < (real NaN) < (both NaN); inside a
+    class by real then imag, by real, by imag, none."""
+    def key(z):
+        rn, inn = z.real != z.real, z.imag != z.imag
+        cls = 2 * rn + inn
+        return cls, (z.real if not rn else (z.imag if not inn else 0.0)), (z.imag if cls == 0 else 0.0)
+    (ca, pa, sa), (cb, pb, sb) = key(a), key(b)
+    if ca != cb:
+        return ca < cb
+    if pa != pb:
+        return pa < pb
+    return sa < sb
+
+
+@pytest.mark.parametrize("dtype", COMPLEX_DTYPES)
+def test_bruteforce_complex_alphabet(dtype):
+    part = [np.nan, -np.inf, -1.0, -0.0, 0.0, 1.0, np.inf]
+    alphabet = np.empty(len(part) ** 2, dtype=dtype)
+    alphabet.real = np.repeat(part, len(part))
+    alphabet.imag = np.tile(part, len(part))
+    rng = np.random.default_rng(11)
+    for trial in range(40):
+        x = alphabet[rng.integers(0, len(alphabet), 60)]
+        order: list[int] = []
+        for i, v in enumerate(x):
+            j = len(order)
+            while j > 0 and complex_rule_less(complex(v), complex(x[order[j - 1]])):
+                j -= 1
+            order.insert(j, i)
+        got = oracle.argsort(x, kind="stable")
+        assert got.tolist() == order, (dtype, trial)
+        assert got.tolist() == np.argsort(x, kind="stable").tolist()
+        assert_same_bits(oracle.sort(x), x[got])

@@ -7,7 +7,9 @@ import ctypes
 
 import numpy as np
 import pytest
-from conftest import ALL_REAL_DTYPES, assert_same_bits, make_input
+from conftest import ALL_REAL_DTYPES, COMPLEX_DTYPES, assert_same_bits, case_array, make_input
+
+ALL_DTYPES = ALL_REAL_DTYPES + COMPLEX_DTYPES
 
 import cupynumeric_amd as num
 from cupynumeric_amd import _lib
@@ -77,13 +79,13 @@ def check_rows(lib, torch, x, what):
 # ---- golden vectors of the reference, through the public API ------------------------------------
 def test_reference_golden_vectors(reference_vectors):
     for case in reference_vectors:
-        x = np.array(case["input"], dtype=case["dtype"]).reshape(case["shape"])
+        x = case_array(case["input"], case["dtype"], case["shape"])
         a = num.array(x)
         kinds = ["mergesort", "stable"] if case["stable_only"] else ["quicksort", "mergesort", "heapsort", "stable"]
         for kind in kinds:
             where = f"{case['where']} shape={case['shape']} axis={case['axis']} kind={kind}"
             if case["op"] == "sort":
-                want = np.array(case["expect"], dtype=case["dtype"]).reshape(case["shape"])
+                want = case_array(case["expect"], case["dtype"], case["shape"])
                 assert_same_bits(np.asarray(num.sort(a, axis=case["axis"], kind=kind)), want, where)
             else:
                 want = np.array(case["expect"], dtype=np.int64).reshape(case["shape"])
@@ -154,9 +156,9 @@ def test_random_module_and_flatten():
 LDS_LENGTHS = [1, 2, 3, 63, 64, 65, 255, 256, 257, 1000, 1023, 1024, 1025, 4095, 4096, 4097, 8191, 8192]
 
 
-@pytest.mark.parametrize("dtype", ALL_REAL_DTYPES)
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
 def test_lds_rows_all_dtypes(lib, torch_cuda, dtype):
-    for seg in LDS_LENGTHS:
+    for seg in LDS_LENGTHS + [2047, 2048, 2049]:
         for rows in (1, 3):
             x = make_input(dtype, (rows, seg), seed=seg * 7 + rows)
             check_rows(lib, torch_cuda, x, f"{np.dtype(dtype)} rows={rows} seg={seg}")
@@ -171,21 +173,21 @@ def test_lds_many_short_rows(lib, torch_cuda):
 GLOBAL_LENGTHS = [1, 2, 100, 4097, 8191, 8192, 8193, 16383, 16384, 16385, 3 * 16384 + 5, 100003]
 
 
-@pytest.mark.parametrize("dtype", ALL_REAL_DTYPES)
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
 def test_global_path_all_dtypes(lib, torch_cuda, global_path, dtype):
     for seg in GLOBAL_LENGTHS:
         x = make_input(dtype, (seg,), seed=seg)
         check_rows(lib, torch_cuda, x, f"{np.dtype(dtype)} seg={seg} (global)")
 
 
-@pytest.mark.parametrize("dtype", [np.int32, np.float32, np.float64, np.uint8, np.float16])
+@pytest.mark.parametrize("dtype", [np.int32, np.float32, np.float64, np.uint8, np.float16, np.complex64, np.complex128])
 def test_global_path_batched_rows(lib, torch_cuda, global_path, dtype):
     # rows shorter than, equal to and longer than a tile; the look-back must stop at row starts
     for shape in [(50, 129), (7, 4096), (5, 8192), (3, 8193), (5, 16384), (3, 16385), (4, 40011), (300, 1)]:
         check_rows(lib, torch_cuda, make_input(dtype, shape, seed=shape[0]), f"{np.dtype(dtype)} {shape} (global)")
 
 
-@pytest.mark.parametrize("dtype", [np.int32, np.float32, np.int64, np.float64, np.float16, np.uint8])
+@pytest.mark.parametrize("dtype", [np.int32, np.float32, np.int64, np.float64, np.float16, np.uint8, np.complex64, np.complex128])
 def test_global_path_default_dispatch(lib, torch_cuda, dtype):
     # long rows take the global path without any override
     for shape in [(1 << 20,), (3, 70001), (2, 8193), (2, 16385)]:
@@ -193,7 +195,7 @@ def test_global_path_default_dispatch(lib, torch_cuda, dtype):
 
 
 @pytest.mark.parametrize("path", ["lds", "global"])
-@pytest.mark.parametrize("dtype", [np.uint8, np.int16, np.float32, np.int64])
+@pytest.mark.parametrize("dtype", [np.uint8, np.int16, np.float32, np.int64, np.complex64, np.complex128])
 def test_outputs_in_place_and_offset(lib, torch_cuda, path, dtype):
     prev = lib.cpn_set_lds_row_limit(0 if path == "global" else -1)
     try:
@@ -230,6 +232,10 @@ def test_skewed_and_degenerate_keys(lib, torch_cuda, path):
             "all NaN": np.full(n, np.nan, dtype=np.float32),
             "NaN and zeros": rng.choice(np.array([np.nan, 0.0, -0.0], dtype=np.float64), n),
             "bool": rng.integers(0, 2, n).astype(np.bool_),
+            "complex real-only": rng.standard_normal(n).astype(np.complex64),
+            "complex NaN classes": rng.choice(
+                np.array([complex(np.nan, 1), complex(1, np.nan), complex(np.nan, np.nan), 1 + 1j, complex(1, -0.0)],
+                         dtype=np.complex128), n),
         }
         for name, x in cases.items():
             _, want_i = check_rows(lib, torch_cuda, x, f"{name} ({path})")
@@ -267,7 +273,7 @@ def test_swapaxes_copy(lib, torch_cuda, elem):
         assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (shape, a, b)
 
 
-@pytest.mark.parametrize("dtype", [np.int32, np.float16, np.float64, np.uint8])
+@pytest.mark.parametrize("dtype", [np.int32, np.float16, np.float64, np.uint8, np.complex64, np.complex128])
 def test_sort_along_other_axes(dtype):
     for shape in [(100, 70), (5, 6, 7), (65, 130), (2, 3, 4, 5), (1000, 3), (3, 9000)]:
         x = make_input(dtype, shape, seed=len(shape))
@@ -277,6 +283,15 @@ def test_sort_along_other_axes(dtype):
             assert_same_bits(np.asarray(num.argsort(a, axis=axis)), oracle.argsort(x, axis=axis), f"{shape} axis={axis}")
 
 
-def test_unsupported_complex_is_reported():
-    with pytest.raises(NotImplementedError):
-        num.sort(np.array([1 + 2j, 0.5 - 1j], dtype=np.complex64))
+def test_complex_integration_cases():
+    # tests/integration/test_sort.py:146-183: complex64 / complex128 inputs against NumPy
+    rng = np.random.default_rng(8)
+    for dtype in COMPLEX_DTYPES:
+        for size in [(5,), (5, 5), (3, 4, 5), (1, 0, 1)]:
+            arr_np = (rng.integers(-10, 10, size) + 1j * rng.integers(-10, 10, size)).astype(dtype)
+            arr_num = num.array(arr_np)
+            for axis in range(-arr_np.ndim + 1, arr_np.ndim):
+                assert np.array_equal(num.sort(arr_num, axis=axis), np.sort(arr_np, axis=axis, kind="stable"))
+                assert np.array_equal(
+                    num.argsort(arr_num, axis=axis, kind="stable"), np.argsort(arr_np, axis=axis, kind="stable")
+                )
