@@ -18,7 +18,10 @@ from . import random  # noqa: F401
 from ._array import convert_to_ndarray, ndarray
 from ._thunk import SUPPORTED_DTYPES, DeviceArray, check_dtype
 
-__all__ = ["ndarray", "array", "asarray", "sort", "argsort", "random", "SUPPORTED_DTYPES"]
+__all__ = [
+    "ndarray", "array", "asarray", "sort", "argsort", "sort_complex", "partition", "argpartition", "random",
+    "SUPPORTED_DTYPES",
+]
 
 __version__ = "0.1.0"
 
@@ -62,4 +65,38 @@ def sort(a: Any, axis: int | None = -1, kind: str = "quicksort", order: Any = No
     else:
         result = ndarray(a.shape, a.dtype)
     result._thunk.sort(rhs=a._thunk, axis=axis, kind=kind, order=order)
+    return result
+
+
+def sort_complex(a: Any) -> ndarray:
+    """Sorted copy along the last axis, always complex (`cupynumeric/_module/ssc_sorting.py:124-159`):
+    complex input keeps its type, integers of at most 16 bits give complex64, everything else
+    complex128."""
+    result = sort(a)
+    # force complex result upon return
+    if np.issubdtype(result.dtype, np.complexfloating):
+        return result
+    elif np.issubdtype(result.dtype, np.integer) and result.dtype.itemsize <= 2:
+        return result.astype_complex(np.complex64)
+    else:
+        return result.astype_complex(np.complex128)
+
+
+def argpartition(a: Any, kth: Any, axis: int | None = -1, kind: str = "introselect", order: Any = None) -> ndarray:
+    """Indirect partition (`cupynumeric/_module/ssc_sorting.py:165-218`); falls back to argsort."""
+    a = convert_to_ndarray(a)
+    result = ndarray(a.shape, np.int64)
+    result._thunk.partition(rhs=a._thunk, argpartition=True, kth=kth, axis=axis, kind=kind, order=order)
+    if axis is None and a.ndim > 1:
+        result._thunk.shape = (a.size,)
+    return result
+
+
+def partition(a: Any, kth: Any, axis: int | None = -1, kind: str = "introselect", order: Any = None) -> ndarray:
+    """Partitioned copy (`cupynumeric/_module/ssc_sorting.py:221-268`); falls back to sort."""
+    a = convert_to_ndarray(a)
+    result = ndarray(a.shape, a.dtype)
+    result._thunk.partition(rhs=a._thunk, kth=kth, axis=axis, kind=kind, order=order)
+    if axis is None and a.ndim > 1:
+        result._thunk.shape = (a.size,)
     return result

@@ -94,6 +94,28 @@ class ndarray:
         return result
 
 
+    def partition(self, kth: Any, axis: Any = -1, kind: str = "introselect", order: Any = None) -> None:
+        """a.partition(kth, axis=-1, kind='introselect', order=None): in place
+        (`cupynumeric/_array/array.py:3441-3467`)."""
+        if not self._writeable:
+            raise ValueError("array is not writeable")
+        self._thunk.partition(rhs=self._thunk, kth=kth, axis=axis, kind=kind, order=order)
+        _adopt_shape(self, self, axis)
+
+    def argpartition(self, kth: Any, axis: Any = -1, kind: str = "introselect", order: Any = None) -> "ndarray":
+        """a.argpartition(kth, axis=-1, kind='introselect', order=None)
+        (`cupynumeric/_array/array.py:3469-3501`)."""
+        result = ndarray(self.shape, np.int64)
+        result._thunk.partition(rhs=self._thunk, argpartition=True, kth=kth, axis=axis, kind=kind, order=order)
+        _adopt_shape(result, self, axis)
+        return result
+
+    def astype_complex(self, dtype: Any) -> "ndarray":
+        """Real -> complex64/complex128 copy (the cast `sort_complex` needs)."""
+        thunk = self._thunk.to_complex(dtype)
+        return ndarray(thunk.shape, thunk.dtype, thunk=thunk)
+
+
 def _adopt_shape(result: ndarray, source: ndarray, axis: Any) -> None:
     """Results of `axis=None` sorts are flat; nothing else changes shape."""
     if axis is None and source.ndim > 1:

@@ -148,3 +148,45 @@ class DeviceArray:
             raise ValueError("invalid axis")
 
         sort_deferred(self, rhs, argsort, axis, stable)
+
+    def partition(
+        self,
+        rhs: "DeviceArray",
+        kth: Any,
+        argpartition: bool = False,
+        axis: int | None = -1,
+        kind: str = "introselect",
+        order: str | list[str] | None = None,
+    ) -> None:
+        """`DeferredArray.partition` (`cupynumeric/_thunk/deferred.py:5476-5494`): falls back to an
+        (unstable-flagged) sort, which satisfies the partition property for every `kth`."""
+        from ._sort import sort_deferred
+
+        if order is not None:
+            raise NotImplementedError(
+                "cuPyNumeric does not support partitioning with 'order' as "
+                "ndarray only supports numeric values"
+            )
+        if axis is not None and (axis >= rhs.ndim or axis < -rhs.ndim):
+            raise ValueError("invalid axis")
+
+        # fallback to sort for now
+        sort_deferred(self, rhs, argpartition, axis, False)
+
+    def to_complex(self, dtype: Any) -> "DeviceArray":
+        """Real -> complex cast (`astype` in `sort_complex`, `cupynumeric/_module/ssc_sorting.py:150-159`)."""
+        dt = check_dtype(dtype)
+        out = DeviceArray(self.shape, dt)
+        if self.size == 0:
+            return out
+        lib = _lib.load()
+        status = lib.cpn_real_to_complex(
+            _lib.DTYPE_CODES[self.dtype],
+            self.base.ptr(),
+            _lib.DTYPE_CODES[dt],
+            out.base.ptr(),
+            self.size,
+            runtime.stream_handle(),
+        )
+        _lib.check(status, "cpn_real_to_complex")
+        return out

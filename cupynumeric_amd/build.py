@@ -24,6 +24,7 @@ SOURCES = [
     "sort_api.hip",
     "swapaxes.hip",
     "profile.hip",
+    "convert.hip",
     "sort_keys8.hip",
     "sort_keys16.hip",
     "sort_keys32.hip",

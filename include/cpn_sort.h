@@ -147,6 +147,14 @@ int cpn_swapaxes_copy(int elem_bytes, const void* in, void* out, const int64_t* 
                       int axis_a, int axis_b, void* stream);
 
 /*
+ * out[i] = complex(in[i], 0): `in` holds `volume` elements of the real type `src_dtype`, `out`
+ * receives complex64 or complex128 (`dst_dtype`).  The cast sort_complex applies to real
+ * results (cupynumeric/_module/ssc_sorting.py:150-159: `result.astype(np.complex64 / complex128)`).
+ */
+int cpn_real_to_complex(int src_dtype, const void* in, int dst_dtype, void* out, uint64_t volume,
+                        void* stream);
+
+/*
  * Per-launch timing.  cpn_profile_enable(1) makes every kernel launch of the library record
  * a pair of HIP events on the stream it is launched on; it returns the previous setting.
  * cpn_profile_collect waits for the recorded events, writes up to `max_records` entries --
