@@ -151,7 +151,8 @@ class GpuJob:
         )
         self.temp = torch.empty(self.temp_bytes, dtype=torch.uint8, device=dev)
         self.stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-        self.uses_lds_rows = self.temp_bytes == 256
+        # rows that fit the per-row LDS kernel need nothing but the workspace header
+        self.uses_lds_rows = self.temp_bytes == self.lib.cpn_local_sort_temp_bytes(self.code, 0, 0, 1, 0, 0)
 
     def step(self) -> None:
         lib, ck = self.lib, self._lib_mod.check

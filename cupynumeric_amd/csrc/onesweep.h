@@ -179,9 +179,14 @@ __global__ __launch_bounds__(HIST_BLOCK) void histogram_kernel(const KeyT* __res
   }
 }
 
-// One block per (row, pass): exclusive scan of 256 counts in place.
+// One block per (row, pass): exclusive scan of 256 counts in place.  A pass on whose digit
+// all keys of a row agree (one bin holds the whole row) would be the identity permutation for
+// that row; `varying[pass]` is raised by every row for which that is not so.
 template <typename OffT>
-__global__ __launch_bounds__(RADIX) void histogram_scan_kernel(OffT* __restrict__ hist)
+__global__ __launch_bounds__(RADIX) void histogram_scan_kernel(OffT* __restrict__ hist,
+                                                               uint32_t* __restrict__ varying,
+                                                               uint64_t seg,
+                                                               uint32_t passes)
 {
   __shared__ OffT s_wsum[RADIX / WAVE];
   const int tid  = threadIdx.x;
@@ -189,6 +194,10 @@ __global__ __launch_bounds__(RADIX) void histogram_scan_kernel(OffT* __restrict_
   const int wave = tid / WAVE;
   OffT* h        = hist + static_cast<uint64_t>(blockIdx.x) * RADIX;
   const OffT c   = h[tid];
+  const int one_bin = __syncthreads_or(c == static_cast<OffT>(seg));
+  if (!one_bin && tid == 0) {
+    __hip_atomic_fetch_or(&varying[blockIdx.x % passes], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
   OffT incl      = c;
 #pragma unroll
   for (int delta = 1; delta < WAVE; delta <<= 1) {
@@ -209,15 +218,125 @@ __global__ __launch_bounds__(RADIX) void histogram_scan_kernel(OffT* __restrict_
 }
 
 // ---------------------------------------------------------------------------------------
+// pass plan: which passes run and between which buffers, decided on the device
+// ---------------------------------------------------------------------------------------
+// Passes whose digit is the same for all keys of every row are skipped.  Which buffer a pass
+// reads and writes then depends on how many passes remain, which only the device knows after
+// the histogram sweep: a one-thread kernel writes one PassPlan per pass and the scatter
+// kernels look their buffers up by id.  The last running pass always writes the caller's
+// arrays; the ones before it alternate, walking backwards, between two scratch buffers.
+constexpr int MAX_PASSES = 24;
+enum KeyBuf : uint32_t { KEY_IN = 0, KEY_OUT = 1, KEY_T1 = 2, KEY_T2 = 3 };
+enum IdxBuf : uint32_t { IDX_FINAL = 1, IDX_T1 = 2, IDX_ALIAS = 3 };  // ALIAS: the int64 output used as narrow scratch
+constexpr uint32_t BUF_NONE = 0xFFu;
+
+struct PassPlan {
+  uint32_t active;   // 0: the pass exits at once
+  uint32_t key_src;  // KeyBuf
+  uint32_t key_dst;  // KeyBuf or BUF_NONE (index-only sort, last pass)
+  uint32_t idx_src;  // IdxBuf or BUF_NONE (first running pass: positions are synthesised)
+  uint32_t idx_dst;  // IdxBuf
+  uint32_t first;    // first running pass
+};
+
+struct SortPlan {
+  PassPlan pass[MAX_PASSES];
+  uint32_t n_active;
+};
+
+struct PlanRequest {
+  uint32_t passes;
+  uint32_t want_values;
+  uint32_t want_indices;
+  uint32_t in_place;
+};
+
+static __global__ void plan_kernel(const uint32_t* __restrict__ varying, SortPlan* __restrict__ plan, PlanRequest rq)
+{
+  if (threadIdx.x != 0 || blockIdx.x != 0) {
+    return;
+  }
+  uint32_t k = 0;
+  for (uint32_t p = 0; p < rq.passes; ++p) {
+    k += (varying[p] != 0) ? 1u : 0u;
+  }
+  plan->n_active = k;
+  // scratch partner of T1: the caller's value array when it is free to be overwritten early
+  const uint32_t key_x = (rq.want_values && !rq.in_place) ? KEY_OUT : KEY_T2;
+  uint32_t j = 0, key_prev = KEY_IN, idx_prev = BUF_NONE;
+  for (uint32_t p = 0; p < rq.passes; ++p) {
+    PassPlan e{};
+    if (varying[p] != 0) {
+      ++j;
+      const uint32_t from_last = k - j;
+      e.active                 = 1;
+      e.first                  = (j == 1) ? 1u : 0u;
+      e.key_src                = key_prev;
+      e.idx_src                = idx_prev;
+      if (from_last == 0) {
+        e.key_dst = rq.want_values ? ((k == 1 && rq.in_place) ? KEY_T1 : KEY_OUT) : BUF_NONE;
+        e.idx_dst = IDX_FINAL;
+      } else {
+        e.key_dst = (from_last & 1u) ? KEY_T1 : key_x;
+        e.idx_dst = (from_last & 1u) ? IDX_T1 : IDX_ALIAS;
+      }
+      key_prev = e.key_dst;
+      idx_prev = e.idx_dst;
+    }
+    plan->pass[p] = e;
+  }
+}
+
+// What the scatter passes leave undone: nothing ran (all keys of every row are equal: the
+// output is the input, the indices are 0..seg-1), or a single pass sorted in place into
+// scratch buffer 1 and its result still has to reach the caller's array.
+template <typename KeyT>
+__global__ __launch_bounds__(256) void finalize_kernel(const SortPlan* __restrict__ plan,
+                                                        const KeyT* in,
+                                                        KeyT* out,
+                                                        const KeyT* __restrict__ t1,
+                                                        int64_t* __restrict__ idx_out,
+                                                        uint64_t volume,
+                                                        uint64_t seg,
+                                                        int64_t index_offset,
+                                                        PlanRequest rq)
+{
+  const uint32_t k      = plan->n_active;
+  const uint64_t stride = static_cast<uint64_t>(gridDim.x) * blockDim.x;
+  const uint64_t first  = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (k == 0) {
+    if (rq.want_values && !rq.in_place) {
+      for (uint64_t i = first; i < volume; i += stride) {
+        out[i] = in[i];
+      }
+    }
+    if (rq.want_indices) {
+      for (uint64_t i = first; i < volume; i += stride) {
+        idx_out[i] = static_cast<int64_t>(i % seg) + index_offset;
+      }
+    }
+  } else if (k == 1 && rq.want_values && rq.in_place) {
+    for (uint64_t i = first; i < volume; i += stride) {
+      out[i] = t1[i];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // onesweep scatter pass
 // ---------------------------------------------------------------------------------------
 template <bool BIG>
 struct SweepArgs {
   using OffT = typename RowWidth<BIG>::off_t;
+  const void* key_buf[4];  // indexed by KeyBuf
+  void* idx_buf[4];        // indexed by IdxBuf
+  const SortPlan* plan;
+  // resolved from the plan by the kernel before the tile is worked on:
   const void* keys_in;     // KeyT[volume]
   void* keys_out;          // KeyT[volume] or nullptr (last pass of an index-only sort)
   const OffT* idx_in;      // row positions from the previous pass, nullptr = synthesise
   void* idx_out;           // OffT[volume], or int64[volume] when idx_final
+  int first;               // first running pass (ordered-key mode transforms the keys there)
   uint32_t* ticket;        // tile ticket counter of this pass (zeroed)
   const OffT* hist_excl;   // this pass's scanned histogram of row 0; row stride = hist_row_stride
   OffT* desc;              // [num_tiles][256] descriptors of this pass (zeroed)
@@ -249,10 +368,10 @@ struct SweepShared {
 // folds away and the body is straight-line code, which lets the compiler batch the LDS and
 // HBM accesses of a phase instead of waiting on each one.
 //
-// XFORM (index-only sorts): the keys are replaced by their order-preserving unsigned image
-// as soon as they are loaded and are written out that way, so that the later passes, which
-// then run with the identity codec, do not pay for the key transform again.  The values
-// themselves are never returned in that case.
+// XFORM (index-only sorts): the first running pass replaces the keys by their order-preserving
+// unsigned image as soon as they are loaded and writes them out that way; every pass extracts
+// digits with the identity codec, so the key transform is paid once per key instead of twice
+// per pass.  The values themselves are never returned in that case.
 template <typename KeyT, int CODEC, bool XFORM, bool BIG, bool HAS_IDX, int BLOCK, int ITEMS, bool FULL>
 __device__ __forceinline__ void onesweep_tile(
   const SweepArgs<BIG>& a,
@@ -288,8 +407,13 @@ __device__ __forceinline__ void onesweep_tile(
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t o = woff + i * WAVE;
     key[i]           = (FULL || o < count) ? kin[o] : KeyT{};
-    if constexpr (XFORM) {
-      key[i] = ordered_bits<CODEC, KeyT>(key[i]);
+  }
+  if constexpr (XFORM) {
+    if (a.first) {  // one uniform branch around all items, so that the loads above stay batched
+#pragma unroll
+      for (int i = 0; i < ITEMS; ++i) {
+        key[i] = ordered_bits<CODEC, KeyT>(key[i]);
+      }
     }
   }
 
@@ -505,7 +629,7 @@ __device__ __forceinline__ void onesweep_tile(
 
 template <typename KeyT, int CODEC, bool XFORM, bool BIG, bool HAS_IDX, int BLOCK, int ITEMS>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(CPN_ONESWEEP_WAVES_PER_EU)))
-void onesweep_kernel(const SweepArgs<BIG> a)
+void onesweep_kernel(const SweepArgs<BIG> a_in)
 {
   using OffT = typename RowWidth<BIG>::off_t;
   static_assert(BLOCK >= RADIX, "one thread per digit is needed for the look-back");
@@ -516,6 +640,18 @@ void onesweep_kernel(const SweepArgs<BIG> a)
   static_assert(TILE <= 65536, "positions inside a tile are kept in 16 bits");
 
   __shared__ SweepShared<KeyT, OffT, WAVES, TILE, STAGE_ELEM> sh;
+
+  const PassPlan pp = a_in.plan->pass[a_in.pass];
+  if (pp.active == 0) {
+    return;  // every key of every row has the same digit here
+  }
+  SweepArgs<BIG> a = a_in;
+  a.keys_in        = a_in.key_buf[pp.key_src];
+  a.keys_out       = (pp.key_dst == BUF_NONE) ? nullptr : const_cast<void*>(a_in.key_buf[pp.key_dst]);
+  a.idx_in         = (pp.idx_src == BUF_NONE) ? nullptr : static_cast<const OffT*>(a_in.idx_buf[pp.idx_src]);
+  a.idx_out        = a_in.idx_buf[pp.idx_dst];
+  a.idx_final      = (pp.idx_dst == IDX_FINAL) ? 1 : 0;
+  a.first          = static_cast<int>(pp.first);
 
   const int tid = threadIdx.x;
   // Tiles are handed out in launch order of the workgroups that are actually running, so

@@ -29,8 +29,15 @@ extern thread_local int g_last_hip_error;
   } while (0)
 
 constexpr uint64_t WORKSPACE_ALIGN  = 256;
-constexpr uint64_t HEADER_BYTES     = 256;  // [0] status word, [64..] tile tickets (one per pass)
+// Workspace header: [0] status word, [64..) tile tickets, [192..) per-pass "digit varies" flags,
+// [320..) the device-side SortPlan.
+constexpr uint64_t HEADER_BYTES     = 1024;
 constexpr uint64_t HEADER_TICKETS   = 64;
+constexpr uint64_t HEADER_VARYING   = 192;
+constexpr uint64_t HEADER_PLAN      = 320;
+static_assert(HEADER_TICKETS + 4 * MAX_PASSES <= HEADER_VARYING, "tickets overlap the flags");
+static_assert(HEADER_VARYING + 4 * MAX_PASSES <= HEADER_PLAN, "flags overlap the plan");
+static_assert(HEADER_PLAN + sizeof(SortPlan) <= HEADER_BYTES, "plan does not fit the header");
 constexpr uint64_t BIG_ROW_ELEMENTS = 1ull << 30;
 
 __host__ __device__ constexpr uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
@@ -120,12 +127,14 @@ inline GlobalLayout global_layout(int key_bytes, int passes, uint64_t volume, ui
   L.key_bytes_total   = align_up(volume * key_bytes, WORKSPACE_ALIGN);
   L.off_key1 = L.off_key2 = 0;
   bool need_key1, need_key2;
+  // (see plan_kernel: intermediate passes alternate between buffer 1 and either the caller's
+  // value array, when it is not also the input, or buffer 2)
   if (L.passes == 1) {
     need_key1 = want_values && in_place;
     need_key2 = false;
   } else {
     need_key1 = true;
-    need_key2 = !want_values && L.passes >= 3;
+    need_key2 = (!want_values || in_place) && L.passes >= 3;
   }
   if (need_key1) {
     L.off_key1 = off;
@@ -237,7 +246,15 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
   }
   uint32_t* status  = reinterpret_cast<uint32_t*>(ws);
   uint32_t* tickets = reinterpret_cast<uint32_t*>(ws + HEADER_TICKETS);
+  uint32_t* varying = reinterpret_cast<uint32_t*>(ws + HEADER_VARYING);
+  SortPlan* plan    = reinterpret_cast<SortPlan*>(ws + HEADER_PLAN);
   OffT* hist        = reinterpret_cast<OffT*>(ws + L.off_hist);
+  static_assert(PASSES <= MAX_PASSES, "plan table too small");
+  PlanRequest rq{};
+  rq.passes       = PASSES;
+  rq.want_values  = want_vals ? 1u : 0u;
+  rq.want_indices = HAS_IDX ? 1u : 0u;
+  rq.in_place     = in_place ? 1u : 0u;
 
   // histogram sweep: about 2048 blocks in total, at least one per row
   {
@@ -267,68 +284,55 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
     {
       ProfileScope prof("histogram_scan", r.stream);
       hipLaunchKernelGGL((histogram_scan_kernel<OffT>), dim3(static_cast<uint32_t>(L.rows * PASSES)),
-                         dim3(RADIX), 0, r.stream, hist);
+                         dim3(RADIX), 0, r.stream, hist, varying, r.seg, static_cast<uint32_t>(PASSES));
+    }
+    CPN_HIP_TRY(hipGetLastError());
+    {
+      ProfileScope prof("plan", r.stream);
+      hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(WAVE), 0, r.stream, varying, plan, rq);
     }
     CPN_HIP_TRY(hipGetLastError());
   }
 
-  // key buffers: the last pass writes the caller's array (or nothing), earlier passes
-  // alternate, walking backwards, between workspace buffer 1 and X = values_out or buffer 2
+  // The buffers a pass may read or write; which ones it uses is in the device-side plan.
   void* key1 = L.off_key1 ? ws + L.off_key1 : nullptr;
   void* key2 = L.off_key2 ? ws + L.off_key2 : nullptr;
-  void* keyX = want_vals ? r.values_out : key2;
   void* idx1 = L.off_idx ? ws + L.off_idx : nullptr;
-  void* idxX = r.indices_out;  // the int64 output doubles as a narrow scratch array
 
-  // Index-only sorts never return the keys: the first pass stores their order-preserving
-  // unsigned image in the workspace and the later passes run with the identity codec.
+  // Index-only sorts never return the keys: the first running pass stores their
+  // order-preserving unsigned image and every pass extracts digits with the identity codec.
   constexpr bool CAN_ORDER_KEYS = HAS_IDX && (CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT) && PASSES >= 2;
   const bool ordered_keys       = CAN_ORDER_KEYS && !want_vals;
 
-  const void* key_src = r.values_in;
-  const void* idx_src = nullptr;
   for (int p = 0; p < PASSES; ++p) {
-    const bool last      = (p == PASSES - 1);
-    const int from_last  = PASSES - 1 - p;
-    void* key_dst;
-    void* idx_dst = nullptr;
-    if (last) {
-      key_dst = (PASSES == 1 && want_vals && in_place) ? key1 : r.values_out;
-    } else {
-      key_dst = (from_last & 1) ? key1 : keyX;
-    }
-    if constexpr (HAS_IDX) {
-      idx_dst = last ? static_cast<void*>(r.indices_out) : ((from_last & 1) ? idx1 : idxX);
-    }
     SweepArgs<BIG> a{};
-    a.keys_in         = key_src;
-    a.keys_out        = key_dst;
-    a.idx_in          = static_cast<const OffT*>(idx_src);
-    a.idx_out         = idx_dst;
-    a.ticket          = tickets + p;
-    a.hist_excl       = hist + p * RADIX;
-    a.desc            = reinterpret_cast<OffT*>(ws + L.off_desc + L.desc_bytes_per_pass * p);
-    a.status          = status;
-    a.seg             = r.seg;
-    a.hist_row_stride = static_cast<uint64_t>(PASSES) * RADIX;
-    a.index_offset    = r.index_offset;
-    a.tiles_per_row   = L.tiles_per_row;
-    a.num_tiles       = static_cast<uint32_t>(L.num_tiles);
-    a.pass            = p;
-    a.idx_final       = last ? 1 : 0;
+    a.key_buf[KEY_IN]    = r.values_in;
+    a.key_buf[KEY_OUT]   = r.values_out;
+    a.key_buf[KEY_T1]    = key1;
+    a.key_buf[KEY_T2]    = key2;
+    a.idx_buf[0]         = nullptr;
+    a.idx_buf[IDX_FINAL] = r.indices_out;
+    a.idx_buf[IDX_T1]    = idx1;
+    a.idx_buf[IDX_ALIAS] = r.indices_out;
+    a.plan               = plan;
+    a.ticket             = tickets + p;
+    a.hist_excl          = hist + p * RADIX;
+    a.desc               = reinterpret_cast<OffT*>(ws + L.off_desc + L.desc_bytes_per_pass * p);
+    a.status             = status;
+    a.seg                = r.seg;
+    a.hist_row_stride    = static_cast<uint64_t>(PASSES) * RADIX;
+    a.index_offset       = r.index_offset;
+    a.tiles_per_row      = L.tiles_per_row;
+    a.num_tiles          = static_cast<uint32_t>(L.num_tiles);
+    a.pass               = p;
     {
       ProfileScope prof("onesweep", r.stream);
       const dim3 grid(static_cast<uint32_t>(L.num_tiles));
       bool launched = false;
       if constexpr (CAN_ORDER_KEYS) {
         if (ordered_keys) {
-          if (p == 0) {
-            hipLaunchKernelGGL((onesweep_kernel<KeyT, CODEC, true, BIG, HAS_IDX, BLOCK, ITEMS>), grid, dim3(BLOCK), 0,
-                               r.stream, a);
-          } else {
-            hipLaunchKernelGGL((onesweep_kernel<KeyT, CODEC_UNSIGNED, false, BIG, HAS_IDX, BLOCK, ITEMS>), grid,
-                               dim3(BLOCK), 0, r.stream, a);
-          }
+          hipLaunchKernelGGL((onesweep_kernel<KeyT, CODEC, true, BIG, HAS_IDX, BLOCK, ITEMS>), grid, dim3(BLOCK), 0,
+                             r.stream, a);
           launched = true;
         }
       }
@@ -338,12 +342,18 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
       }
     }
     CPN_HIP_TRY(hipGetLastError());
-    key_src = key_dst;
-    idx_src = idx_dst;
   }
-  if (PASSES == 1 && want_vals && in_place) {
-    CPN_HIP_TRY(hipMemcpyAsync(r.values_out, key1, r.volume * KB, hipMemcpyDeviceToDevice, r.stream));
+  {
+    uint64_t blocks = (r.volume + 1023) / 1024;
+    if (blocks > 8192) {
+      blocks = 8192;
+    }
+    ProfileScope prof("finalize", r.stream);
+    hipLaunchKernelGGL((finalize_kernel<KeyT>), dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, r.stream, plan,
+                       static_cast<const KeyT*>(r.values_in), static_cast<KeyT*>(r.values_out),
+                       static_cast<const KeyT*>(key1), r.indices_out, r.volume, r.seg, r.index_offset, rq);
   }
+  CPN_HIP_TRY(hipGetLastError());
   return CPN_OK;
 }
 

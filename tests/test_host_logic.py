@@ -54,18 +54,18 @@ def test_version_status_strings_and_sizes(lib):
 def test_argument_validation_without_a_device(lib):
     # every check below fails before the first HIP call
     sort = lib.cpn_local_sort
-    assert sort(99, 16, 16, None, 4, 4, 0, 1, 256, 256, None) == _lib.CPN_ERR_DTYPE
+    assert sort(99, 16, 16, None, 4, 4, 0, 1, 256, 1024, None) == _lib.CPN_ERR_DTYPE
     assert sort(3, None, None, None, 0, 0, 0, 1, None, 0, None) == _lib.CPN_OK  # volume 0: no-op
-    assert sort(3, 16, 32, None, 10, 3, 0, 1, 256, 256, None) == _lib.CPN_ERR_SHAPE  # 3 does not divide 10
-    assert sort(3, 16, 32, None, 10, 0, 0, 1, 256, 256, None) == _lib.CPN_ERR_SHAPE
-    assert sort(3, None, 32, None, 4, 4, 0, 1, 256, 256, None) == _lib.CPN_ERR_NULL
-    assert sort(3, 16, None, None, 4, 4, 0, 1, 256, 256, None) == _lib.CPN_ERR_NULL  # no output at all
-    assert sort(3, 18, 32, None, 4, 4, 0, 1, 256, 256, None) == _lib.CPN_ERR_ALIGN
-    assert sort(3, 16, None, 36, 4, 4, 0, 1, 256, 256, None) == _lib.CPN_ERR_ALIGN  # int64 out misaligned
+    assert sort(3, 16, 32, None, 10, 3, 0, 1, 256, 1024, None) == _lib.CPN_ERR_SHAPE  # 3 does not divide 10
+    assert sort(3, 16, 32, None, 10, 0, 0, 1, 256, 1024, None) == _lib.CPN_ERR_SHAPE
+    assert sort(3, None, 32, None, 4, 4, 0, 1, 256, 1024, None) == _lib.CPN_ERR_NULL
+    assert sort(3, 16, None, None, 4, 4, 0, 1, 256, 1024, None) == _lib.CPN_ERR_NULL  # no output at all
+    assert sort(3, 18, 32, None, 4, 4, 0, 1, 256, 1024, None) == _lib.CPN_ERR_ALIGN
+    assert sort(3, 16, None, 36, 4, 4, 0, 1, 256, 1024, None) == _lib.CPN_ERR_ALIGN  # int64 out misaligned
     assert sort(3, 16, 32, None, 4, 4, 0, 1, None, 0, None) == _lib.CPN_ERR_TEMP
     assert sort(3, 16, 32, None, 4, 4, 0, 1, 256, 16, None) == _lib.CPN_ERR_TEMP  # too small
     assert sort(3, 16, 32, None, 4, 4, 0, 1, 264, 4096, None) == _lib.CPN_ERR_TEMP  # misaligned
-    assert sort(13, 24, 32, None, 4, 4, 0, 1, 256, 256, None) == _lib.CPN_ERR_ALIGN  # complex128 needs 16-byte alignment
+    assert sort(13, 24, 32, None, 4, 4, 0, 1, 256, 1024, None) == _lib.CPN_ERR_ALIGN  # complex128 needs 16-byte alignment
     assert lib.cpn_local_sort_check(None, None) == _lib.CPN_ERR_NULL
     swap = lib.cpn_swapaxes_copy
     import ctypes
@@ -80,21 +80,25 @@ def test_argument_validation_without_a_device(lib):
 
 
 def test_temp_bytes_layout(lib):
+    def align256(v):
+        return (v + 255) // 256 * 256
+
     tb = lib.cpn_local_sort_temp_bytes
     f32, i64, u8, f16 = 10, 4, 5, 9
     assert tb(99, 100, 100, 1, 0, 0) == 0
     assert tb(f32, 100, 7, 1, 0, 0) == 0  # 7 does not divide 100
-    assert tb(f32, 0, 0, 1, 0, 0) == 256
-    assert tb(f32, 1 << 20, 1024, 1, 1, 0) == 256  # rows that fit LDS need only the status header
+    header = tb(f32, 0, 0, 1, 0, 0)
+    assert header == 1024
+    assert tb(f32, 1 << 20, 1024, 1, 1, 0) == header  # rows that fit LDS need only the header
     n = 1 << 24
     tiles = n // 16384  # 512 threads x 32 keys per tile for keys of up to 4 bytes
-    fixed = 256 + 4 * 256 * 4 + 4 * tiles * 256 * 4
+    fixed = header + 4 * 256 * 4 + 4 * tiles * 256 * 4
     assert tb(f32, n, n, 1, 0, 0) == fixed + 4 * n  # one key buffer
-    assert tb(f32, n, n, 1, 0, 1) == fixed + 4 * n  # in place, even pass count: same
+    assert tb(f32, n, n, 1, 0, 1) == fixed + 2 * 4 * n  # in place: a second buffer, in case an odd number of passes runs
     assert tb(f32, n, n, 0, 1, 0) == fixed + 2 * 4 * n + 4 * n  # index-only: two key buffers + narrow indices
     assert tb(f32, n, n, 1, 1, 0) == fixed + 4 * n + 4 * n
     # 8-bit keys take one pass: no key buffer unless sorting in place
-    t8 = 256 + 256 * 4 + tiles * 256 * 4
+    t8 = header + 256 * 4 + tiles * 256 * 4
     assert tb(u8, n, n, 1, 0, 0) == t8
     assert tb(u8, n, n, 1, 0, 1) == t8 + n
     assert tb(u8, n, n, 0, 1, 0) == t8
@@ -102,15 +106,15 @@ def test_temp_bytes_layout(lib):
     assert tb(i64, n, n, 0, 1, 0) > tb(f32, n, n, 0, 1, 0) > tb(f16, n, n, 0, 1, 0)
     # complex keys take one more pass (the NaN class) than their bytes
     c64, c128 = 12, 13
-    assert tb(c64, n, n, 1, 0, 0) == 256 + 9 * 256 * 4 + 9 * (n // 8192) * 256 * 4 + 8 * n
-    assert tb(c128, n, n, 1, 0, 0) == 256 + 17 * 256 * 4 + 17 * (n // 4096) * 256 * 4 + 16 * n
+    assert tb(c64, n, n, 1, 0, 0) == header + 9 * 256 * 4 + 9 * (n // 8192) * 256 * 4 + 8 * n
+    assert tb(c128, n, n, 1, 0, 0) == header + align256(17 * 256 * 4) + 17 * (n // 4096) * 256 * 4 + 16 * n
     # the row-length switch moves work to the global path
     prev = lib.cpn_set_lds_row_limit(0)
     try:
-        assert tb(f32, 1 << 20, 1024, 1, 1, 0) > 256
+        assert tb(f32, 1 << 20, 1024, 1, 1, 0) > header
     finally:
         lib.cpn_set_lds_row_limit(prev)
-    assert tb(f32, 1 << 20, 1024, 1, 1, 0) == 256
+    assert tb(f32, 1 << 20, 1024, 1, 1, 0) == header
 
 
 @pytest.mark.parametrize("dtype", ALL_REAL_DTYPES)

@@ -50,7 +50,7 @@ def abi_sort(lib, torch, x: np.ndarray, want_values=True, want_indices=False, in
     d_val = d_in if in_place else (torch.zeros_like(d_in) if want_values else None)
     d_idx = torch.full((volume,), -7, dtype=torch.int64, device=dev) if want_indices else None
     tb = lib.cpn_local_sort_temp_bytes(code, volume, seg, int(want_values), int(want_indices), int(in_place))
-    assert tb >= 256
+    assert tb >= 1024
     temp = torch.empty(tb, dtype=torch.uint8, device=dev)
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     rc = lib.cpn_local_sort(
@@ -250,6 +250,48 @@ def test_skewed_and_degenerate_keys(lib, torch_cuda, path):
         assert np.array_equal(i, inv)  # argsort of a permutation is its inverse
     finally:
         lib.cpn_set_lds_row_limit(prev)
+
+
+# ---- passes on which all keys agree are skipped; the buffers used then depend on how many remain ----
+@pytest.mark.parametrize("dtype,nbytes", [(np.uint32, 4), (np.int64, 8), (np.float32, 4), (np.uint16, 2)])
+def test_global_path_skipped_passes(lib, torch_cuda, global_path, dtype, nbytes):
+    rng = np.random.default_rng(21)
+    n = 40000
+    ub = {2: np.uint16, 4: np.uint32, 8: np.uint64}[nbytes]
+    subsets = range(1 << nbytes) if nbytes <= 4 else [0, 1, 0x80, 0x11, 0x07, 0x70, 0xFE, 0x55, 0xFF]
+    for mask in subsets:
+        bits_ = np.zeros(n, dtype=ub)
+        const = ub(int(rng.integers(0, 1 << 62)) & ((1 << (8 * nbytes)) - 1))
+        for b in range(nbytes):
+            byte = rng.integers(0, 256, n).astype(ub) if (mask >> b) & 1 else np.full(n, (const >> ub(8 * b)) & ub(0xFF), dtype=ub)
+            bits_ |= byte << ub(8 * b)
+        x = bits_.view(dtype)
+        if np.dtype(dtype).kind == "f":
+            x = np.where(np.isnan(x), np.float32(1.5), x).astype(dtype)
+        want_v = oracle.local_sort(x, argsort=False)
+        want_i = oracle.local_sort(x, argsort=True)
+        what = f"{np.dtype(dtype)} varying-bytes mask {mask:#x}"
+        v, _ = abi_sort(lib, torch_cuda, x, want_values=True)
+        assert_same_bits(v, want_v, what + " sort")
+        _, i = abi_sort(lib, torch_cuda, x, want_values=False, want_indices=True, offset=3)
+        assert_same_bits(i, want_i + 3, what + " argsort")
+        v, _ = abi_sort(lib, torch_cuda, x, want_values=True, in_place=True)
+        assert_same_bits(v, want_v, what + " in place")
+        v, i = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=True, in_place=True)
+        assert_same_bits(v, want_v, what + " in place + indices")
+        assert_same_bits(i, want_i, what + " in place + indices")
+
+
+def test_global_path_skipping_needs_every_row(lib, torch_cuda, global_path):
+    # a byte that is constant inside each row but differs between rows may be skipped; a byte
+    # that varies in one row only may not
+    rng = np.random.default_rng(22)
+    rows, seg = 6, 20000
+    x = rng.integers(0, 256, (rows, seg)).astype(np.uint32)  # byte 0 varies everywhere
+    x |= (np.arange(rows, dtype=np.uint32)[:, None] + 1) << 8  # byte 1: constant per row
+    x[3] |= rng.integers(0, 256, seg).astype(np.uint32) << 16  # byte 2 varies in row 3 only
+    check_rows(lib, torch_cuda, x, "per-row constant bytes")
+    check_rows(lib, torch_cuda, x.astype(np.int64), "per-row constant bytes, int64")
 
 
 # ---- swapaxes copy ------------------------------------------------------------------------------------
