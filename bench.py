@@ -294,7 +294,11 @@ def main() -> None:
     for label, ms in records:
         by_label.setdefault(label, []).append(ms)
     alg = algorithmic_bytes(cfg, job.uses_lds_rows)
-    dominant = "lds_row_sort" if job.uses_lds_rows else "onesweep"
+    if job.uses_lds_rows:  # one wavefront per row up to 1024 elements, one workgroup per row above
+        dominant = "wave_row_sort" if "wave_row_sort" in by_label else "lds_row_sort"
+        alg[dominant] = alg["lds_row_sort"]
+    else:
+        dominant = "onesweep"
     avg_ms = float(np.mean(by_label[dominant]))
     achieved = alg[dominant] / (avg_ms * 1e-3)
     kernels = {
@@ -332,7 +336,7 @@ def main() -> None:
         "dtype": {1: "u8", 2: "u16", 4: "u32", 8: "u64"}[cfg["x"].dtype.itemsize],
         "data": "synthetic",
         "config": {"workload": cfg["workload"], "keys": int(cfg["x"].size), "op": cfg["op"],
-                   "path": "lds_row_sort" if job.uses_lds_rows else "onesweep, 8-bit digits",
+                   "path": dominant if job.uses_lds_rows else "onesweep, 8-bit digits",
                    "workspace_bytes": int(job.temp_bytes)},
         "roofline": roofline,
         "whole_step": {"algorithmic_bytes": step_bytes, "GBps": step_bytes / (elapsed / args.steps) / 1e9,

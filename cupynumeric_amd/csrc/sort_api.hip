@@ -23,6 +23,18 @@ static std::atomic<long long> g_lds_row_limit{[] {
   return (e != nullptr && *e != 0) ? atoll(e) : -1ll;
 }()};
 
+// Longest row given to the one-wavefront-per-row kernel (0 = never).
+static std::atomic<long long> g_wave_row_limit{[] {
+  const char* e = getenv("CPN_SORT_WAVE_ROW_LIMIT");
+  return (e != nullptr && *e != 0) ? atoll(e) : 1024ll;
+}()};
+
+uint64_t wave_row_limit()
+{
+  const long long limit = g_wave_row_limit.load(std::memory_order_relaxed);
+  return limit < 0 ? 0 : (limit > 1024 ? 1024 : static_cast<uint64_t>(limit));
+}
+
 uint64_t lds_row_limit(int key_bytes)
 {
   const long long limit = g_lds_row_limit.load(std::memory_order_relaxed);
@@ -86,6 +98,11 @@ int cpn_last_hip_error(void) { return cpn::g_last_hip_error; }
 int64_t cpn_set_lds_row_limit(int64_t limit)
 {
   return static_cast<int64_t>(cpn::g_lds_row_limit.exchange(limit < 0 ? -1ll : static_cast<long long>(limit)));
+}
+
+int64_t cpn_set_wave_row_limit(int64_t limit)
+{
+  return static_cast<int64_t>(cpn::g_wave_row_limit.exchange(limit < 0 ? 1024ll : static_cast<long long>(limit)));
 }
 
 uint64_t cpn_dtype_size(int dtype) { return static_cast<uint64_t>(cpn::key_kind(dtype).bytes); }

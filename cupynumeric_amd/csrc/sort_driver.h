@@ -12,6 +12,8 @@
 #include "lds_row_sort.h"
 #include "onesweep.h"
 #include "profile.h"
+#include "tiny_row_sort.h"
+#include "wave_row_sort.h"
 
 namespace cpn {
 
@@ -71,6 +73,10 @@ __host__ __device__ constexpr int key_passes(int key_bytes, int codec)
 {
   return codec == CODEC_COMPLEX ? key_bytes + 1 : key_bytes;
 }
+
+// Row length up to which one wavefront (instead of one workgroup) sorts a row; at most 1024.
+// Changed by cpn_set_wave_row_limit / CPN_SORT_WAVE_ROW_LIMIT for A/B runs.
+uint64_t wave_row_limit();
 
 // Row length up to which the LDS kernel is used.  Equals lds_row_capacity unless the
 // environment variable CPN_SORT_LDS_ROW_LIMIT or cpn_set_lds_row_limit lowers it, e.g. to 0
@@ -199,12 +205,76 @@ inline int launch_lds_rows(const SortRequest& r)
   return CPN_OK;
 }
 
-// Rows are bucketed by length; each bucket has its own workgroup shape.
+template <typename KeyT, int CODEC, bool HAS_IDX, int ITEMS>
+inline int launch_wave_rows(const SortRequest& r)
+{
+  constexpr int LDS_PER_ROW    = wave_row_lds_bytes<CODEC, KeyT, ITEMS>();
+  constexpr int ROWS_PER_BLOCK = LDS_PER_ROW <= 12 * 1024 ? 4 : (LDS_PER_ROW <= 24 * 1024 ? 2 : 1);
+  const uint64_t rows          = r.volume / r.seg;
+  const uint64_t blocks        = (rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
+  {
+    ProfileScope prof("wave_row_sort", r.stream);
+    hipLaunchKernelGGL((wave_row_sort_kernel<KeyT, CODEC, HAS_IDX, ITEMS, ROWS_PER_BLOCK>),
+                       dim3(static_cast<uint32_t>(blocks)), dim3(WAVE * ROWS_PER_BLOCK), 0, r.stream,
+                       static_cast<const KeyT*>(r.values_in), static_cast<KeyT*>(r.values_out), r.indices_out,
+                       static_cast<uint32_t>(r.seg), rows, r.index_offset);
+  }
+  CPN_HIP_TRY(hipGetLastError());
+  return CPN_OK;
+}
+
+template <typename KeyT, int CODEC, bool HAS_IDX, int S>
+inline int launch_tiny_rows(const SortRequest& r)
+{
+  const uint64_t rows          = r.volume / r.seg;
+  const uint64_t rows_per_block = (256 / WAVE) * (WAVE / S);
+  const uint64_t blocks        = (rows + rows_per_block - 1) / rows_per_block;
+  {
+    ProfileScope prof("tiny_row_sort", r.stream);
+    hipLaunchKernelGGL((tiny_row_sort_kernel<KeyT, CODEC, HAS_IDX, S>), dim3(static_cast<uint32_t>(blocks)), dim3(256),
+                       0, r.stream, static_cast<const KeyT*>(r.values_in), static_cast<KeyT*>(r.values_out),
+                       r.indices_out, static_cast<uint32_t>(r.seg), rows, r.index_offset);
+  }
+  CPN_HIP_TRY(hipGetLastError());
+  return CPN_OK;
+}
+
+// Rows are bucketed by length; each bucket has its own kernel shape: several rows per wavefront
+// up to 32 elements, one wavefront per row for short rows, one workgroup per row above.
 template <typename KeyT, int CODEC, bool HAS_IDX>
 inline int sort_rows_in_lds(const SortRequest& r)
 {
   if (r.volume / r.seg >= (1ull << 31)) {
     return CPN_ERR_UNSUPPORTED;
+  }
+  if (r.seg <= 32 && r.seg <= wave_row_limit()) {
+    if (r.seg <= 1) {
+      return launch_tiny_rows<KeyT, CODEC, HAS_IDX, 1>(r);
+    } else if (r.seg <= 2) {
+      return launch_tiny_rows<KeyT, CODEC, HAS_IDX, 2>(r);
+    } else if (r.seg <= 4) {
+      return launch_tiny_rows<KeyT, CODEC, HAS_IDX, 4>(r);
+    } else if (r.seg <= 8) {
+      return launch_tiny_rows<KeyT, CODEC, HAS_IDX, 8>(r);
+    } else if (r.seg <= 16) {
+      return launch_tiny_rows<KeyT, CODEC, HAS_IDX, 16>(r);
+    } else {
+      return launch_tiny_rows<KeyT, CODEC, HAS_IDX, 32>(r);
+    }
+  }
+  // (keys of 8 bytes and more hold too many registers per lane at 16 items: 512 there)
+  if (r.seg <= wave_row_limit() && (sizeof(KeyT) < 8 || r.seg <= 512)) {
+    if (r.seg <= 64) {
+      return launch_wave_rows<KeyT, CODEC, HAS_IDX, 1>(r);
+    } else if (r.seg <= 128) {
+      return launch_wave_rows<KeyT, CODEC, HAS_IDX, 2>(r);
+    } else if (r.seg <= 256) {
+      return launch_wave_rows<KeyT, CODEC, HAS_IDX, 4>(r);
+    } else if (r.seg <= 512) {
+      return launch_wave_rows<KeyT, CODEC, HAS_IDX, 8>(r);
+    } else {
+      return launch_wave_rows<KeyT, CODEC, HAS_IDX, 16>(r);
+    }
   }
   if (r.seg <= 64) {
     return launch_lds_rows<KeyT, CODEC, HAS_IDX, 64, 1>(r);

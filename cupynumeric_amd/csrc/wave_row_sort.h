@@ -1,0 +1,275 @@
+// Short rows (up to 1024 elements): one wavefront sorts one row, several rows per workgroup,
+// and no workgroup barrier anywhere -- the 64 lanes of a wave execute their LDS operations in
+// order, so the phases of a pass need no synchronisation beyond that.
+//
+// The keys are turned into their order-preserving unsigned words once, when they are loaded,
+// and stay in registers in that form: a pass only extracts a byte.  Integer keys are mapped
+// back at the end (the transform is a bijection); float and complex keys cannot be (-0.0 and
+// NaN payloads are folded), so those rows always carry the 16-bit source position along and
+// the sorted values are gathered from the input row by position after the last pass.
+//
+// Replaces, for such rows, the (segment id, value) tuple merge sort of
+// src/cupynumeric/sort/thrust_sort.cuh:68-122 (rows of at most 400 elements) and
+// cub::DeviceSegmentedRadixSort (src/cupynumeric/sort/cub_sort.cuh:81-105,153-182).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "radix_common.h"
+
+namespace cpn {
+
+// The ordered key of one element as 32-bit words, least significant first; digit p is byte
+// p%4 of word p/4.
+template <int CODEC, typename KeyT>
+struct OrderedWords {
+  using KT                     = KeyTraits<CODEC, KeyT>;
+  static constexpr int PASSES  = KT::PASSES;
+  static constexpr int NW      = (PASSES + 3) / 4;
+  static constexpr bool BIJECT = (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED);
+
+  static __device__ __forceinline__ void encode(KeyT raw, uint32_t (&w)[NW])
+  {
+    uint64_t q[KT::NWORDS];
+    KT::words(raw, q);
+#pragma unroll
+    for (int n = 0; n < NW; ++n) {
+      w[n] = static_cast<uint32_t>(q[n / 2] >> ((n % 2) * 32));
+    }
+  }
+  // only for bijective codecs
+  static __device__ __forceinline__ KeyT decode(const uint32_t (&w)[NW])
+  {
+    if constexpr (sizeof(KeyT) <= 8 && BIJECT) {
+      uint64_t v = w[0];
+      if constexpr (NW > 1) {
+        v |= static_cast<uint64_t>(w[1]) << 32;
+      }
+      const KeyT o = static_cast<KeyT>(v);
+      if constexpr (CODEC == CODEC_SIGNED) {
+        return static_cast<KeyT>(o ^ (static_cast<KeyT>(1) << (sizeof(KeyT) * 8 - 1)));
+      } else {
+        return o;
+      }
+    } else {
+      return KeyT{};
+    }
+  }
+};
+
+template <typename T>
+__device__ __forceinline__ T wave_all_and(T v)
+{
+#pragma unroll
+  for (int delta = WAVE / 2; delta > 0; delta >>= 1) {
+    v &= __shfl_xor(v, delta, WAVE);
+  }
+  return v;
+}
+template <typename T>
+__device__ __forceinline__ T wave_all_or(T v)
+{
+#pragma unroll
+  for (int delta = WAVE / 2; delta > 0; delta >>= 1) {
+    v |= __shfl_xor(v, delta, WAVE);
+  }
+  return v;
+}
+
+// bytes of LDS one wave (= one row) needs
+template <int CODEC, typename KeyT, int ITEMS>
+__host__ __device__ constexpr int wave_row_lds_bytes()
+{
+  return OrderedWords<CODEC, KeyT>::NW * 4 * ITEMS * WAVE + 2 * ITEMS * WAVE + RADIX * 4;
+}
+
+template <typename KeyT, int CODEC, bool HAS_IDX, int ITEMS, int ROWS_PER_BLOCK>
+__global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(const KeyT* keys_in,
+                                                                              KeyT* keys_out,
+                                                                              int64_t* idx_out,
+                                                                              uint32_t seg,
+                                                                              uint64_t rows,
+                                                                              int64_t index_offset)
+{
+  using OW                = OrderedWords<CODEC, KeyT>;
+  constexpr int NW        = OW::NW;
+  constexpr int PASSES    = OW::PASSES;
+  constexpr int TILE      = ITEMS * WAVE;
+  constexpr bool CARRY    = HAS_IDX || !OW::BIJECT;  // source positions travel with the keys
+  static_assert(TILE <= 65536, "positions are 16 bits");
+
+  __shared__ uint32_t s_words[ROWS_PER_BLOCK][NW][TILE];
+  __shared__ uint16_t s_pos[ROWS_PER_BLOCK][CARRY ? TILE : 1];
+  __shared__ uint32_t s_ctr[ROWS_PER_BLOCK][RADIX];
+
+  const int lane     = threadIdx.x & (WAVE - 1);
+  const int wave     = threadIdx.x / WAVE;
+  const uint64_t row = static_cast<uint64_t>(blockIdx.x) * ROWS_PER_BLOCK + wave;
+  if (row >= rows) {
+    return;  // whole wave; no workgroup barrier is used below
+  }
+  const uint64_t base = row * seg;
+  uint32_t* ctr       = s_ctr[wave];
+  const bool full     = (seg == TILE);
+
+  // ---- load, item i of lane l is element i*64 + l of the row; encode once ----
+  uint32_t w[ITEMS][NW];
+  uint32_t pos2[CARRY ? (ITEMS + 1) / 2 : 1];  // source positions, two per register
+  uint32_t vary_and[NW], vary_or[NW];
+#pragma unroll
+  for (int n = 0; n < NW; ++n) {
+    vary_and[n] = 0xFFFFFFFFu;
+    vary_or[n]  = 0;
+  }
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t o = i * WAVE + lane;
+    if (full || o < seg) {
+      OW::encode(keys_in[base + o], w[i]);
+#pragma unroll
+      for (int n = 0; n < NW; ++n) {
+        vary_and[n] &= w[i][n];
+        vary_or[n] |= w[i][n];
+      }
+    } else {
+#pragma unroll
+      for (int n = 0; n < NW; ++n) {
+        w[i][n] = 0;
+      }
+    }
+    if constexpr (CARRY) {
+      pos2[i / 2] = (i % 2 == 0) ? o : (pos2[i / 2] | (o << 16));
+    }
+  }
+  // passes on whose digit the whole row agrees are the identity permutation: skip them
+  uint32_t active = 0;
+#pragma unroll
+  for (int n = 0; n < NW; ++n) {
+    const uint32_t v = wave_all_and(vary_and[n]) ^ wave_all_or(vary_or[n]);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      if (n * 4 + b < PASSES && ((v >> (8 * b)) & 0xFFu) != 0) {
+        active |= 1u << (n * 4 + b);
+      }
+    }
+  }
+
+  for (int pass = 0; pass < PASSES; ++pass) {
+    if (((active >> pass) & 1u) == 0) {
+      continue;  // uniform for the wave
+    }
+    const int word  = pass / 4;
+    const int shift = (pass % 4) * 8;
+#pragma unroll
+    for (int j = 0; j < RADIX / WAVE; ++j) {
+      ctr[j * WAVE + lane] = 0;
+    }
+    __builtin_amdgcn_wave_barrier();
+    // ---- rank: counters run from zero ----
+    uint32_t dpk[(ITEMS + 3) / 4];   // digits, four per register
+    uint32_t rnk2[(ITEMS + 1) / 2];  // ranks, two per register
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      uint32_t wsel = w[i][0];
+#pragma unroll
+      for (int n = 1; n < NW; ++n) {
+        wsel = (word == n) ? w[i][n] : wsel;
+      }
+      const uint32_t d = (wsel >> shift) & 0xFFu;
+      const uint32_t r = wave_match_rank(d, full || (i * WAVE + lane < seg), ctr) & 0xFFFFu;
+      dpk[i / 4]       = (i % 4 == 0) ? d : (dpk[i / 4] | (d << (8 * (i % 4))));
+      rnk2[i / 2]      = (i % 2 == 0) ? r : (rnk2[i / 2] | (r << 16));
+      // opaque to the optimiser, which would otherwise keep one register per digit and rank
+      asm volatile("" : "+v"(dpk[i / 4]), "+v"(rnk2[i / 2]));
+    }
+    // ---- exclusive scan of the 256 counts: lane l owns digits 4l .. 4l+3 ----
+    {
+      uint32_t c[RADIX / WAVE], sum = 0;
+#pragma unroll
+      for (int j = 0; j < RADIX / WAVE; ++j) {
+        c[j] = ctr[lane * (RADIX / WAVE) + j];
+        sum += c[j];
+      }
+      uint32_t run = wave_inclusive_scan(sum, lane) - sum;
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int j = 0; j < RADIX / WAVE; ++j) {
+        ctr[lane * (RADIX / WAVE) + j] = run;
+        run += c[j];
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+    // ---- exchange through LDS ----
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      if (full || (i * WAVE + lane < seg)) {
+        const uint32_t p = ctr[(dpk[i / 4] >> (8 * (i % 4))) & 0xFFu] + ((rnk2[i / 2] >> (16 * (i % 2))) & 0xFFFFu);
+#pragma unroll
+        for (int n = 0; n < NW; ++n) {
+          s_words[wave][n][p] = w[i][n];
+        }
+        if constexpr (CARRY) {
+          s_pos[wave][p] = static_cast<uint16_t>(pos2[i / 2] >> (16 * (i % 2)));
+        }
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      const uint32_t o = i * WAVE + lane;
+      if (full || o < seg) {
+#pragma unroll
+        for (int n = 0; n < NW; ++n) {
+          w[i][n] = s_words[wave][n][o];
+        }
+        if constexpr (CARRY) {
+          const uint32_t q = s_pos[wave][o];
+          pos2[i / 2]      = (i % 2 == 0) ? q : (pos2[i / 2] | (q << 16));
+        }
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+
+  // ---- results ----
+  if (keys_out != nullptr) {
+    KeyT v[ITEMS];
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      const uint32_t o = i * WAVE + lane;
+      if (full || o < seg) {
+        if constexpr (OW::BIJECT) {
+          v[i] = OW::decode(w[i]);
+        } else {
+          v[i] = keys_in[base + ((pos2[i / 2] >> (16 * (i % 2))) & 0xFFFFu)];  // every gather of the row is issued before any store
+        }
+      } else {
+        v[i] = KeyT{};
+      }
+    }
+    if constexpr (!OW::BIJECT) {
+      // keys_out may alias keys_in: every gather of the row must have returned before the
+      // first store overwrites it (the asm also keeps the compiler from moving either across)
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      const uint32_t o = i * WAVE + lane;
+      if (full || o < seg) {
+        keys_out[base + o] = v[i];
+      }
+    }
+  }
+  if constexpr (HAS_IDX) {
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      const uint32_t o = i * WAVE + lane;
+      if (full || o < seg) {
+        idx_out[base + o] = static_cast<int64_t>((pos2[i / 2] >> (16 * (i % 2))) & 0xFFFFu) + index_offset;
+      }
+    }
+  }
+}
+
+}  // namespace cpn

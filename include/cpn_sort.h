@@ -79,6 +79,14 @@ int cpn_last_hip_error(void);
  */
 int64_t cpn_set_lds_row_limit(int64_t limit);
 
+/*
+ * Process-wide tunable: rows of at most `limit` elements (at most 1024) are sorted by one
+ * wavefront each, longer rows that fit in LDS by one workgroup each.  A negative value
+ * restores the default; the previous setting is returned.  Also initialised from the
+ * environment variable CPN_SORT_WAVE_ROW_LIMIT.  Does not affect workspace sizes.
+ */
+int64_t cpn_set_wave_row_limit(int64_t limit);
+
 /* Size in bytes of one element of `dtype`, or 0 for an unknown code. */
 uint64_t cpn_dtype_size(int dtype);
 
