@@ -205,19 +205,23 @@ def verify_sample(job: GpuJob, cfg: dict) -> str:
 # -------------------------------------------------------------------------------------------------
 # CPU baseline: restatement of the reference's CPU / OpenMP variant on a bounded sample
 # -------------------------------------------------------------------------------------------------
+# keys of the workload the CPU baseline sorts: about 10 s on one core plus 1-2 s on all of them
+CPU_SAMPLE_KEYS = 1 << 26
+
+
 def cpu_baseline(cfg: dict) -> dict:
     from oracle import sort_oracle as oracle
 
     x = cfg["x"]
     argsort = cfg["op"] == "argsort"
     if x.ndim == 1:
-        sample = x[: min(x.size, 1 << 24)]
+        sample = x[: min(x.size, CPU_SAMPLE_KEYS)]
         what = f"first 2^{int(np.log2(sample.size))} keys of the workload"
     elif cfg["axis"] == 0:
-        sample = np.ascontiguousarray(x[:, : min(x.shape[1], 512)].T)
+        sample = np.ascontiguousarray(x[:, : min(x.shape[1], max(1, CPU_SAMPLE_KEYS // x.shape[0]))].T)
         what = f"{sample.shape[0]} columns of the workload (transposes not timed)"
     else:
-        sample = x[: min(x.shape[0], 8192)]
+        sample = x[: min(x.shape[0], max(1, CPU_SAMPLE_KEYS // x.shape[1]))]
         what = f"first {sample.shape[0]} rows of the workload"
     threads = min(oracle.max_threads(), os.cpu_count() or 1, 16)
     best = None
