@@ -35,9 +35,15 @@ if str(ROOT) not in sys.path:
 HBM_PEAK_BYTES_PER_S = 8.0e12  # MI355X HBM3E
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# of this file scaled by a plain copy of known size (profiles/onesweep_c2_traffic.txt).  Keyed by
+# of this file scaled by a plain copy of known size (profiles/*_traffic.txt).  Keyed by
 # (config, keys); workloads without such a measurement report null.
-MEASURED_TRAFFIC_BYTES = {("c2", 1 << 28): 4.519e9}
+MEASURED_TRAFFIC_BYTES = {
+    ("c1", 1 << 24): 1.466e8,   # onesweep, profiles/onesweep_c1_traffic.txt
+    ("c2", 1 << 28): 4.384e9,   # onesweep, profiles/onesweep_c2_traffic.txt
+    ("c3", 1 << 26): 1.0738e9,  # lds_row_sort, profiles/lds_row_sort_c3_traffic.txt
+    ("c4", 1 << 27): 3.2465e9,  # onesweep, profiles/onesweep_c4_traffic.txt
+    ("c5", 1 << 26): 2.687e8,   # lds_row_sort, profiles/lds_row_sort_c5_traffic.txt
+}
 
 
 # -------------------------------------------------------------------------------------------------
