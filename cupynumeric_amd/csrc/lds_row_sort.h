@@ -9,6 +9,13 @@
 // Digits on which every key of the row agrees are found up front with one AND/OR
 // reduction of the ordered keys and their passes are skipped (the pass would be the
 // identity permutation).
+//
+// Wide keys: a row of n keys is almost always put in order by its leading 2*log2(n) or so
+// varying bits.  When more passes than that are due, the kernel first runs only the passes of
+// the most significant varying digits, then checks that every neighbouring pair of the result
+// is in order on the whole key.  If so the row is sorted (stably: ties on the leading digits
+// whose remaining digits also tie kept their input order).  If not, all passes are run, from
+// the state reached, which is still a stable sort of the input.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -127,9 +134,27 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
     }
   }
 
+  // leading-digits shortcut (see the head of this file)
+  uint32_t todo  = active;
+  bool shortcut  = false;
+  if constexpr (PASSES >= 5) {
+    const int lead = (2 * (32 - __builtin_clz(seg - 1 | 1u)) + 4 + RADIX_BITS - 1) / RADIX_BITS;
+    if (__builtin_popcount(active) >= lead + 2) {
+      uint32_t rem = active;
+      todo         = 0;
+      for (int t = 0; t < lead; ++t) {
+        const uint32_t top = 1u << (31 - __builtin_clz(rem));
+        todo |= top;
+        rem ^= top;
+      }
+      shortcut = true;
+    }
+  }
+
   uint32_t* wctr = s_ctr + wave * RADIX;
+  for (;;) {
   for (int pass = 0; pass < PASSES; ++pass) {
-    if (((active >> pass) & 1u) == 0) {
+    if (((todo >> pass) & 1u) == 0) {
       continue;  // uniform for the block
     }
     for (int j = tid; j < WAVES * RADIX; j += BLOCK) {
@@ -203,6 +228,33 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
       }
     }
     // the next pass (or nothing) touches s_keys only after its own barriers
+  }
+    if (!shortcut) {
+      break;
+    }
+    // s_keys holds the row as ordered by the leading digits: is every neighbouring pair in order?
+    int bad = 0;
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      const uint32_t o = woff + i * WAVE;
+      if (o + 1 < seg) {
+        uint64_t a[NW], b[NW];
+        KT::words(key[i], a);
+        KT::words(s_keys[o + 1], b);
+        bool gt = false, eq = true;  // a > b, most significant word first
+#pragma unroll
+        for (int n = NW - 1; n >= 0; --n) {
+          gt = gt || (eq && a[n] > b[n]);
+          eq = eq && (a[n] == b[n]);
+        }
+        bad |= gt ? 1 : 0;
+      }
+    }
+    if (__syncthreads_or(bad) == 0) {
+      break;
+    }
+    shortcut = false;
+    todo     = active;
   }
 
 #pragma unroll

@@ -281,10 +281,12 @@ inline int sort_rows_in_lds(const SortRequest& r)
   } else if (r.seg <= 256) {
     return launch_lds_rows<KeyT, CODEC, HAS_IDX, 64, 4>(r);
   } else if (r.seg <= 1024) {
-    return launch_lds_rows<KeyT, CODEC, HAS_IDX, 256, 4>(r);
+    return launch_lds_rows<KeyT, CODEC, HAS_IDX, 128, 8>(r);
+  } else if (r.seg <= 2048) {
+    return launch_lds_rows<KeyT, CODEC, HAS_IDX, 256, 8>(r);
   }
   if constexpr (sizeof(KeyT) == 16) {
-    return launch_lds_rows<KeyT, CODEC, HAS_IDX, 256, 8>(r);  // up to lds_row_capacity(16) == 2048
+    return CPN_ERR_UNSUPPORTED;  // not reached: lds_row_capacity(16) == 2048
   } else {
     if (r.seg <= 4096) {
       return launch_lds_rows<KeyT, CODEC, HAS_IDX, 256, 16>(r);

@@ -155,8 +155,28 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
     }
   }
 
+  // Wide keys: run the passes of the leading varying digits only (2*log2(n) + 4 bits put n keys
+  // in order almost always), then check every neighbouring pair on the whole key; if one is
+  // out of order, run all passes from the state reached (still a stable sort of the input).
+  uint32_t todo = active;
+  bool shortcut = false;
+  if constexpr (PASSES >= 5) {
+    const int lead = (2 * (32 - __builtin_clz(seg - 1 | 1u)) + 4 + RADIX_BITS - 1) / RADIX_BITS;
+    if (__builtin_popcount(active) >= lead + 2) {
+      uint32_t rem = active;
+      todo         = 0;
+      for (int t = 0; t < lead; ++t) {
+        const uint32_t top = 1u << (31 - __builtin_clz(rem));
+        todo |= top;
+        rem ^= top;
+      }
+      shortcut = true;
+    }
+  }
+
+  for (;;) {
   for (int pass = 0; pass < PASSES; ++pass) {
-    if (((active >> pass) & 1u) == 0) {
+    if (((todo >> pass) & 1u) == 0) {
       continue;  // uniform for the wave
     }
     const int word  = pass / 4;
@@ -230,6 +250,31 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
       }
     }
     __builtin_amdgcn_wave_barrier();
+  }
+    if (!shortcut) {
+      break;
+    }
+    // s_words holds the row as ordered by the leading digits
+    bool bad = false;
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      const uint32_t o = i * WAVE + lane;
+      if (o + 1 < seg) {
+        bool gt = false, eq = true;  // this key > its right neighbour, most significant word first
+#pragma unroll
+        for (int n = NW - 1; n >= 0; --n) {
+          const uint32_t b = s_words[wave][n][o + 1];
+          gt               = gt || (eq && w[i][n] > b);
+          eq               = eq && (w[i][n] == b);
+        }
+        bad = bad || gt;
+      }
+    }
+    if (__builtin_amdgcn_ballot_w64(bad) == 0) {
+      break;
+    }
+    shortcut = false;
+    todo     = active;
   }
 
   // ---- results ----

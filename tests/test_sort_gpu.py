@@ -169,6 +169,50 @@ def test_lds_many_short_rows(lib, torch_cuda):
         check_rows(lib, torch_cuda, make_input(dtype, shape, seed=11), f"{np.dtype(dtype)} {shape}")
 
 
+@pytest.mark.parametrize("dtype", [np.int64, np.uint64, np.float64, np.complex64, np.complex128])
+@pytest.mark.parametrize("seg", [600, 1024, 1500, 4096])
+def test_lds_rows_leading_digit_shortcut(lib, torch_cuda, dtype, seg):
+    """Wide keys in the row kernels: rows that the leading digits order completely, rows with ties on
+    the leading digits whose low digits are out of order (the check must fail and every pass run),
+    and rows with ties that happen to be in order; mixed in one launch."""
+    rng = np.random.default_rng(seg + np.dtype(dtype).itemsize)
+    rows = 12
+    if np.dtype(dtype).kind == "c":
+        comp = np.float32 if dtype == np.complex64 else np.float64
+        re = rng.standard_normal((rows, seg)).astype(comp)
+        im = rng.standard_normal((rows, seg)).astype(comp)
+        re[3:6] = rng.integers(0, 3, (3, seg)).astype(comp)           # ties on the real part: imag decides
+        im[6:8] = np.sort(im[6:8], axis=-1)
+        re[6:8] = np.repeat(np.sort(rng.integers(0, 4, (2, seg // 4 + 1)), axis=-1), 4, axis=-1)[:, :seg]
+        re[8, ::7] = np.nan
+        im[9, ::5] = np.nan
+        x = (re + 1j * im).astype(dtype)
+        x.real[8, ::7] = np.nan
+    else:
+        info_bits = 8 * np.dtype(dtype).itemsize
+        lo = rng.integers(0, 1 << 40, (rows, seg), dtype=np.uint64)
+        hi = rng.integers(0, 1 << 23, (rows, seg), dtype=np.uint64) << np.uint64(40)
+        hi[3:6] = rng.integers(0, 5, (3, seg), dtype=np.uint64) << np.uint64(40)     # heavy ties, low bits random
+        hi[6:8] = np.sort(rng.integers(0, 9, (2, seg), dtype=np.uint64), axis=-1) << np.uint64(40)
+        lo[6:8] = np.sort(lo[6:8], axis=-1)                                            # ties, already in order
+        lo[8] &= np.uint64(0xFF)                                                       # few low digits vary
+        bits = hi | lo
+        if np.dtype(dtype).kind == "f":
+            bits = (bits & np.uint64((1 << 62) - 1)) | (np.uint64(0x3F) << np.uint64(56)) & np.uint64((1 << 64) - 1)
+            x = bits.view(np.float64).copy()
+            x[9, ::3] *= -1.0
+            x[10, ::11] = np.nan
+            x[10, 1::11] = -0.0
+            x[10, 2::11] = 0.0
+        else:
+            x = bits.view(dtype).copy()
+            assert info_bits == 64
+    check_rows(lib, torch_cuda, x, f"{np.dtype(dtype)} seg={seg} shortcut")
+    v, i = abi_sort(lib, torch_cuda, x.copy(), want_values=True, want_indices=True, in_place=True)
+    assert_same_bits(v, oracle.local_sort(x, argsort=False), "in place values")
+    assert_same_bits(i, oracle.local_sort(x, argsort=True), "in place indices")
+
+
 # ---- global onesweep path ---------------------------------------------------------------------------
 GLOBAL_LENGTHS = [1, 2, 100, 4097, 8191, 8192, 8193, 16383, 16384, 16385, 3 * 16384 + 5, 100003]
 
