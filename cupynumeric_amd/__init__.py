@@ -19,7 +19,7 @@ from ._array import convert_to_ndarray, ndarray
 from ._thunk import SUPPORTED_DTYPES, DeviceArray, check_dtype
 
 __all__ = [
-    "ndarray", "array", "asarray", "sort", "argsort", "sort_complex", "partition", "argpartition", "random",
+    "ndarray", "array", "asarray", "sort", "argsort", "sort_complex", "partition", "argpartition", "lexsort", "random",
     "SUPPORTED_DTYPES",
 ]
 
@@ -100,3 +100,68 @@ def partition(a: Any, kth: Any, axis: int | None = -1, kind: str = "introselect"
     if axis is None and a.ndim > 1:
         result._thunk.shape = (a.size,)
     return result
+
+
+def lexsort(keys: Any, axis: int | None = -1) -> ndarray:
+    """Indirect stable sort on several keys, the last key being the primary one
+    (`cupynumeric/_module/ssc_sorting.py:271-444`).  `keys` is a sequence of arrays of one
+    shape, or one array whose first dimension runs over the keys.  Returns int64 indices of
+    the shape of one key.  `axis=None` is rejected as NumPy does."""
+    from numpy.exceptions import AxisError
+
+    from ._sort import lexsort_deferred
+
+    if keys is None:
+        raise TypeError("'NoneType' object is not iterable")
+    if axis is None:
+        raise TypeError("'NoneType' object cannot be interpreted as an integer")
+
+    if isinstance(keys, ndarray):
+        if keys.ndim == 0:
+            raise TypeError("need sequence of keys with len > 0 in lexsort")
+        key_list = _split_first_axis(keys)
+    else:
+        try:
+            key_list = [convert_to_ndarray(k) for k in keys]
+        except TypeError as exc:
+            if "does not support dtype" in str(exc):
+                raise
+            raise TypeError(str(exc))
+    if len(key_list) == 0:
+        raise TypeError("Need at least one key to sort")
+
+    # all keys must have one shape
+    first_shape = key_list[0].shape
+    for i, key in enumerate(key_list[1:], 1):
+        if key.shape != first_shape:
+            raise ValueError(
+                f"All keys must have the same shape. Key {i} has shape {key.shape}, expected {first_shape}"
+            )
+
+    # scalar keys: there is only one element
+    if len(first_shape) == 0:
+        return array(np.zeros((), dtype=np.int64))
+
+    ndim = len(first_shape)
+    if axis >= ndim or axis < -ndim:
+        raise AxisError(f"axis {axis} is out of bounds for array of dimension {ndim}")
+
+    # valid keys without data
+    if key_list[0].size == 0:
+        return ndarray(first_shape, np.int64)
+
+    thunk = lexsort_deferred([k._thunk for k in key_list], axis)
+    return ndarray(thunk.shape, np.int64, thunk=thunk)
+
+
+def _split_first_axis(a: ndarray) -> list[ndarray]:
+    """The keys of a single stacked array: `a[0], a[1], ...` as dense arrays sharing nothing."""
+    if a.shape[0] == 0:
+        return []
+    host_or_dev = a._thunk
+    inner = a.shape[1:]
+    n_inner = int(np.prod(inner, dtype=np.int64))
+    out = []
+    for i in range(a.shape[0]):
+        out.append(ndarray(inner, a.dtype, thunk=host_or_dev.slice_first_axis(i, n_inner, inner)))
+    return out

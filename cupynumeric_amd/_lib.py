@@ -60,6 +60,9 @@ PROTOTYPES: dict[str, tuple] = {
     ),
     "cpn_local_sort_check": (c_int, [c_void_p, c_void_p]),
     "cpn_real_to_complex": (c_int, [c_int, c_void_p, c_int, c_void_p, c_uint64, c_void_p]),
+    "cpn_take_along_last_axis": (
+        c_int, [c_int, c_void_p, c_void_p, c_void_p, c_uint64, c_uint64, c_uint64, c_void_p, c_void_p]
+    ),
     "cpn_profile_enable": (c_int, [c_int]),
     "cpn_profile_collect": (c_int, [c_void_p, c_uint64, c_void_p, c_int]),
     "cpn_swapaxes_copy": (c_int, [c_int, c_void_p, c_void_p, ctypes.POINTER(c_int64), c_int, c_int, c_int, c_void_p]),

@@ -137,3 +137,34 @@ def sort_deferred(
                 sort_task(output, input, argsort, stable)
             else:
                 sort_swapped(output, input, argsort, computed_axis, stable)
+
+
+def lexsort_deferred(keys: "list[DeviceArray]", axis: int) -> "DeviceArray":
+    """The loop of `lexsort` (`cupynumeric/_module/ssc_sorting.py:423-444`): a stable argsort of
+    the least significant key, then for every further key: reorder the key by the indices so
+    far, argsort it (stable), reorder the indices by that order.  `keys[-1]` is the primary key.
+
+    Every key is sorted in its own element type under the NumPy order, which already puts
+    -inf < finite < +inf < NaN, so the reference's remapping of special float values
+    (`ssc_sorting.py:352-420`) has nothing to do here.  Axes other than the last are moved
+    there once (one transpose per key, one for the result) instead of once per argsort.
+    """
+    from ._thunk import DeviceArray
+
+    ndim = keys[0].ndim
+    axis = normalize_axis_index(axis, ndim)
+    last = ndim - 1
+    if axis != last:
+        keys = [k.swapaxes_copy(axis, last) for k in keys]
+
+    indices = DeviceArray(keys[0].shape, dtype="int64")
+    sort_task(indices, keys[0], True, True)
+    for key in keys[1:]:
+        key_reordered = key.take_along_last_axis(indices)
+        order = DeviceArray(key.shape, dtype="int64")
+        sort_task(order, key_reordered, True, True)
+        indices = indices.take_along_last_axis(order)
+
+    if axis != last:
+        indices = indices.swapaxes_copy(last, axis)
+    return indices

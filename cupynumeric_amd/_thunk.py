@@ -98,6 +98,18 @@ class DeviceArray:
             raise ValueError("cannot reshape array: sizes differ")
         return out
 
+    def slice_first_axis(self, i: int, count: int, shape: tuple[int, ...]) -> "DeviceArray":
+        """`self[i]` as an array of `shape` (`count` elements) over the same memory: rows of a
+        dense row-major buffer are themselves dense."""
+        nbytes = count * self.dtype.itemsize
+        sub = Storage(nbytes)
+        if self.base._dev is None and self.base._host is not None:
+            host = np.asarray(self.base._host).reshape(self.shape)
+            sub._host = np.ascontiguousarray(host[i])
+        else:
+            sub._dev = self.base.device()[i * nbytes : (i + 1) * nbytes] if nbytes else runtime.empty_bytes(0)
+        return DeviceArray(shape, self.dtype, sub)
+
     def swapaxes_copy(self, axis1: int, axis2: int) -> "DeviceArray":
         """Dense copy with two axes exchanged: the reference's `swapaxes` view followed by
         `copy(deep=True)` (`cupynumeric/_thunk/_sort.py:59-65`) in one kernel."""
@@ -119,6 +131,39 @@ class DeviceArray:
             runtime.stream_handle(),
         )
         _lib.check(status, "cpn_swapaxes_copy")
+        return out
+
+    def take_along_last_axis(self, indices: "DeviceArray") -> "DeviceArray":
+        """`take_along_axis(self, indices, axis=-1)` for arrays whose leading dimensions agree
+        (`cupynumeric/_module/indexing.py:648-760`; the TAKE task's no-broadcast case)."""
+        if indices.dtype != np.dtype(np.int64):
+            raise TypeError("`indices` must be an int64 array")
+        if self.ndim != indices.ndim or self.ndim == 0:
+            raise ValueError("`indices` and `a` must have the same number of dimensions")
+        if self.shape[:-1] != indices.shape[:-1]:
+            raise ValueError("take_along_last_axis: leading dimensions must agree")
+        out = DeviceArray(indices.shape, self.dtype)
+        if out.size == 0:
+            return out
+        if self.shape[-1] == 0:
+            raise IndexError("index out of bounds: cannot take from an empty axis")
+        lib = _lib.load()
+        rows = indices.size // indices.shape[-1]
+        flag = runtime.zero_flag()
+        status = lib.cpn_take_along_last_axis(
+            self.dtype.itemsize,
+            self.base.ptr(),
+            indices.base.ptr(),
+            out.base.ptr(),
+            rows,
+            self.shape[-1],
+            indices.shape[-1],
+            flag.data_ptr(),
+            ctypes.c_void_p(runtime.stream_handle()),
+        )
+        _lib.check(status, "cpn_take_along_last_axis")
+        if runtime.check_status and int(flag.item()) != 0:
+            raise IndexError("index out of bounds in take_along_axis")
         return out
 
     # -- the sort entry point ---------------------------------------------------------------

@@ -25,6 +25,7 @@ SOURCES = [
     "swapaxes.hip",
     "profile.hip",
     "convert.hip",
+    "gather.hip",
     "sort_keys8.hip",
     "sort_keys16.hip",
     "sort_keys32.hip",

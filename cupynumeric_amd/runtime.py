@@ -54,6 +54,11 @@ class Runtime:
         dev = self.require_device()
         return self.torch.empty(max(int(nbytes), 1), dtype=self.torch.uint8, device=dev)
 
+    def zero_flag(self) -> "torch.Tensor":
+        """A cleared 4-byte device word for kernels that report a condition (e.g. a bad index)."""
+        dev = self.require_device()
+        return self.torch.zeros(1, dtype=self.torch.int32, device=dev)
+
     def upload(self, host: np.ndarray) -> "torch.Tensor":
         """Copy a C-contiguous host array to a new device byte buffer."""
         dev = self.require_device()

@@ -163,6 +163,19 @@ int cpn_real_to_complex(int src_dtype, const void* in, int dst_dtype, void* out,
                         void* stream);
 
 /*
+ * out[r][j] = src[r][indices[r][j]] for `rows` dense rows: src rows hold src_seg elements of
+ * elem_bytes (1, 2, 4, 8 or 16) bytes, indices and out rows hold idx_seg elements.  Indices are
+ * int64, negative ones count from the end of the row.  An index outside [-src_seg, src_seg)
+ * writes nothing and stores 1 to *oob_flag (device memory, may be NULL; the caller clears it).
+ * This is the take_along_axis that lexsort applies between its argsorts
+ * (cupynumeric/_module/ssc_sorting.py:430-442, cupynumeric/_module/indexing.py:648-760), on the
+ * last axis; other axes go through cpn_swapaxes_copy first.  out must not overlap the inputs.
+ */
+int cpn_take_along_last_axis(int elem_bytes, const void* src, const int64_t* indices, void* out,
+                             uint64_t rows, uint64_t src_seg, uint64_t idx_seg, uint32_t* oob_flag,
+                             void* stream);
+
+/*
  * Per-launch timing.  cpn_profile_enable(1) makes every kernel launch of the library record
  * a pair of HIP events on the stream it is launched on; it returns the previous setting.
  * cpn_profile_collect waits for the recorded events, writes up to `max_records` entries --

@@ -12,6 +12,9 @@ Two layers, mirroring the reference:
   `cupynumeric/_thunk/_sort.py:37-136` (flatten / last axis / swap-sort-swap), with NumPy doing the
   `swapaxes` copies.
 
+* `lexsort` restates the loop of `cupynumeric/_module/ssc_sorting.py:271-444` over `argsort`
+  above, with NumPy's `take_along_axis` between the steps.
+
 Deviation kept on purpose (same as the product): results are always stable.
 """
 from __future__ import annotations
@@ -142,3 +145,44 @@ def argsort(a, axis=-1, kind="quicksort", order=None, threads: int = 1) -> np.nd
     if x.dtype not in DTYPE_CODES:
         raise TypeError(f"cuPyNumeric does not support dtype={x.dtype}")
     return _thunk_sort(x, True, axis, kind, order, threads)
+
+
+def lexsort(keys, axis=-1, threads: int = 1) -> np.ndarray:
+    """`cupynumeric/_module/ssc_sorting.py:271-444`: validation, then a stable argsort of the first
+    key and, for every further key, reorder / argsort / reorder.  Keys keep their own element
+    type; the oracle's ordering already is -inf < finite < +inf < NaN, which is what the
+    reference's remapping of special values (:352-420) establishes before it sorts."""
+    if keys is None:
+        raise TypeError("'NoneType' object is not iterable")
+    if axis is None:
+        raise TypeError("'NoneType' object cannot be interpreted as an integer")
+    if isinstance(keys, np.ndarray):
+        if keys.ndim == 0:
+            raise TypeError("need sequence of keys with len > 0 in lexsort")
+        key_list = [keys[i] for i in range(keys.shape[0])]
+    else:
+        key_list = [np.asarray(k) for k in keys]
+    if len(key_list) == 0:
+        raise TypeError("Need at least one key to sort")
+    for k in key_list:
+        if k.dtype not in DTYPE_CODES:
+            raise TypeError(f"cuPyNumeric does not support dtype={k.dtype}")
+    first_shape = key_list[0].shape
+    for i, key in enumerate(key_list[1:], 1):
+        if key.shape != first_shape:
+            raise ValueError(
+                f"All keys must have the same shape. Key {i} has shape {key.shape}, expected {first_shape}"
+            )
+    if key_list[0].ndim == 0:
+        return np.zeros((), dtype=np.int64)
+    ndim = key_list[0].ndim
+    if axis >= ndim or axis < -ndim:
+        raise AxisError(f"axis {axis} is out of bounds for array of dimension {ndim}")
+    if key_list[0].size == 0:
+        return np.empty(first_shape, dtype=np.int64)
+    indices = argsort(key_list[0], axis=axis, kind="stable", threads=threads)
+    for key in key_list[1:]:
+        key_reordered = np.take_along_axis(key, indices, axis=axis)
+        order = argsort(key_reordered, axis=axis, kind="stable", threads=threads)
+        indices = np.take_along_axis(indices, order, axis=axis)
+    return indices

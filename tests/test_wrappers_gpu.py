@@ -62,3 +62,47 @@ def test_partition_validation():
         num.partition(a, 1, axis=2)
     with pytest.raises(NotImplementedError):
         num.argpartition(a, 1, order="x")
+
+
+# ---- lexsort (cupynumeric/_module/ssc_sorting.py:271-444, tests/integration/test_lexsort.py) ---------
+def test_lexsort_reference_cases():
+    from lexsort_cases import cases, random_cases
+
+    from oracle import sort_oracle as oracle
+
+    for name, keys, axis in cases() + random_cases():
+        want = oracle.lexsort(keys, axis=axis)
+        assert np.array_equal(want, np.lexsort(keys, axis=axis)), name
+        if isinstance(keys, np.ndarray):
+            got = num.lexsort(num.array(keys), axis=axis)
+        else:
+            got = num.lexsort(tuple(num.array(k) for k in keys), axis=axis)
+        assert got.dtype == np.int64 and got.shape == want.shape, name
+        assert np.array_equal(np.asarray(got), want), name
+
+
+def test_lexsort_large_rows_and_global_path():
+    """Keys long enough for the global radix path, 1-D and along the first axis."""
+    from oracle import sort_oracle as oracle
+
+    rng = np.random.default_rng(5)
+    n = 300_000
+    k1 = rng.integers(0, 1000, n).astype(np.int32)
+    k2 = rng.integers(0, 50, n).astype(np.float64)
+    k3 = rng.integers(0, 7, n).astype(np.uint8)
+    got = np.asarray(num.lexsort((num.array(k1), num.array(k2), num.array(k3))))
+    assert np.array_equal(got, oracle.lexsort((k1, k2, k3), threads=8))
+    a = rng.integers(0, 5, (20_000, 6)).astype(np.int16)
+    b = rng.integers(0, 5, (20_000, 6)).astype(np.float32)
+    got = np.asarray(num.lexsort((num.array(a), num.array(b)), axis=0))
+    assert np.array_equal(got, np.lexsort((a, b), axis=0))
+
+
+def test_take_along_last_axis_bounds():
+    a = num.array(np.arange(12, dtype=np.float32).reshape(3, 4))
+    idx = num.array(np.array([[0, -1], [3, 1], [-4, 2]], dtype=np.int64))
+    got = a._thunk.take_along_last_axis(idx._thunk)
+    assert np.array_equal(got.__numpy_array__(), np.take_along_axis(np.asarray(a), np.asarray(idx), axis=-1))
+    bad = num.array(np.array([[0, 4], [0, 0], [0, 0]], dtype=np.int64))
+    with pytest.raises(IndexError):
+        a._thunk.take_along_last_axis(bad._thunk)
