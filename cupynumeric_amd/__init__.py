@@ -19,7 +19,7 @@ from ._array import convert_to_ndarray, ndarray
 from ._thunk import SUPPORTED_DTYPES, DeviceArray, check_dtype
 
 __all__ = [
-    "ndarray", "array", "asarray", "sort", "argsort", "sort_complex", "partition", "argpartition", "lexsort", "random",
+    "ndarray", "array", "asarray", "sort", "argsort", "sort_complex", "partition", "argpartition", "lexsort", "searchsorted", "unique", "random",
     "SUPPORTED_DTYPES",
 ]
 
@@ -152,6 +152,32 @@ def lexsort(keys: Any, axis: int | None = -1) -> ndarray:
 
     thunk = lexsort_deferred([k._thunk for k in key_list], axis)
     return ndarray(thunk.shape, np.int64, thunk=thunk)
+
+
+def searchsorted(a: Any, v: Any, side: str = "left", sorter: Any = None) -> ndarray:
+    """Indices at which `v` would be inserted into the sorted 1-D array `a` keeping it sorted
+    (`cupynumeric/_module/ssc_searching.py:31-68`).  `a` must be an array object
+    (the reference calls `a.searchsorted`, so `None` fails with AttributeError there too)."""
+    if not isinstance(a, ndarray):
+        if a is None:
+            raise AttributeError("'NoneType' object has no attribute 'searchsorted'")
+        a = convert_to_ndarray(a)
+    return a.searchsorted(v, side, sorter)
+
+
+def unique(
+    ar: Any,
+    return_index: bool = False,
+    return_inverse: bool = False,
+    return_counts: bool = False,
+    axis: int | None = None,
+) -> ndarray:
+    """Sorted distinct elements of `ar`, flattened (`cupynumeric/_module/sets_making.py:25-122`).
+    The optional outputs and `axis` are not supported, as in the reference."""
+    ar = convert_to_ndarray(ar)
+    if any((return_index, return_inverse, return_counts)) or axis is not None:
+        raise NotImplementedError("Keyword arguments for `unique` are not yet supported")
+    return ar.unique()
 
 
 def _split_first_axis(a: ndarray) -> list[ndarray]:

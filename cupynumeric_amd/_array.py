@@ -110,6 +110,59 @@ class ndarray:
         _adopt_shape(result, self, axis)
         return result
 
+    def astype(self, dtype: Any) -> "ndarray":
+        """Copy of the array cast to `dtype` (`cupynumeric/_array/array.py:2277-2343`, default casting)."""
+        dtype = check_dtype(dtype)
+        if dtype == self.dtype:
+            return self
+        thunk = self._thunk.astype(dtype)
+        return ndarray(thunk.shape, thunk.dtype, thunk=thunk)
+
+    def take_1d(self, indices: "ndarray") -> "ndarray":
+        """`a.take(indices)` for 1-D `a` and 1-D integer `indices`: what `searchsorted` does with
+        its `sorter` (`cupynumeric/_array/array.py:3766`)."""
+        idx = indices if indices.dtype == np.dtype(np.int64) else indices.astype(np.int64)
+        thunk = self._thunk.take_along_last_axis(idx._thunk)
+        return ndarray(thunk.shape, thunk.dtype, thunk=thunk)
+
+    def searchsorted(self, v: Any, side: str = "left", sorter: Any = None) -> "ndarray":
+        """a.searchsorted(v, side='left', sorter=None) (`cupynumeric/_array/array.py:3700-3771`):
+        insertion points of `v` into the sorted 1-D array; int64, shape of `v`."""
+        if self.ndim != 1:
+            raise ValueError("Dimension mismatch: self must be a 1D array")
+
+        # this is needed in case v is a scalar
+        v_ndarray = convert_to_ndarray(v)
+
+        a = self
+        # in case we have different dtypes we need to find a common type
+        if a.dtype != v_ndarray.dtype:
+            ch_dtype = np.result_type(a.dtype, v_ndarray.dtype)
+
+            if v_ndarray.dtype != ch_dtype:
+                v_ndarray = v_ndarray.astype(ch_dtype)
+            if a.dtype != ch_dtype:
+                a = a.astype(ch_dtype)
+
+        if sorter is not None and a.shape[0] > 1:
+            sorter = convert_to_ndarray(sorter)
+            if sorter.ndim != 1:
+                raise ValueError("Dimension mismatch: sorter must be a 1D array")
+            if sorter.shape != a.shape:
+                raise ValueError("Shape mismatch: sorter must have the same shape as self")
+            if not np.issubdtype(sorter.dtype, np.integer):
+                raise ValueError("Dtype mismatch: sorter must be of integer type")
+            a = a.take_1d(sorter)
+
+        result = ndarray(v_ndarray.shape, np.int64)
+        result._thunk.searchsorted(a._thunk, v_ndarray._thunk, side)
+        return result
+
+    def unique(self) -> "ndarray":
+        """a.unique(): sorted distinct values of the flattened array (`cupynumeric/_array/array.py:4208-4227`)."""
+        thunk = self._thunk.unique()
+        return ndarray(thunk.shape, thunk.dtype, thunk=thunk)
+
     def astype_complex(self, dtype: Any) -> "ndarray":
         """Real -> complex64/complex128 copy (the cast `sort_complex` needs)."""
         thunk = self._thunk.to_complex(dtype)

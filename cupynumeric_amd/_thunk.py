@@ -218,6 +218,71 @@ class DeviceArray:
         # fallback to sort for now
         sort_deferred(self, rhs, argpartition, axis, False)
 
+    def astype(self, dtype: Any) -> "DeviceArray":
+        """Dense copy converted to `dtype` (`DeferredArray.convert`, `cupynumeric/_thunk/deferred.py:1899-1937`,
+        a UNARY_OP convert task in the reference)."""
+        dt = check_dtype(dtype)
+        out = DeviceArray(self.shape, dt)
+        if self.size == 0:
+            return out
+        lib = _lib.load()
+        status = lib.cpn_astype(
+            _lib.DTYPE_CODES[self.dtype],
+            self.base.ptr(),
+            _lib.DTYPE_CODES[dt],
+            out.base.ptr(),
+            self.size,
+            ctypes.c_void_p(runtime.stream_handle()),
+        )
+        _lib.check(status, "cpn_astype")
+        return out
+
+    def searchsorted(self, rhs: "DeviceArray", v: "DeviceArray", side: str = "left") -> None:
+        """`DeferredArray.searchsorted` (`cupynumeric/_thunk/deferred.py:5425-5451`): `self` (int64,
+        shape of `v`) receives the insertion points of `v` into the sorted 1-D `rhs`.  Any
+        `side` other than "left" means "right", as in the reference (`is_left = side == "left"`)."""
+        is_left = side == "left"
+        if v.size == 0:
+            return
+        if rhs.dtype != v.dtype or self.dtype != np.dtype(np.int64):
+            raise TypeError("searchsorted: arrays must share one dtype and the result must be int64")
+        lib = _lib.load()
+        status = lib.cpn_searchsorted(
+            _lib.DTYPE_CODES[rhs.dtype],
+            rhs.base.ptr() if rhs.size else None,
+            rhs.size,
+            v.base.ptr(),
+            v.size,
+            int(is_left),
+            self.base.ptr(),
+            ctypes.c_void_p(runtime.stream_handle()),
+        )
+        _lib.check(status, "cpn_searchsorted")
+
+    def unique(self) -> "DeviceArray":
+        """`DeferredArray.unique` (`cupynumeric/_thunk/deferred.py:5375-5395`): sorted distinct
+        values of the flattened array.  The result size is only known on the device (an unbound
+        store in the reference); reading it back is the one synchronisation of this call."""
+        if self.size == 0:
+            return DeviceArray((0,), self.dtype)
+        lib = _lib.load()
+        code = _lib.DTYPE_CODES[self.dtype]
+        temp_bytes = lib.cpn_unique_temp_bytes(code, self.size)
+        if temp_bytes == 0:
+            raise NotImplementedError(f"cpn_unique: no workspace layout for dtype={self.dtype}, size={self.size}")
+        temp = runtime.empty_bytes(temp_bytes)
+        out = DeviceArray((self.size,), self.dtype)
+        count = runtime.torch.zeros(1, dtype=runtime.torch.int64, device=runtime.require_device())
+        stream = ctypes.c_void_p(runtime.stream_handle())
+        status = lib.cpn_unique(
+            code, self.base.ptr(), out.base.ptr(), self.size, count.data_ptr(), temp.data_ptr(), temp_bytes, stream
+        )
+        _lib.check(status, "cpn_unique")
+        if runtime.check_status:
+            _lib.check(lib.cpn_local_sort_check(temp.data_ptr(), stream), "cpn_unique")
+        n_unique = int(count.item())
+        return DeviceArray((n_unique,), self.dtype, out.base)
+
     def to_complex(self, dtype: Any) -> "DeviceArray":
         """Real -> complex cast (`astype` in `sort_complex`, `cupynumeric/_module/ssc_sorting.py:150-159`)."""
         dt = check_dtype(dtype)

@@ -26,6 +26,8 @@ SOURCES = [
     "profile.hip",
     "convert.hip",
     "gather.hip",
+    "searchsorted.hip",
+    "unique.hip",
     "sort_keys8.hip",
     "sort_keys16.hip",
     "sort_keys32.hip",

@@ -45,32 +45,6 @@ uint64_t lds_row_limit(int key_bytes)
   return cap;
 }
 
-struct KeyKind {
-  int bytes;  // 0 = unknown code
-  int codec;  // -1 = known but unsupported
-};
-
-static KeyKind key_kind(int dtype)
-{
-  switch (dtype) {
-    case CPN_BOOL: return {1, CODEC_UNSIGNED};
-    case CPN_INT8: return {1, CODEC_SIGNED};
-    case CPN_INT16: return {2, CODEC_SIGNED};
-    case CPN_INT32: return {4, CODEC_SIGNED};
-    case CPN_INT64: return {8, CODEC_SIGNED};
-    case CPN_UINT8: return {1, CODEC_UNSIGNED};
-    case CPN_UINT16: return {2, CODEC_UNSIGNED};
-    case CPN_UINT32: return {4, CODEC_UNSIGNED};
-    case CPN_UINT64: return {8, CODEC_UNSIGNED};
-    case CPN_FLOAT16: return {2, CODEC_FLOAT};
-    case CPN_FLOAT32: return {4, CODEC_FLOAT};
-    case CPN_FLOAT64: return {8, CODEC_FLOAT};
-    case CPN_COMPLEX64: return {8, CODEC_COMPLEX};
-    case CPN_COMPLEX128: return {16, CODEC_COMPLEX};
-    default: return {0, -1};
-  }
-}
-
 }  // namespace cpn
 
 extern "C" {

@@ -163,6 +163,41 @@ int cpn_real_to_complex(int src_dtype, const void* in, int dst_dtype, void* out,
                         void* stream);
 
 /*
+ * out[i] = (dst type) in[i] for `volume` elements; any of the 14 element types to any other.
+ * Conversions follow C++ static_cast (float16 goes through float32), bool results are
+ * `x != 0`, complex -> real keeps the real part.  Used for the `astype` to the common type
+ * that searchsorted applies to its two arguments (cupynumeric/_array/array.py:3743-3751); a
+ * UNARY_OP convert task in the reference (src/cupynumeric/unary/convert.cu).
+ */
+int cpn_astype(int src_dtype, const void* in, int dst_dtype, void* out, uint64_t volume, void* stream);
+
+/*
+ * positions_out[i] = where values[i] would be inserted into the ascending array `sorted` of n
+ * elements: the first position whose element is not less than the value (left != 0, NumPy
+ * side='left') or the first position whose element is greater (left == 0, side='right').
+ * Both arrays have element type `dtype`; the order is the one cpn_local_sort produces.
+ * Replaces SearchSortedTask::gpu_variant (src/cupynumeric/sort/searchsorted.cu:27-116,
+ * cupynumeric/_thunk/deferred.py:5425-5451) for a sorted array held by one GPU.
+ */
+int cpn_searchsorted(int dtype, const void* sorted, uint64_t n, const void* values,
+                     uint64_t num_values, int left, int64_t* positions_out, void* stream);
+
+/*
+ * Sorted distinct values.  values_out has room for `volume` elements and receives the
+ * distinct values in ascending order (the first of every run of equal keys in the stable
+ * sorted order: all NaNs count as one value, -0.0 and +0.0 as one); *count_out (device
+ * memory, 8-byte aligned) receives how many there are.  `temp` is a 256-byte aligned
+ * workspace of at least cpn_unique_temp_bytes(dtype, volume) bytes; the device status word of
+ * the sort is at its start, so cpn_local_sort_check(temp, stream) applies.  values_in is not
+ * modified.  Replaces UniqueTask::gpu_variant on one processor
+ * (src/cupynumeric/set/unique.cu:137-204, cupynumeric/_thunk/deferred.py:5375-5395).
+ * cpn_unique_temp_bytes returns 0 for an unknown dtype.
+ */
+uint64_t cpn_unique_temp_bytes(int dtype, uint64_t volume);
+int cpn_unique(int dtype, const void* values_in, void* values_out, uint64_t volume,
+               uint64_t* count_out, void* temp, uint64_t temp_bytes, void* stream);
+
+/*
  * out[r][j] = src[r][indices[r][j]] for `rows` dense rows: src rows hold src_seg elements of
  * elem_bytes (1, 2, 4, 8 or 16) bytes, indices and out rows hold idx_seg elements.  Indices are
  * int64, negative ones count from the end of the row.  An index outside [-src_seg, src_seg)

@@ -15,6 +15,12 @@ Two layers, mirroring the reference:
 * `lexsort` restates the loop of `cupynumeric/_module/ssc_sorting.py:271-444` over `argsort`
   above, with NumPy's `take_along_axis` between the steps.
 
+* `searchsorted` restates `cupynumeric/_array/array.py:3700-3771` (common type, `sorter`) over the
+  binary searches of `src/cupynumeric/sort/searchsorted.cc` (lower / upper bound per value);
+  `unique` restates `src/cupynumeric/set/unique.cc:31-55` (copy, sort, drop repeated neighbours).
+  Both use NumPy's order and equality (NaN last and equal to itself) where the reference's
+  backends compare with `<` / `==`.
+
 Deviation kept on purpose (same as the product): results are always stable.
 """
 from __future__ import annotations
@@ -186,3 +192,81 @@ def lexsort(keys, axis=-1, threads: int = 1) -> np.ndarray:
         order = argsort(key_reordered, axis=axis, kind="stable", threads=threads)
         indices = np.take_along_axis(indices, order, axis=axis)
     return indices
+
+
+def _less(a, b) -> bool:
+    """NumPy's sort order for one pair of scalars (npysort_common.h: FLOAT_LT, CFLOAT_LT)."""
+    if isinstance(a, (complex, np.complexfloating)):
+        ar, ai, br, bi = a.real, a.imag, b.real, b.imag
+        if ar < br:
+            return ai == ai or bi != bi
+        if ar > br:
+            return bi != bi and ai == ai
+        if ar == br or (ar != ar and br != br):
+            return ai < bi or (bi != bi and ai == ai)
+        return br != br
+    if isinstance(a, (float, np.floating)):
+        return bool(a < b or (b != b and a == a))
+    return bool(a < b)
+
+
+def searchsorted(a, v, side="left", sorter=None) -> np.ndarray:
+    """`ndarray.searchsorted` (`cupynumeric/_array/array.py:3737-3771`) with one binary search per
+    value (`src/cupynumeric/sort/searchsorted.cc:45-70`: std::lower_bound / std::upper_bound).
+    Pure-Python loops: for small inputs."""
+    a = np.asarray(a)
+    if a.ndim != 1:
+        raise ValueError("Dimension mismatch: self must be a 1D array")
+    v = np.asarray(v)
+    for x in (a, v):
+        if x.dtype not in DTYPE_CODES:
+            raise TypeError(f"cuPyNumeric does not support dtype={x.dtype}")
+    if a.dtype != v.dtype:
+        ch_dtype = np.result_type(a.dtype, v.dtype)
+        v = v.astype(ch_dtype)
+        a = a.astype(ch_dtype)
+    if sorter is not None and a.shape[0] > 1:
+        sorter = np.asarray(sorter)
+        if sorter.ndim != 1:
+            raise ValueError("Dimension mismatch: sorter must be a 1D array")
+        if sorter.shape != a.shape:
+            raise ValueError("Shape mismatch: sorter must have the same shape as self")
+        if not np.issubdtype(sorter.dtype, np.integer):
+            raise ValueError("Dtype mismatch: sorter must be of integer type")
+        a = a.take(sorter).copy()
+    is_left = side == "left"
+    out = np.empty(v.shape, dtype=np.int64)
+    flat_v = v.reshape(-1)
+    flat_o = out.reshape(-1)
+    for i in range(flat_v.size):
+        x = flat_v[i]
+        lo, hi = 0, a.shape[0]
+        while lo < hi:
+            mid = (lo + hi) // 2
+            right = _less(a[mid], x) if is_left else not _less(x, a[mid])
+            if right:
+                lo = mid + 1
+            else:
+                hi = mid
+        flat_o[i] = lo
+    return out
+
+
+def unique(ar, threads: int = 1) -> np.ndarray:
+    """`UniqueImplBody<CPU>` (`src/cupynumeric/set/unique.cc:31-55`): flatten, sort, keep the first
+    of every run of equal neighbours.  Equality is NumPy's for `unique`: NaNs are equal, complex
+    numbers with a NaN part are all equal."""
+    x = np.asarray(ar)
+    if x.dtype not in DTYPE_CODES:
+        raise TypeError(f"cuPyNumeric does not support dtype={x.dtype}")
+    flat = np.ascontiguousarray(x.reshape(-1))
+    if flat.size == 0:
+        return flat.copy()
+    s = local_sort(flat, argsort=False, stable=True, threads=threads)
+    with np.errstate(invalid="ignore"):
+        differ = s[1:] != s[:-1]
+    if s.dtype.kind in "fc":
+        nan = np.isnan(s)
+        differ &= ~(nan[1:] & nan[:-1])
+    keep = np.concatenate(([True], differ))
+    return s[keep]

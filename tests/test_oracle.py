@@ -220,3 +220,65 @@ def test_lexsort_errors():
         oracle.lexsort((np.arange(3), np.arange(3)), axis=None)
     with pytest.raises(TypeError, match="cuPyNumeric does not support dtype"):
         oracle.lexsort((("Heinrich", "Galileo", "Gustav"), ("Hertz", "Galilei", "Hertz")))
+
+
+# ---- searchsorted / unique ---------------------------------------------------------------------------
+def _consumer_inputs(dt, size, rng):
+    if np.dtype(dt).kind == "c":
+        a = (rng.integers(0, 5, size) + 1j * rng.integers(0, 5, size)).astype(dt)
+        if size > 4:
+            a[::7] = complex(np.nan, 1)
+            a[3] = complex(2, np.nan)
+            a[4] = complex(np.nan, np.nan)
+        v = (rng.integers(-1, 6, 31) + 1j * rng.integers(-1, 6, 31)).astype(dt)
+        v[5] = complex(np.nan, 0)
+        v[6] = complex(1, np.nan)
+    elif np.dtype(dt).kind == "f":
+        a = np.round(rng.standard_normal(size) * 3).astype(dt)
+        if size > 4:
+            a[::5] = np.nan
+            a[1], a[2], a[3] = -0.0, 0.0, np.inf
+        v = np.round(rng.standard_normal(31) * 3).astype(dt)
+        v[3], v[4], v[5] = np.nan, -0.0, -np.inf
+    else:
+        hi = 2 if dt == np.bool_ else 50
+        a = rng.integers(0, hi, size).astype(dt)
+        v = rng.integers(0, hi + (0 if dt == np.bool_ else 10), 31).astype(dt)
+    return a, v
+
+
+@pytest.mark.parametrize("dtype", ALL_REAL_DTYPES + COMPLEX_DTYPES)
+def test_searchsorted_and_unique_match_numpy(dtype):
+    """NumPy's own searchsorted / unique are the independent statement of the contract (NaN last and
+    equal to itself, complex values with a NaN part one value for unique)."""
+    rng = np.random.default_rng(np.dtype(dtype).num)
+    for size in (0, 1, 2, 17, 200):
+        a, v = _consumer_inputs(dtype, size, rng)
+        srt = np.sort(a, kind="stable")
+        order = np.argsort(a, kind="stable")
+        for side in ("left", "right"):
+            assert np.array_equal(oracle.searchsorted(srt, v, side), np.searchsorted(srt, v, side))
+            v2 = v.reshape(-1, 1)
+            assert np.array_equal(
+                oracle.searchsorted(a, v2, side, sorter=order), np.searchsorted(a, v2, side, sorter=order)
+            )
+        # (float16 through float32, exact: NumPy 2.2.6's default float16 sort mis-sorts -0.0 on AVX-512)
+        u, w = oracle.unique(a), (np.unique(a.astype(np.float32)).astype(a.dtype) if a.dtype == np.float16 else np.unique(a))
+        assert u.dtype == w.dtype and u.shape == w.shape and np.array_equal(u, w, equal_nan=True)
+
+
+def test_searchsorted_common_type_and_errors():
+    # tests/integration/test_searchsorted.py:46-53 (dtype pairs), :79-128 (errors)
+    rng = np.random.default_rng(3)
+    for n, d1, d2 in [(3, np.uint64, np.float32), (51, np.uint32, np.complex64), (23, np.uint32, np.float64),
+                      (51, np.complex64, np.float64), (21, np.complex64, np.int32), (22, np.complex128, np.float32)]:
+        a = np.sort((rng.random(n) * 100).astype(d1))
+        v = (rng.random(10) * 100).astype(d2)
+        for side in ("left", "right"):
+            assert np.array_equal(oracle.searchsorted(a, v, side), np.searchsorted(a, v, side))
+    with pytest.raises(ValueError):
+        oracle.searchsorted(rng.random((5, 5, 5)), 5)
+    with pytest.raises(ValueError):
+        oracle.searchsorted(np.arange(100), np.arange(10), sorter=np.arange(10))
+    with pytest.raises(TypeError):
+        oracle.searchsorted([2, 3, 10, 9], None)
