@@ -248,13 +248,235 @@ def cpu_baseline(cfg: dict) -> dict:
     }
 
 
+
+# -------------------------------------------------------------------------------------------------
+# callers and consumers of the sort path: lexsort, searchsorted, unique
+# -------------------------------------------------------------------------------------------------
+class LexsortJob:
+    """np.lexsort((k0, k1)): int32 secondary key with 1000 distinct values, float32 primary key with
+    about 2^16 distinct values.  argsort(k0) -> gather k1 -> argsort -> gather the indices."""
+
+    name = "lexsort"
+
+    def __init__(self, torch, lib, log2n):
+        n = 1 << (26 if log2n is None else log2n)
+        rng = np.random.default_rng(5)
+        self.k0 = rng.integers(0, 1000, n).astype(np.int32)
+        self.k1 = np.round(rng.standard_normal(n, dtype=np.float32) * 8192).astype(np.float32)
+        self.n = n
+        self.workload = f"lexsort((int32 1000 distinct, float32 ~2^16 distinct)) N=2^{int(np.log2(n))}, seed 5"
+        dev = "cuda:0"
+        self.torch, self.lib = torch, lib
+        self.d_k0 = torch.from_numpy(self.k0).to(dev)
+        self.d_k1 = torch.from_numpy(self.k1).to(dev)
+        self.d_k1r = torch.empty_like(self.d_k1)
+        self.d_idx = torch.empty(n, dtype=torch.int64, device=dev)
+        self.d_ord = torch.empty(n, dtype=torch.int64, device=dev)
+        self.d_out = torch.empty(n, dtype=torch.int64, device=dev)
+        self.tb = max(lib.cpn_local_sort_temp_bytes(3, n, n, 0, 1, 0), lib.cpn_local_sort_temp_bytes(10, n, n, 0, 1, 0))
+        self.temp = torch.empty(self.tb, dtype=torch.uint8, device=dev)
+        self.stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        # argsort int32 (4 passes) + gather 4-byte + argsort float32 + gather 8-byte
+        sort_bytes = lambda kb: n * (kb + (kb + kb + 4) + 2 * (kb + 4 + kb + 4) + (kb + 4 + 8))
+        self.alg = {"total": sort_bytes(4) * 2 + n * (8 + 4 + 4) + n * (8 + 8 + 8),
+                    "onesweep": n * ((4 + 8) + 2 * 16 + 16) / 4, "take_last_axis": n * 20}
+        self.dominant = "onesweep"
+        self.dtype = "u32"
+
+    def step(self):
+        lib, n, s = self.lib, self.n, self.stream
+        rc = lib.cpn_local_sort(3, self.d_k0.data_ptr(), None, self.d_idx.data_ptr(), n, n, 0, 1, self.temp.data_ptr(), self.tb, s)
+        rc |= lib.cpn_take_along_last_axis(4, self.d_k1.data_ptr(), self.d_idx.data_ptr(), self.d_k1r.data_ptr(), 1, n, n, None, s)
+        rc |= lib.cpn_local_sort(10, self.d_k1r.data_ptr(), None, self.d_ord.data_ptr(), n, n, 0, 1, self.temp.data_ptr(), self.tb, s)
+        rc |= lib.cpn_take_along_last_axis(8, self.d_idx.data_ptr(), self.d_ord.data_ptr(), self.d_out.data_ptr(), 1, n, n, None, s)
+        assert rc == 0, rc
+
+    def verify(self):
+        m = min(self.n, 1 << 22)  # a prefix is not a sub-problem of lexsort: check the properties instead
+        idx = self.d_out
+        a0, a1 = self.d_k0[idx], self.d_k1[idx]
+        ordered = bool(((a1[:-1] < a1[1:]) | ((a1[:-1] == a1[1:]) & (a0[:-1] <= a0[1:]))).all())
+        tie = (a1[:-1] == a1[1:]) & (a0[:-1] == a0[1:])
+        stable = bool((idx[1:][tie] > idx[:-1][tie]).all())
+        seen = self.torch.zeros(self.n, dtype=self.torch.bool, device=idx.device)
+        seen[idx] = True
+        del m
+        return "ok" if ordered and stable and bool(seen.all()) else "FAILED"
+
+    def cpu(self, oracle, threads):
+        m = min(self.n, 1 << 24)
+        t0 = time.perf_counter()
+        oracle.lexsort((self.k0[:m], self.k1[:m]), threads=threads)
+        return m, time.perf_counter() - t0, f"first 2^{int(np.log2(m))} elements of both keys; oracle.lexsort over oracle/sort_oracle.c"
+
+
+class SearchsortedJob:
+    """np.searchsorted(a, v, 'left'): a = 2^28 sorted float32, v = 2^24 float32 drawn from the same law."""
+
+    name = "searchsorted"
+
+    def __init__(self, torch, lib, log2n):
+        n = 1 << (28 if log2n is None else log2n)
+        m = max(n >> 4, 1)
+        rng = np.random.default_rng(6)
+        self.v = rng.standard_normal(m, dtype=np.float32)
+        self.n, self.m = n, m
+        self.workload = (f"searchsorted(sorted float32 N=2^{int(np.log2(n))}, float32 values M=2^{int(np.log2(m))}, "
+                         "side=left), normal, seed 6")
+        dev = "cuda:0"
+        self.torch, self.lib = torch, lib
+        g = torch.Generator(device=dev)
+        g.manual_seed(6)
+        self.d_a = torch.randn(n, dtype=torch.float32, device=dev, generator=g).sort().values  # input preparation only
+        self.d_v = torch.from_numpy(self.v).to(dev)
+        self.d_out = torch.empty(m, dtype=torch.int64, device=dev)
+        self.stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        self.alg = {"total": m * (4 + 8), "searchsorted": m * (4 + 8)}
+        self.dominant = "searchsorted"
+        self.dtype = "u32"
+        self.n_keys = m
+
+    def step(self):
+        rc = self.lib.cpn_searchsorted(10, self.d_a.data_ptr(), self.n, self.d_v.data_ptr(), self.m, 1,
+                                       self.d_out.data_ptr(), self.stream)
+        assert rc == 0, rc
+
+    def verify(self):
+        p = self.d_out
+        a, v = self.d_a, self.d_v
+        n = self.n
+        right_ok = (p == n) | (a[p.clamp(max=n - 1)] >= v)
+        left_ok = (p == 0) | (a[(p - 1).clamp(min=0)] < v)
+        return "ok" if bool((right_ok & left_ok).all()) else "FAILED"
+
+    def cpu(self, oracle, threads):
+        a = self.d_a[: min(self.n, 1 << 26)].cpu().numpy()
+        t0 = time.perf_counter()
+        np.searchsorted(a, self.v, side="left")
+        return self.m, time.perf_counter() - t0, (f"all {self.m} values against the first 2^{int(np.log2(a.size))} sorted elements; "
+                                                  "numpy.searchsorted on one core (the oracle's own search is a Python loop)")
+
+
+class UniqueJob:
+    """np.unique(x): int32, 2^26 elements, about 2^20 distinct values."""
+
+    name = "unique"
+
+    def __init__(self, torch, lib, log2n):
+        n = 1 << (26 if log2n is None else log2n)
+        rng = np.random.default_rng(7)
+        self.x = rng.integers(0, max(n >> 6, 2), n).astype(np.int32)
+        self.n = n
+        self.workload = f"unique(int32 N=2^{int(np.log2(n))}, values below N/64), seed 7"
+        dev = "cuda:0"
+        self.torch, self.lib = torch, lib
+        self.d_in = torch.from_numpy(self.x).to(dev)
+        self.d_out = torch.empty_like(self.d_in)
+        self.count = torch.zeros(1, dtype=torch.int64, device=dev)
+        self.tb = lib.cpn_unique_temp_bytes(3, n)
+        self.temp = torch.empty(self.tb, dtype=torch.uint8, device=dev)
+        self.stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        distinct = min(n, max(n >> 6, 2))
+        self.alg = {"total": n * 4 + 4 * n * 8 + 2 * n * 4 + distinct * 4, "onesweep": n * 8,
+                    "unique_count": n * 4, "unique_scatter": n * 4 + distinct * 4, "histogram": n * 4}
+        self.dominant = "onesweep"
+        self.dtype = "u32"
+
+    def step(self):
+        rc = self.lib.cpn_unique(3, self.d_in.data_ptr(), self.d_out.data_ptr(), self.n, self.count.data_ptr(),
+                                 self.temp.data_ptr(), self.tb, self.stream)
+        assert rc == 0, rc
+
+    def verify(self):
+        c = int(self.count.item())
+        u = self.d_out[:c]
+        strictly = bool((u[1:] > u[:-1]).all())
+        present = self.torch.zeros(max(self.n >> 6, 2), dtype=self.torch.bool, device=u.device)
+        present[self.d_in.long()] = True
+        return "ok" if strictly and c == int(present.sum()) and bool(present[u.long()].all()) else "FAILED"
+
+    def cpu(self, oracle, threads):
+        t0 = time.perf_counter()
+        oracle.unique(self.x, threads=threads)
+        return self.n, time.perf_counter() - t0, "the whole workload; oracle.unique over oracle/sort_oracle.c"
+
+
+CONSUMERS = {"lexsort": LexsortJob, "searchsorted": SearchsortedJob, "unique": UniqueJob}
+
+
+def run_consumer(args) -> dict:
+    import torch
+
+    from cupynumeric_amd import _lib
+
+    if not torch.cuda.is_available():
+        raise RuntimeError("bench.py needs a HIP device")
+    lib = _lib.load()
+    job = CONSUMERS[args.config](torch, lib, args.log2n)
+    for _ in range(args.warmup):
+        job.step()
+    torch.cuda.synchronize()
+    lib.cpn_profile_enable(1)
+    _lib.profile_collect()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        job.step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    lib.cpn_profile_enable(0)
+    by_label: dict[str, list[float]] = {}
+    for label, ms in _lib.profile_collect():
+        by_label.setdefault(label, []).append(ms)
+    n_keys = getattr(job, "n_keys", job.n)
+    step_s = elapsed / args.steps
+    dom = job.dominant
+    avg_ms = float(np.mean(by_label[dom]))
+    achieved = job.alg[dom] / (avg_ms * 1e-3)
+    line = {
+        "metric": f"elements/sec, {job.name}, 1 GPU",
+        "value": n_keys / step_s,
+        "unit": "keys/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": step_s * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": job.dtype,
+        "data": "synthetic",
+        "config": {"workload": job.workload, "keys": int(n_keys), "op": job.name},
+        "roofline": {"kernel": dom, "bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_PEAK_BYTES_PER_S / 1e9,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_BYTES_PER_S, "traffic": None,
+                     "bytes_per_launch": job.alg[dom], "avg_launch_ms": avg_ms,
+                     "launches_per_step": len(by_label[dom]) / args.steps},
+        "whole_step": {"algorithmic_bytes": job.alg["total"], "GBps": job.alg["total"] / step_s / 1e9,
+                       "frac_of_hbm_peak": job.alg["total"] / step_s / HBM_PEAK_BYTES_PER_S},
+        "kernels": {label: {"launches_per_step": len(v) / args.steps, "avg_ms": float(np.mean(v))}
+                    for label, v in by_label.items()},
+        "verify": job.verify(),
+    }
+    if not args.no_cpu_baseline:
+        from oracle import sort_oracle as oracle
+
+        threads = min(oracle.max_threads(), os.cpu_count() or 1, 16)
+        count, dt, what = job.cpu(oracle, threads)
+        line["cpu_baseline"] = {"value": count / dt, "unit": "keys/s", "cores": 1 if job.name == "searchsorted" else threads,
+                                "kind": "port", "sample": f"{what}, {dt:.2f} s"}
+    return line
+
+
 # -------------------------------------------------------------------------------------------------
 def main() -> None:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--config", default="c2",
+                    choices=["c1", "c2", "c3", "c4", "c5", "lexsort", "searchsorted", "unique"],
+                    help="c1..c5: the sort workloads of the baseline; lexsort / searchsorted / unique: the "
+                         "callers and consumers of the sort path, on workloads of this file's own choosing")
     ap.add_argument("--log2n", type=int, default=None, help="shrink a 1-D workload to 2^L keys")
     ap.add_argument("--rows", type=int, default=None, help="shrink a 2-D workload to this many rows")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -264,6 +486,10 @@ def main() -> None:
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build sorts on one GPU; --gpus must be 1 (no multi-GPU sample sort is built)")
+
+    if args.config in CONSUMERS:
+        print(json.dumps(run_consumer(args)))
+        return
 
     cfg = make_config(args.config, args.log2n, args.rows)
     job = GpuJob(cfg)
