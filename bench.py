@@ -254,7 +254,7 @@ def cpu_baseline(cfg: dict) -> dict:
 # -------------------------------------------------------------------------------------------------
 class LexsortJob:
     """np.lexsort((k0, k1)): int32 secondary key with 1000 distinct values, float32 primary key with
-    about 2^16 distinct values.  argsort(k0) -> gather k1 -> argsort -> gather the indices."""
+    about 2^16 distinct values.  Both keys packed into one 64-bit word per element, one argsort."""
 
     name = "lexsort"
 
@@ -269,30 +269,28 @@ class LexsortJob:
         self.torch, self.lib = torch, lib
         self.d_k0 = torch.from_numpy(self.k0).to(dev)
         self.d_k1 = torch.from_numpy(self.k1).to(dev)
-        self.d_k1r = torch.empty_like(self.d_k1)
-        self.d_idx = torch.empty(n, dtype=torch.int64, device=dev)
-        self.d_ord = torch.empty(n, dtype=torch.int64, device=dev)
+        self.d_packed = torch.empty(n, dtype=torch.int64, device=dev)
         self.d_out = torch.empty(n, dtype=torch.int64, device=dev)
-        self.tb = max(lib.cpn_local_sort_temp_bytes(3, n, n, 0, 1, 0), lib.cpn_local_sort_temp_bytes(10, n, n, 0, 1, 0))
+        self.tb = lib.cpn_local_sort_temp_bytes(8, n, n, 0, 1, 0)
         self.temp = torch.empty(self.tb, dtype=torch.uint8, device=dev)
         self.stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-        # argsort int32 (4 passes) + gather 4-byte + argsort float32 + gather 8-byte
-        sort_bytes = lambda kb: n * (kb + (kb + kb + 4) + 2 * (kb + 4 + kb + 4) + (kb + 4 + 8))
-        self.alg = {"total": sort_bytes(4) * 2 + n * (8 + 4 + 4) + n * (8 + 8 + 8),
-                    "onesweep": n * ((4 + 8) + 2 * 16 + 16) / 4, "take_last_axis": n * 20}
+        self.dtypes = (ctypes.c_int * 2)(3, 10)
+        self.ptrs = (ctypes.c_void_p * 2)(self.d_k0.data_ptr(), self.d_k1.data_ptr())
+        # pack: read 4+4, write 8; histogram: read 8; the passes that run (digits that vary): first reads
+        # 8 and writes 8+4, middle ones move 8+4 both ways, the last reads 8+4 and writes 8
+        self.alg = {"lexsort_pack": n * 16, "histogram": n * 8, "onesweep": n * 24}
+        self.alg["total"] = None  # filled in from the number of passes that ran
         self.dominant = "onesweep"
-        self.dtype = "u32"
+        self.dtype = "u64"
 
     def step(self):
         lib, n, s = self.lib, self.n, self.stream
-        rc = lib.cpn_local_sort(3, self.d_k0.data_ptr(), None, self.d_idx.data_ptr(), n, n, 0, 1, self.temp.data_ptr(), self.tb, s)
-        rc |= lib.cpn_take_along_last_axis(4, self.d_k1.data_ptr(), self.d_idx.data_ptr(), self.d_k1r.data_ptr(), 1, n, n, None, s)
-        rc |= lib.cpn_local_sort(10, self.d_k1r.data_ptr(), None, self.d_ord.data_ptr(), n, n, 0, 1, self.temp.data_ptr(), self.tb, s)
-        rc |= lib.cpn_take_along_last_axis(8, self.d_idx.data_ptr(), self.d_ord.data_ptr(), self.d_out.data_ptr(), 1, n, n, None, s)
+        rc = lib.cpn_lexsort_pack(2, self.dtypes, self.ptrs, None, 8, self.d_packed.data_ptr(), 1, n, s)
+        rc |= lib.cpn_local_sort(8, self.d_packed.data_ptr(), None, self.d_out.data_ptr(), n, n, 0, 1,
+                                 self.temp.data_ptr(), self.tb, s)
         assert rc == 0, rc
 
     def verify(self):
-        m = min(self.n, 1 << 22)  # a prefix is not a sub-problem of lexsort: check the properties instead
         idx = self.d_out
         a0, a1 = self.d_k0[idx], self.d_k1[idx]
         ordered = bool(((a1[:-1] < a1[1:]) | ((a1[:-1] == a1[1:]) & (a0[:-1] <= a0[1:]))).all())
@@ -300,7 +298,6 @@ class LexsortJob:
         stable = bool((idx[1:][tie] > idx[:-1][tie]).all())
         seen = self.torch.zeros(self.n, dtype=self.torch.bool, device=idx.device)
         seen[idx] = True
-        del m
         return "ok" if ordered and stable and bool(seen.all()) else "FAILED"
 
     def cpu(self, oracle, threads):
@@ -431,6 +428,15 @@ def run_consumer(args) -> dict:
     n_keys = getattr(job, "n_keys", job.n)
     step_s = elapsed / args.steps
     dom = job.dominant
+    if dom == "onesweep":  # launches of skipped passes exit at once: keep the ones that moved data
+        longest = max(by_label[dom])
+        by_label["onesweep_skipped"] = [t for t in by_label[dom] if t < 0.1 * longest]
+        by_label[dom] = [t for t in by_label[dom] if t >= 0.1 * longest]
+        if not by_label["onesweep_skipped"]:
+            del by_label["onesweep_skipped"]
+    if job.alg.get("total") is None:
+        ran = len(by_label["onesweep"]) / args.steps
+        job.alg["total"] = job.alg["lexsort_pack"] + job.alg["histogram"] + ran * job.alg["onesweep"]
     avg_ms = float(np.mean(by_label[dom]))
     achieved = job.alg[dom] / (avg_ms * 1e-3)
     line = {

@@ -67,6 +67,10 @@ PROTOTYPES: dict[str, tuple] = {
     "cpn_take_along_last_axis": (
         c_int, [c_int, c_void_p, c_void_p, c_void_p, c_uint64, c_uint64, c_uint64, c_void_p, c_void_p]
     ),
+    "cpn_lexsort_pack": (
+        c_int,
+        [c_int, ctypes.POINTER(c_int), ctypes.POINTER(c_void_p), c_void_p, c_int, c_void_p, c_uint64, c_uint64, c_void_p],
+    ),
     "cpn_profile_enable": (c_int, [c_int]),
     "cpn_profile_collect": (c_int, [c_void_p, c_uint64, c_void_p, c_int]),
     "cpn_swapaxes_copy": (c_int, [c_int, c_void_p, c_void_p, ctypes.POINTER(c_int64), c_int, c_int, c_int, c_void_p]),

@@ -139,15 +139,69 @@ def sort_deferred(
                 sort_swapped(output, input, argsort, computed_axis, stable)
 
 
+def _pack_keys(group: "list[DeviceArray]", indices: "DeviceArray | None") -> "DeviceArray":
+    """One unsigned word per element holding the keys of `group` (least significant first) as
+    order-preserving images, read through `indices` when given (`cpn_lexsort_pack`)."""
+    import numpy as np
+
+    from ._thunk import DeviceArray
+
+    lib = _lib.load()
+    width = sum(k.dtype.itemsize for k in group)
+    packed_dtype = np.dtype(np.uint32) if width <= 4 else np.dtype(np.uint64)
+    shape = group[0].shape
+    out = DeviceArray(shape, packed_dtype)
+    n = len(group)
+    dtypes = (ctypes.c_int * n)(*[_lib.DTYPE_CODES[k.dtype] for k in group])
+    ptrs = (ctypes.c_void_p * n)(*[k.base.ptr() for k in group])
+    seg = shape[-1]
+    status = lib.cpn_lexsort_pack(
+        n,
+        dtypes,
+        ptrs,
+        indices.base.ptr() if indices is not None else None,
+        packed_dtype.itemsize,
+        out.base.ptr(),
+        out.size // seg,
+        seg,
+        ctypes.c_void_p(runtime.stream_handle()),
+    )
+    _lib.check(status, "cpn_lexsort_pack")
+    return out
+
+
+def _lexsort_groups(keys: "list[DeviceArray]") -> "list[list[DeviceArray]]":
+    """Consecutive real keys whose widths add up to at most 8 bytes (and at most 8 keys) are
+    sorted as one packed key; a complex key, or a real key that would not fit, starts a new
+    group."""
+    groups: list[list] = []
+    width = 0
+    for k in keys:
+        kb = k.dtype.itemsize
+        packable = k.dtype.kind != "c"
+        if groups and packable and groups[-1][0].dtype.kind != "c" and width + kb <= 8 and len(groups[-1]) < 8:
+            groups[-1].append(k)
+            width += kb
+        else:
+            groups.append([k])
+            width = kb if packable else 16
+    return groups
+
+
 def lexsort_deferred(keys: "list[DeviceArray]", axis: int) -> "DeviceArray":
     """The loop of `lexsort` (`cupynumeric/_module/ssc_sorting.py:423-444`): a stable argsort of
     the least significant key, then for every further key: reorder the key by the indices so
     far, argsort it (stable), reorder the indices by that order.  `keys[-1]` is the primary key.
 
+    Two changes of schedule, none of result.  Neighbouring real keys of at most 8 bytes together
+    are packed into one unsigned word and sorted in one argsort (a lexicographic order is the
+    order of the concatenated order-preserving images), and the reordering of the keys of a
+    later group is fused into its packing.  Axes other than the last are moved there once (one
+    transpose per key, one for the result) instead of once per argsort.
+
     Every key is sorted in its own element type under the NumPy order, which already puts
     -inf < finite < +inf < NaN, so the reference's remapping of special float values
-    (`ssc_sorting.py:352-420`) has nothing to do here.  Axes other than the last are moved
-    there once (one transpose per key, one for the result) instead of once per argsort.
+    (`ssc_sorting.py:352-420`) has nothing to do here.
     """
     from ._thunk import DeviceArray
 
@@ -157,13 +211,17 @@ def lexsort_deferred(keys: "list[DeviceArray]", axis: int) -> "DeviceArray":
     if axis != last:
         keys = [k.swapaxes_copy(axis, last) for k in keys]
 
-    indices = DeviceArray(keys[0].shape, dtype="int64")
-    sort_task(indices, keys[0], True, True)
-    for key in keys[1:]:
-        key_reordered = key.take_along_last_axis(indices)
-        order = DeviceArray(key.shape, dtype="int64")
+    indices = None
+    for group in _lexsort_groups(keys):
+        if len(group) == 1 and indices is None:
+            key_reordered = group[0]  # first key: nothing to reorder, no need to pack
+        elif group[0].dtype.kind == "c":
+            key_reordered = group[0].take_along_last_axis(indices)
+        else:
+            key_reordered = _pack_keys(group, indices)
+        order = DeviceArray(key_reordered.shape, dtype="int64")
         sort_task(order, key_reordered, True, True)
-        indices = indices.take_along_last_axis(order)
+        indices = order if indices is None else indices.take_along_last_axis(order)
 
     if axis != last:
         indices = indices.swapaxes_copy(last, axis)

@@ -60,7 +60,132 @@ static int launch_take(const void* src, const int64_t* idx, void* out, uint64_t 
   return CPN_OK;
 }
 
+// ---- lexsort: several keys packed into one ------------------------------------------------
+//
+// A lexicographic order on keys (k_last, ..., k_0) is the order of the unsigned number whose
+// bytes are the order-preserving images of the keys, most significant key on top.  Packing up
+// to 8 bytes of real keys into one word turns the reference's chain of argsort +
+// take_along_axis per key (cupynumeric/_module/ssc_sorting.py:423-444) into one argsort of
+// the packed word; with `indices` the keys are read through the permutation found so far,
+// which is the take_along_axis of the chain fused into the packing.
+constexpr int PACK_MAX_KEYS = 8;
+
+struct PackArgs {
+  const void* key[PACK_MAX_KEYS];
+  int bytes[PACK_MAX_KEYS];
+  int codec[PACK_MAX_KEYS];
+  int shift[PACK_MAX_KEYS];  // bit position of the key inside the packed word
+  int num_keys;
+};
+
+__device__ __forceinline__ uint64_t ordered_image(const void* base, uint64_t i, int bytes, int codec)
+{
+  switch (bytes) {
+    case 1: {
+      const uint8_t raw = static_cast<const uint8_t*>(base)[i];
+      return codec == CODEC_SIGNED ? ordered_bits<CODEC_SIGNED, uint8_t>(raw) : raw;
+    }
+    case 2: {
+      const uint16_t raw = static_cast<const uint16_t*>(base)[i];
+      return codec == CODEC_FLOAT ? ordered_bits<CODEC_FLOAT, uint16_t>(raw)
+                                  : (codec == CODEC_SIGNED ? ordered_bits<CODEC_SIGNED, uint16_t>(raw) : raw);
+    }
+    case 4: {
+      const uint32_t raw = static_cast<const uint32_t*>(base)[i];
+      return codec == CODEC_FLOAT ? ordered_bits<CODEC_FLOAT, uint32_t>(raw)
+                                  : (codec == CODEC_SIGNED ? ordered_bits<CODEC_SIGNED, uint32_t>(raw) : raw);
+    }
+    default: {
+      const uint64_t raw = static_cast<const uint64_t*>(base)[i];
+      return codec == CODEC_FLOAT ? ordered_bits<CODEC_FLOAT, uint64_t>(raw)
+                                  : (codec == CODEC_SIGNED ? ordered_bits<CODEC_SIGNED, uint64_t>(raw) : raw);
+    }
+  }
+}
+
+template <typename OutT>
+__global__ __launch_bounds__(256) void lexsort_pack_kernel(PackArgs a,
+                                                            const int64_t* __restrict__ indices,
+                                                            OutT* __restrict__ out,
+                                                            uint64_t total,
+                                                            uint64_t seg)
+{
+  const uint64_t stride = static_cast<uint64_t>(gridDim.x) * blockDim.x;
+  for (uint64_t o = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x; o < total; o += stride) {
+    uint64_t src = o;
+    if (indices != nullptr) {
+      src = (o / seg) * seg + static_cast<uint64_t>(indices[o]);
+    }
+    uint64_t packed = 0;
+    for (int k = 0; k < a.num_keys; ++k) {
+      packed |= ordered_image(a.key[k], src, a.bytes[k], a.codec[k]) << a.shift[k];
+    }
+    out[o] = static_cast<OutT>(packed);
+  }
+}
+
 }  // namespace cpn
+
+extern "C" int cpn_lexsort_pack(int num_keys, const int* dtypes, const void* const* keys, const int64_t* indices,
+                                int packed_bytes, void* packed_out, uint64_t rows, uint64_t seg, void* stream)
+{
+  using namespace cpn;
+  if (num_keys < 1 || num_keys > PACK_MAX_KEYS || (packed_bytes != 4 && packed_bytes != 8)) {
+    return CPN_ERR_SHAPE;
+  }
+  if (dtypes == nullptr || keys == nullptr) {
+    return CPN_ERR_NULL;
+  }
+  PackArgs a{};
+  a.num_keys = num_keys;
+  int bits   = 0;
+  for (int k = 0; k < num_keys; ++k) {
+    const KeyKind kind = key_kind(dtypes[k]);
+    if (kind.bytes == 0 || kind.codec < 0 || kind.codec == CODEC_COMPLEX) {
+      return CPN_ERR_DTYPE;  // complex keys do not pack: their order needs a ninth byte
+    }
+    if (keys[k] == nullptr && rows * seg != 0) {
+      return CPN_ERR_NULL;
+    }
+    if ((reinterpret_cast<uintptr_t>(keys[k]) % static_cast<uint64_t>(kind.bytes)) != 0) {
+      return CPN_ERR_ALIGN;
+    }
+    a.key[k]   = keys[k];
+    a.bytes[k] = kind.bytes;
+    a.codec[k] = kind.codec;
+    a.shift[k] = bits;
+    bits += 8 * kind.bytes;
+  }
+  if (bits > 8 * packed_bytes) {
+    return CPN_ERR_SHAPE;
+  }
+  const uint64_t total = rows * seg;
+  if (total == 0) {
+    return CPN_OK;
+  }
+  if (packed_out == nullptr) {
+    return CPN_ERR_NULL;
+  }
+  if ((reinterpret_cast<uintptr_t>(packed_out) % static_cast<uint64_t>(packed_bytes)) != 0 ||
+      (reinterpret_cast<uintptr_t>(indices) % 8) != 0) {
+    return CPN_ERR_ALIGN;
+  }
+  uint64_t grid = (total + 255) / 256;
+  if (grid > (1u << 20)) {
+    grid = 1u << 20;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  ProfileScope prof("lexsort_pack", s);
+  if (packed_bytes == 4) {
+    hipLaunchKernelGGL((lexsort_pack_kernel<uint32_t>), dim3(static_cast<uint32_t>(grid)), dim3(256), 0, s, a, indices,
+                       static_cast<uint32_t*>(packed_out), total, seg);
+  } else {
+    hipLaunchKernelGGL((lexsort_pack_kernel<uint64_t>), dim3(static_cast<uint32_t>(grid)), dim3(256), 0, s, a, indices,
+                       static_cast<uint64_t*>(packed_out), total, seg);
+  }
+  CPN_HIP_TRY(hipGetLastError());
+  return CPN_OK;
+}
 
 extern "C" int cpn_take_along_last_axis(int elem_bytes, const void* src, const int64_t* indices, void* out,
                                         uint64_t rows, uint64_t src_seg, uint64_t idx_seg, uint32_t* oob_flag,

@@ -211,6 +211,20 @@ int cpn_take_along_last_axis(int elem_bytes, const void* src, const int64_t* ind
                              void* stream);
 
 /*
+ * Packs num_keys (1..8) real keys of `rows` dense rows of `seg` elements into one unsigned
+ * word per element (packed_bytes = 4 or 8, at least the summed width of the keys):
+ * keys[0] is the least significant key, as in lexsort; each key enters as the
+ * order-preserving unsigned image of its element type, so that the unsigned order of the
+ * packed words is the lexicographic order of the keys under NumPy's rules.  With `indices`
+ * (int64, row relative, may be NULL) element j of a row takes its keys from position
+ * indices[j] of that row.  An argsort of the packed words (dtype CPN_UINT32 / CPN_UINT64)
+ * then replaces the reference's argsort + take_along_axis per key
+ * (cupynumeric/_module/ssc_sorting.py:423-444).  Complex keys return CPN_ERR_DTYPE.
+ */
+int cpn_lexsort_pack(int num_keys, const int* dtypes, const void* const* keys, const int64_t* indices,
+                     int packed_bytes, void* packed_out, uint64_t rows, uint64_t seg, void* stream);
+
+/*
  * Per-launch timing.  cpn_profile_enable(1) makes every kernel launch of the library record
  * a pair of HIP events on the stream it is launched on; it returns the previous setting.
  * cpn_profile_collect waits for the recorded events, writes up to `max_records` entries --

@@ -106,3 +106,40 @@ def test_take_along_last_axis_bounds():
     bad = num.array(np.array([[0, 4], [0, 0], [0, 0]], dtype=np.int64))
     with pytest.raises(IndexError):
         a._thunk.take_along_last_axis(bad._thunk)
+
+
+def test_lexsort_pack_c_abi():
+    """cpn_lexsort_pack directly: the unsigned order of the packed words is the lexicographic order of
+    the keys, with and without reading through a permutation; widths that do not fit are refused."""
+    import ctypes
+
+    import torch
+
+    from cupynumeric_amd import _lib
+
+    lib = _lib.load()
+    dev = torch.device("cuda")
+    rng = np.random.default_rng(8)
+    rows, seg = 3, 1000
+    k0 = rng.integers(-3, 3, (rows, seg)).astype(np.int8)
+    k1 = np.round(rng.standard_normal((rows, seg)) * 2).astype(np.float16)
+    k1[rng.random((rows, seg)) < 0.05] = np.nan
+    k1[rng.random((rows, seg)) < 0.05] = -0.0
+    k2 = rng.integers(0, 2, (rows, seg)).astype(np.bool_)
+    k3 = rng.integers(-2, 2, (rows, seg)).astype(np.int32)
+    keys = [k0, k1, k2, k3]  # 1 + 2 + 1 + 4 = 8 bytes
+    d_keys = [torch.from_numpy(k.view(np.uint8).reshape(-1).copy()).to(dev) for k in keys]
+    dtypes = (ctypes.c_int * 4)(*[_lib.DTYPE_CODES[k.dtype] for k in keys])
+    ptrs = (ctypes.c_void_p * 4)(*[d.data_ptr() for d in d_keys])
+    out = torch.zeros(rows * seg, dtype=torch.int64, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    assert lib.cpn_lexsort_pack(4, dtypes, ptrs, None, 8, out.data_ptr(), rows, seg, stream) == 0
+    packed = out.cpu().numpy().view(np.uint64).reshape(rows, seg)
+    assert np.array_equal(np.argsort(packed, axis=-1, kind="stable"), np.lexsort(keys, axis=-1))
+    perm = np.stack([rng.permutation(seg) for _ in range(rows)]).astype(np.int64)
+    d_perm = torch.from_numpy(perm.reshape(-1)).to(dev)
+    assert lib.cpn_lexsort_pack(4, dtypes, ptrs, d_perm.data_ptr(), 8, out.data_ptr(), rows, seg, stream) == 0
+    assert np.array_equal(out.cpu().numpy().view(np.uint64).reshape(rows, seg), np.take_along_axis(packed, perm, axis=-1))
+    assert lib.cpn_lexsort_pack(4, dtypes, ptrs, None, 4, out.data_ptr(), rows, seg, stream) == -3  # 8 bytes into 4
+    cdt = (ctypes.c_int * 1)(_lib.DTYPE_CODES[np.dtype(np.complex64)])
+    assert lib.cpn_lexsort_pack(1, cdt, ptrs, None, 8, out.data_ptr(), rows, seg, stream) == -1
