@@ -29,6 +29,18 @@ static std::atomic<long long> g_wave_row_limit{[] {
   return (e != nullptr && *e != 0) ? atoll(e) : 1024ll;
 }()};
 
+// Rows from this length on take the 64-bit variant of the global kernels (never above 2^30).
+static std::atomic<long long> g_wide_row_threshold{[] {
+  const char* e = getenv("CPN_SORT_WIDE_ROW_THRESHOLD");
+  return (e != nullptr && *e != 0) ? atoll(e) : -1ll;
+}()};
+
+uint64_t wide_row_threshold()
+{
+  const long long t = g_wide_row_threshold.load(std::memory_order_relaxed);
+  return (t < 0 || static_cast<uint64_t>(t) > BIG_ROW_ELEMENTS) ? BIG_ROW_ELEMENTS : static_cast<uint64_t>(t);
+}
+
 uint64_t wave_row_limit()
 {
   const long long limit = g_wave_row_limit.load(std::memory_order_relaxed);
@@ -72,6 +84,11 @@ int cpn_last_hip_error(void) { return cpn::g_last_hip_error; }
 int64_t cpn_set_lds_row_limit(int64_t limit)
 {
   return static_cast<int64_t>(cpn::g_lds_row_limit.exchange(limit < 0 ? -1ll : static_cast<long long>(limit)));
+}
+
+int64_t cpn_set_wide_row_threshold(int64_t elements)
+{
+  return static_cast<int64_t>(cpn::g_wide_row_threshold.exchange(elements < 0 ? -1ll : static_cast<long long>(elements)));
 }
 
 int64_t cpn_set_wave_row_limit(int64_t limit)

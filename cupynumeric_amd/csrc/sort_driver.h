@@ -41,6 +41,10 @@ static_assert(HEADER_TICKETS + 4 * MAX_PASSES <= HEADER_VARYING, "tickets overla
 static_assert(HEADER_VARYING + 4 * MAX_PASSES <= HEADER_PLAN, "flags overlap the plan");
 static_assert(HEADER_PLAN + sizeof(SortPlan) <= HEADER_BYTES, "plan does not fit the header");
 constexpr uint64_t BIG_ROW_ELEMENTS = 1ull << 30;
+// Rows of at least this many elements use 64-bit counts, descriptors and row positions:
+// BIG_ROW_ELEMENTS unless lowered by cpn_set_wide_row_threshold / CPN_SORT_WIDE_ROW_THRESHOLD
+// (for tests that exercise the 64-bit kernels without a 2^30-element row).
+uint64_t wide_row_threshold();
 
 __host__ __device__ constexpr uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
 
@@ -142,7 +146,7 @@ inline GlobalLayout global_layout(int key_bytes, int passes, uint64_t volume, ui
                                   bool want_indices, bool in_place)
 {
   GlobalLayout L{};
-  L.big           = seg >= BIG_ROW_ELEMENTS;
+  L.big           = seg >= wide_row_threshold();
   L.passes        = passes;
   L.rows          = volume / seg;
   const uint64_t tile = static_cast<uint64_t>(global_tile(key_bytes, L.big));

@@ -87,6 +87,16 @@ int64_t cpn_set_lds_row_limit(int64_t limit);
  */
 int64_t cpn_set_wave_row_limit(int64_t limit);
 
+/*
+ * Process-wide tunable: rows of at least `elements` elements on the global path keep their
+ * per-row counts, tile descriptors and row positions in 64 bits.  The default and the maximum
+ * is 2^30 (shorter rows use 32 bits); a negative value restores the default and the previous
+ * setting is returned (-1 = default).  Lower values exist so that tests can run the 64-bit
+ * kernels on small inputs; they change workspace sizes (cpn_local_sort_temp_bytes follows).
+ * Also initialised from the environment variable CPN_SORT_WIDE_ROW_THRESHOLD.
+ */
+int64_t cpn_set_wide_row_threshold(int64_t elements);
+
 /* Size in bytes of one element of `dtype`, or 0 for an unknown code. */
 uint64_t cpn_dtype_size(int dtype);
 

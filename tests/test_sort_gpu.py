@@ -259,6 +259,43 @@ def test_outputs_in_place_and_offset(lib, torch_cuda, path, dtype):
         lib.cpn_set_lds_row_limit(prev)
 
 
+@pytest.fixture()
+def wide_rows(lib):
+    """Rows from 5000 elements on take the kernels with 64-bit counts, descriptors and row positions
+    (by default only rows of 2^30 elements and more do)."""
+    prev = lib.cpn_set_wide_row_threshold(5000)
+    yield
+    lib.cpn_set_wide_row_threshold(prev)
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+def test_global_path_wide_rows(lib, torch_cuda, wide_rows, dtype):
+    """The 64-bit variant of the global path: tiles are 8192 keys (4096 for 16-byte keys) there."""
+    for shape in [(5000,), (8192,), (8193,), (3, 20011), (100003,), (2, 4 * 8192)]:
+        x = make_input(dtype, shape, seed=shape[-1])
+        check_rows(lib, torch_cuda, x, f"{np.dtype(dtype)} {shape} (wide rows)")
+    x = make_input(dtype, (2, 30001), seed=3)
+    want_v = oracle.local_sort(x, argsort=False)
+    want_i = oracle.local_sort(x, argsort=True, offset=-7)
+    v, i = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=True, in_place=True, offset=-7)
+    assert_same_bits(v, want_v, "wide rows, in place + indices")
+    assert_same_bits(i, want_i, "wide rows, in place + indices")
+    # rows below the threshold in the same process keep the 32-bit kernels
+    check_rows(lib, torch_cuda, make_input(dtype, (4999,), seed=1), f"{np.dtype(dtype)} below the threshold")
+
+
+def test_wide_row_threshold_setter(lib):
+    prev = lib.cpn_set_wide_row_threshold(12345)
+    assert lib.cpn_set_wide_row_threshold(-1) == 12345
+    assert lib.cpn_set_wide_row_threshold(prev) == -1
+    code = _lib.DTYPE_CODES[np.dtype(np.float32)]
+    narrow = lib.cpn_local_sort_temp_bytes(code, 1 << 20, 1 << 20, 0, 1, 0)
+    lib.cpn_set_wide_row_threshold(1000)
+    wide = lib.cpn_local_sort_temp_bytes(code, 1 << 20, 1 << 20, 0, 1, 0)
+    lib.cpn_set_wide_row_threshold(prev)
+    assert wide > narrow  # 64-bit row positions and descriptors
+
+
 # ---- adversarial key distributions ------------------------------------------------------------------
 @pytest.mark.parametrize("path", ["lds", "global"])
 def test_skewed_and_degenerate_keys(lib, torch_cuda, path):
