@@ -148,3 +148,54 @@ def test_c5_full_size_axis0():
     job2.step()
     torch.cuda.synchronize()
     assert bool((job2.d_val == job.d_val).all())
+
+
+def test_more_than_2_to_31_elements():
+    """One row of 2^31 + 12345 uint16 keys: element counts and offsets beyond 32 bits, the 64-bit row
+    kernels at their real size.  Checked on the device through the properties that characterise a
+    stable argsort (permutation, order, ties in input order) and a sort (order, same histogram)."""
+    import ctypes
+
+    import torch
+
+    from cupynumeric_amd import _lib
+
+    free, _total = torch.cuda.mem_get_info()
+    if free < 90 * (1 << 30):
+        pytest.skip("needs about 80 GiB of free device memory")
+    lib = _lib.load()
+    dev = torch.device("cuda")
+    n = (1 << 31) + 12345
+    g = torch.Generator(device=dev)
+    g.manual_seed(31)
+    keys = torch.randint(0, 1 << 16, (n,), dtype=torch.int32, device=dev, generator=g).to(torch.int16)  # uint16 bit patterns
+    code = _lib.DTYPE_CODES[np.dtype(np.uint16)]
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    # argsort
+    idx = torch.empty(n, dtype=torch.int64, device=dev)
+    tb = lib.cpn_local_sort_temp_bytes(code, n, n, 0, 1, 0)
+    temp = torch.empty(tb, dtype=torch.uint8, device=dev)
+    rc = lib.cpn_local_sort(code, keys.data_ptr(), None, idx.data_ptr(), n, n, 0, 1, temp.data_ptr(), tb, stream)
+    assert rc == 0, _lib.status_string(rc)
+    assert lib.cpn_local_sort_check(temp.data_ptr(), stream) == 0
+    del temp
+    assert int(idx.min()) == 0 and int(idx.max()) == n - 1
+    seen = torch.zeros(n, dtype=torch.bool, device=dev)
+    seen[idx] = True
+    assert bool(seen.all()), "indices are not a permutation"
+    del seen
+    k = (keys[idx].to(torch.int32) & 0xFFFF)
+    assert bool((k[1:] >= k[:-1]).all()), "keys[idx] is not ascending"
+    out_of_order_tie = (k[1:] == k[:-1]) & (idx[1:] <= idx[:-1])  # (no mask indexing: 2^31 elements overflow it)
+    assert not bool(out_of_order_tie.any()), "ties are not in input order"
+    del out_of_order_tie, idx
+
+    # sort (values only): ascending and the same multiset
+    out = torch.empty_like(keys)
+    tb = lib.cpn_local_sort_temp_bytes(code, n, n, 1, 0, 0)
+    temp = torch.empty(tb, dtype=torch.uint8, device=dev)
+    rc = lib.cpn_local_sort(code, keys.data_ptr(), out.data_ptr(), None, n, n, 0, 1, temp.data_ptr(), tb, stream)
+    assert rc == 0, _lib.status_string(rc)
+    assert lib.cpn_local_sort_check(temp.data_ptr(), stream) == 0
+    assert bool(((out.to(torch.int32) & 0xFFFF) == k).all()), "sorted values differ from keys[argsort]"
