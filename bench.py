@@ -328,6 +328,8 @@ class SearchsortedJob:
         self.d_v = torch.from_numpy(self.v).to(dev)
         self.d_out = torch.empty(m, dtype=torch.int64, device=dev)
         self.stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        self.tb = 0 if os.environ.get("CPN_BENCH_SEARCH_DIRECT") else lib.cpn_searchsorted_temp_bytes(10, n, m)
+        self.temp = torch.empty(max(self.tb, 1), dtype=torch.uint8, device=dev)
         self.alg = {"total": m * (4 + 8), "searchsorted": m * (4 + 8)}
         self.dominant = "searchsorted"
         self.dtype = "u32"
@@ -335,7 +337,8 @@ class SearchsortedJob:
 
     def step(self):
         rc = self.lib.cpn_searchsorted(10, self.d_a.data_ptr(), self.n, self.d_v.data_ptr(), self.m, 1,
-                                       self.d_out.data_ptr(), self.stream)
+                                       self.d_out.data_ptr(), self.temp.data_ptr() if self.tb else None, self.tb,
+                                       self.stream)
         assert rc == 0, rc
 
     def verify(self):

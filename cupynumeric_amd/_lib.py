@@ -62,7 +62,10 @@ PROTOTYPES: dict[str, tuple] = {
     "cpn_local_sort_check": (c_int, [c_void_p, c_void_p]),
     "cpn_real_to_complex": (c_int, [c_int, c_void_p, c_int, c_void_p, c_uint64, c_void_p]),
     "cpn_astype": (c_int, [c_int, c_void_p, c_int, c_void_p, c_uint64, c_void_p]),
-    "cpn_searchsorted": (c_int, [c_int, c_void_p, c_uint64, c_void_p, c_uint64, c_int, c_void_p, c_void_p]),
+    "cpn_searchsorted_temp_bytes": (c_uint64, [c_int, c_uint64, c_uint64]),
+    "cpn_searchsorted": (
+        c_int, [c_int, c_void_p, c_uint64, c_void_p, c_uint64, c_int, c_void_p, c_void_p, c_uint64, c_void_p]
+    ),
     "cpn_unique_temp_bytes": (c_uint64, [c_int, c_uint64]),
     "cpn_unique": (c_int, [c_int, c_void_p, c_void_p, c_uint64, c_void_p, c_void_p, c_uint64, c_void_p]),
     "cpn_take_along_last_axis": (

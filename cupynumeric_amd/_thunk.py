@@ -247,17 +247,25 @@ class DeviceArray:
         if rhs.dtype != v.dtype or self.dtype != np.dtype(np.int64):
             raise TypeError("searchsorted: arrays must share one dtype and the result must be int64")
         lib = _lib.load()
+        code = _lib.DTYPE_CODES[rhs.dtype]
+        temp_bytes = lib.cpn_searchsorted_temp_bytes(code, rhs.size, v.size)
+        temp = runtime.empty_bytes(temp_bytes) if temp_bytes else None
+        stream = ctypes.c_void_p(runtime.stream_handle())
         status = lib.cpn_searchsorted(
-            _lib.DTYPE_CODES[rhs.dtype],
+            code,
             rhs.base.ptr() if rhs.size else None,
             rhs.size,
             v.base.ptr(),
             v.size,
             int(is_left),
             self.base.ptr(),
-            ctypes.c_void_p(runtime.stream_handle()),
+            temp.data_ptr() if temp is not None else None,
+            temp_bytes,
+            stream,
         )
         _lib.check(status, "cpn_searchsorted")
+        if temp is not None and runtime.check_status:
+            _lib.check(lib.cpn_local_sort_check(temp.data_ptr(), stream), "cpn_searchsorted")
 
     def unique(self) -> "DeviceArray":
         """`DeferredArray.unique` (`cupynumeric/_thunk/deferred.py:5375-5395`): sorted distinct

@@ -11,6 +11,13 @@
 // A probe of the sorted array is a dependent load, so the first eleven steps of every search
 // run over a table of up to 2048 evenly spaced elements that each workgroup stages in LDS;
 // the remaining steps stay inside one stride of the array.
+//
+// Every remaining probe of an unordered value is a sector of its own from HBM.  When the
+// array is too large for the caches and there are many values, the values are therefore
+// sorted first (with their positions, by the library's own sort, in the caller's workspace):
+// neighbouring lanes then search for neighbouring values, their probes fall into the same
+// cache lines, and the array is read about once instead of once per probe.  The answers go
+// back to the positions the values came from.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -46,6 +53,7 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void searchsorted_kernel(const KeyT* 
                                                                     const KeyT* __restrict__ values,
                                                                     uint64_t num_values,
                                                                     int64_t* __restrict__ out,
+                                                                    const int64_t* __restrict__ origin,
                                                                     uint64_t step,
                                                                     uint32_t num_pivots)
 {
@@ -99,13 +107,14 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void searchsorted_kernel(const KeyT* 
         hi = mid;
       }
     }
-    out[i] = static_cast<int64_t>(lo);
+    // `origin` (values sorted beforehand): the position the value had in the caller's array
+    out[origin != nullptr ? static_cast<uint64_t>(origin[i]) : i] = static_cast<int64_t>(lo);
   }
 }
 
 template <typename KeyT, int CODEC>
 static int launch_searchsorted(const void* sorted, uint64_t n, const void* values, uint64_t num_values, bool left,
-                               int64_t* out, hipStream_t stream)
+                               int64_t* out, const int64_t* origin, hipStream_t stream)
 {
   uint64_t step       = 0;
   uint32_t num_pivots = 0;
@@ -123,20 +132,52 @@ static int launch_searchsorted(const void* sorted, uint64_t n, const void* value
   if (left) {
     hipLaunchKernelGGL((searchsorted_kernel<KeyT, CODEC, true>), dim3(static_cast<uint32_t>(grid)), dim3(SEARCH_BLOCK),
                        0, stream, static_cast<const KeyT*>(sorted), n, static_cast<const KeyT*>(values), num_values, out,
-                       step, num_pivots);
+                       origin, step, num_pivots);
   } else {
     hipLaunchKernelGGL((searchsorted_kernel<KeyT, CODEC, false>), dim3(static_cast<uint32_t>(grid)),
                        dim3(SEARCH_BLOCK), 0, stream, static_cast<const KeyT*>(sorted), n,
-                       static_cast<const KeyT*>(values), num_values, out, step, num_pivots);
+                       static_cast<const KeyT*>(values), num_values, out, origin, step, num_pivots);
   }
   CPN_HIP_TRY(hipGetLastError());
   return CPN_OK;
 }
 
+// Sorting the values first pays when the sorted array is far larger than the caches and the
+// values are many; otherwise (and whenever the caller brings no workspace) values are searched
+// in the order given.
+static bool presort_pays(int key_bytes, uint64_t n, uint64_t num_values)
+{
+  return n * static_cast<uint64_t>(key_bytes) >= (64ull << 20) && num_values >= (1ull << 16);
+}
+
+struct SearchLayout {
+  uint64_t sort_bytes, off_values, off_origin, total;
+};
+
+static SearchLayout search_layout(int dtype, int key_bytes, uint64_t num_values)
+{
+  SearchLayout L{};
+  L.sort_bytes = cpn_local_sort_temp_bytes(dtype, num_values, num_values, 1, 1, 0);
+  L.off_values = align_up(L.sort_bytes, WORKSPACE_ALIGN);
+  L.off_origin = L.off_values + align_up(num_values * static_cast<uint64_t>(key_bytes), WORKSPACE_ALIGN);
+  L.total      = L.off_origin + align_up(num_values * 8, WORKSPACE_ALIGN);
+  return L;
+}
+
 }  // namespace cpn
 
+extern "C" uint64_t cpn_searchsorted_temp_bytes(int dtype, uint64_t n, uint64_t num_values)
+{
+  const cpn::KeyKind k = cpn::key_kind(dtype);
+  if (k.bytes == 0 || k.codec < 0 || !cpn::presort_pays(k.bytes, n, num_values)) {
+    return 0;
+  }
+  const cpn::SearchLayout L = cpn::search_layout(dtype, k.bytes, num_values);
+  return L.sort_bytes == 0 ? 0 : L.total;
+}
+
 extern "C" int cpn_searchsorted(int dtype, const void* sorted, uint64_t n, const void* values, uint64_t num_values,
-                                int left, int64_t* positions_out, void* stream)
+                                int left, int64_t* positions_out, void* temp, uint64_t temp_bytes, void* stream)
 {
   using namespace cpn;
   const KeyKind k = key_kind(dtype);
@@ -154,9 +195,29 @@ extern "C" int cpn_searchsorted(int dtype, const void* sorted, uint64_t n, const
       (reinterpret_cast<uintptr_t>(positions_out) % 8) != 0) {
     return CPN_ERR_ALIGN;
   }
+  const int64_t* origin = nullptr;
+  if (temp != nullptr && presort_pays(k.bytes, n, num_values)) {
+    const SearchLayout L = search_layout(dtype, k.bytes, num_values);
+    if (L.sort_bytes != 0 && temp_bytes >= L.total) {
+      if ((reinterpret_cast<uintptr_t>(temp) % WORKSPACE_ALIGN) != 0) {
+        return CPN_ERR_TEMP;
+      }
+      unsigned char* ws = static_cast<unsigned char*>(temp);
+      void* sorted_vals = ws + L.off_values;
+      int64_t* where    = reinterpret_cast<int64_t*>(ws + L.off_origin);
+      const int rc = cpn_local_sort(dtype, values, sorted_vals, where, num_values, num_values, 0, 1, ws, L.sort_bytes,
+                                    stream);
+      if (rc != CPN_OK) {
+        return rc;
+      }
+      values = sorted_vals;
+      origin = where;
+    }
+  }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool l  = left != 0;
-#define CPN_SEARCH_CASE(T, C) return launch_searchsorted<T, C>(sorted, n, values, num_values, l, positions_out, s)
+#define CPN_SEARCH_CASE(T, C) \
+  return launch_searchsorted<T, C>(sorted, n, values, num_values, l, positions_out, origin, s)
   switch (k.codec) {
     case CODEC_UNSIGNED:
       switch (k.bytes) {

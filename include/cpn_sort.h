@@ -188,9 +188,19 @@ int cpn_astype(int src_dtype, const void* in, int dst_dtype, void* out, uint64_t
  * Both arrays have element type `dtype`; the order is the one cpn_local_sort produces.
  * Replaces SearchSortedTask::gpu_variant (src/cupynumeric/sort/searchsorted.cu:27-116,
  * cupynumeric/_thunk/deferred.py:5425-5451) for a sorted array held by one GPU.
+ *
+ * `temp` is optional.  cpn_searchsorted_temp_bytes returns the size of the workspace with
+ * which a large search (sorted array beyond the caches, many values) first sorts the values
+ * so that neighbouring lanes probe neighbouring memory, or 0 when the request is searched
+ * directly anyway.  With temp == NULL, or a workspace smaller than that, the values are
+ * searched in the order given; the results are the same.  A workspace must be 256-byte
+ * aligned; when it is used its first word is the sort's device status
+ * (cpn_local_sort_check applies).
  */
+uint64_t cpn_searchsorted_temp_bytes(int dtype, uint64_t n, uint64_t num_values);
 int cpn_searchsorted(int dtype, const void* sorted, uint64_t n, const void* values,
-                     uint64_t num_values, int left, int64_t* positions_out, void* stream);
+                     uint64_t num_values, int left, int64_t* positions_out, void* temp,
+                     uint64_t temp_bytes, void* stream);
 
 /*
  * Sorted distinct values.  values_out has room for `volume` elements and receives the

@@ -139,6 +139,47 @@ def test_searchsorted_follows_sort_output():
     assert (right > left).all()  # every value is present
 
 
+def test_searchsorted_presorted_values_path():
+    """Array beyond the cache threshold (64 MiB) with many values: with a workspace the values are sorted
+    first; without one they are searched as given.  Same answers, both sides, float and complex."""
+    import torch
+
+    lib = _lib.load()
+    dev = torch.device("cuda")
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rng = np.random.default_rng(12)
+    for dtype, n, m in [(np.float32, (1 << 24) + 77, 200_001), (np.complex64, (1 << 23) + 5, 70_000), (np.uint8, 1 << 26, 1 << 16)]:
+        if dtype == np.uint8:
+            a = np.sort(rng.integers(0, 256, n).astype(dtype))
+            v = rng.integers(0, 256, m).astype(dtype)
+        elif dtype == np.float32:
+            a = np.sort(rng.standard_normal(n).astype(dtype))
+            a[-1000:] = np.nan
+            v = rng.standard_normal(m).astype(dtype)
+            v[::97] = np.nan
+            v[1::97] = a[rng.integers(0, n - 1000, v[1::97].size)]  # values that are present
+        else:
+            a = np.sort((np.round(rng.standard_normal(n) * 1000) + 1j * np.round(rng.standard_normal(n) * 3)).astype(dtype))
+            v = (np.round(rng.standard_normal(m) * 1000) + 1j * np.round(rng.standard_normal(m) * 3)).astype(dtype)
+        code = _lib.DTYPE_CODES[np.dtype(dtype)]
+        d_a = torch.from_numpy(a.view(np.uint8)).to(dev)
+        d_v = torch.from_numpy(v.view(np.uint8)).to(dev)
+        tb = lib.cpn_searchsorted_temp_bytes(code, n, m)
+        assert tb > 0
+        assert lib.cpn_searchsorted_temp_bytes(code, 1000, m) == 0 and lib.cpn_searchsorted_temp_bytes(code, n, 100) == 0
+        temp = torch.empty(tb, dtype=torch.uint8, device=dev)
+        for left in (1, 0):
+            want = np.searchsorted(a, v, side="left" if left else "right")
+            with_ws = torch.full((m,), -1, dtype=torch.int64, device=dev)
+            rc = lib.cpn_searchsorted(code, d_a.data_ptr(), n, d_v.data_ptr(), m, left, with_ws.data_ptr(), temp.data_ptr(), tb, stream)
+            assert rc == 0 and lib.cpn_local_sort_check(temp.data_ptr(), stream) == 0
+            direct = torch.full((m,), -1, dtype=torch.int64, device=dev)
+            assert lib.cpn_searchsorted(code, d_a.data_ptr(), n, d_v.data_ptr(), m, left, direct.data_ptr(), None, 0, stream) == 0
+            assert np.array_equal(with_ws.cpu().numpy(), want), (dtype, left)
+            assert np.array_equal(direct.cpu().numpy(), want), (dtype, left)
+            assert np.array_equal(d_v.cpu().numpy(), v.view(np.uint8))  # values untouched
+
+
 # ---- unique --------------------------------------------------------------------------------------------
 def numpy_unique(x: np.ndarray) -> np.ndarray:
     """np.unique, except that float16 goes through float32 (exact and order preserving): the default
