@@ -63,6 +63,66 @@ __global__ __launch_bounds__(256) void transpose_last_kernel(const T* __restrict
   }
 }
 
+// 2-byte elements, both extents even and both pointers 4-byte aligned: 128 x 128 tiles moved as
+// 32-bit words.  A thread loads the two words of a 2 x 2 block, exchanges the halves in
+// registers (v_perm_b32) and stores two words that already hold two elements of an output
+// row each, so that the LDS tile is transposed at word granularity and every HBM access of a
+// wavefront is 256 contiguous bytes.
+constexpr int PAIR_TS = 128;
+__global__ __launch_bounds__(256) void transpose_pairs_kernel(const uint32_t* __restrict__ in,
+                                                               uint32_t* __restrict__ out,
+                                                               uint64_t A,
+                                                               uint64_t M,
+                                                               uint64_t B,
+                                                               uint32_t tiles_a,
+                                                               uint32_t tiles_b)
+{
+  constexpr int HP = PAIR_TS / 2;  // words per tile row
+  __shared__ uint32_t tile[PAIR_TS][HP + 1];  // [column of the input][pair of input rows]
+
+  uint64_t bid         = blockIdx.x;
+  const uint32_t tb    = static_cast<uint32_t>(bid % tiles_b);
+  bid /= tiles_b;
+  const uint32_t ta    = static_cast<uint32_t>(bid % tiles_a);
+  const uint64_t batch = bid / tiles_a;
+  const uint64_t p     = batch / M;
+  const uint64_t m     = batch - p * M;
+  // element offsets; all even, so halving them gives word offsets
+  const uint64_t in_base  = (p * A * M + m) * B;
+  const uint64_t out_base = (p * B * M + m) * A;
+  const uint64_t in_row   = M * B;
+  const uint64_t out_row  = M * A;
+  const uint64_t a0       = static_cast<uint64_t>(ta) * PAIR_TS;
+  const uint64_t b0       = static_cast<uint64_t>(tb) * PAIR_TS;
+
+  const int x = threadIdx.x % HP;  // word inside a row (load: column pair, store: row pair)
+  const int y = threadIdx.x / HP;  // 0..3
+  {
+    const uint64_t ib = b0 + 2 * x;
+#pragma unroll 4
+    for (int rp = y; rp < HP; rp += 256 / HP) {
+      const uint64_t ia = a0 + 2 * rp;
+      if (ia < A && ib < B) {
+        const uint32_t w0 = in[(in_base + ia * in_row + ib) / 2];        // x[ia][ib], x[ia][ib+1]
+        const uint32_t w1 = in[(in_base + (ia + 1) * in_row + ib) / 2];  // x[ia+1][ib], x[ia+1][ib+1]
+        tile[2 * x][rp]     = __builtin_amdgcn_perm(w1, w0, 0x05040100u);  // x[ia][ib],   x[ia+1][ib]
+        tile[2 * x + 1][rp] = __builtin_amdgcn_perm(w1, w0, 0x07060302u);  // x[ia][ib+1], x[ia+1][ib+1]
+      }
+    }
+  }
+  __syncthreads();
+  {
+    const uint64_t ia = a0 + 2 * x;
+#pragma unroll 4
+    for (int c = y; c < PAIR_TS; c += 256 / HP) {
+      const uint64_t ib = b0 + c;
+      if (ia < A && ib < B) {
+        out[(out_base + ib * out_row + ia) / 2] = tile[c][x];
+      }
+    }
+  }
+}
+
 // General case: in [P][A][M][B][Q] -> out [P][B][M][A][Q], one output element per thread step.
 template <typename T>
 __global__ __launch_bounds__(256) void swapaxes_generic_kernel(const T* __restrict__ in,
@@ -93,6 +153,24 @@ static int swapaxes_typed(const void* in, void* out, uint64_t P, uint64_t A, uin
                           hipStream_t stream)
 {
   const uint64_t total = P * A * M * B * Q;
+  if constexpr (sizeof(T) == 2) {
+    if (Q == 1 && A % 2 == 0 && B % 2 == 0 && (reinterpret_cast<uintptr_t>(in) % 4) == 0 &&
+        (reinterpret_cast<uintptr_t>(out) % 4) == 0) {
+      const uint64_t tiles_a = (A + PAIR_TS - 1) / PAIR_TS;
+      const uint64_t tiles_b = (B + PAIR_TS - 1) / PAIR_TS;
+      const uint64_t grid    = tiles_a * tiles_b * P * M;
+      if (tiles_a < (1ull << 31) && tiles_b < (1ull << 31) && grid < (1ull << 31)) {
+        {
+          ProfileScope prof("transpose_last", stream);
+          hipLaunchKernelGGL(transpose_pairs_kernel, dim3(static_cast<uint32_t>(grid)), dim3(256), 0, stream,
+                             static_cast<const uint32_t*>(in), static_cast<uint32_t*>(out), A, M, B,
+                             static_cast<uint32_t>(tiles_a), static_cast<uint32_t>(tiles_b));
+        }
+        CPN_HIP_TRY(hipGetLastError());
+        return CPN_OK;
+      }
+    }
+  }
   if (Q == 1) {
     const uint64_t tiles_a = (A + TS - 1) / TS;
     const uint64_t tiles_b = (B + TS - 1) / TS;

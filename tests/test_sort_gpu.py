@@ -381,7 +381,10 @@ def test_swapaxes_copy(lib, torch_cuda, elem):
     torch = torch_cuda
     shapes = [((3, 4), 0, 1), ((65, 130), 0, 1), ((64, 64), 1, 0), ((5, 6, 7), 0, 2), ((5, 6, 7), 1, 2), ((5, 6, 7), 0, 1),
               ((2, 3, 4, 5), 1, 3), ((2, 3, 4, 5), 0, 2), ((1, 12, 1), 1, 2), ((7, 1), 0, 1), ((300, 3), 0, 1),
-              ((4, 5), 1, 1), ((2, 2, 1, 1, 2, 1, 2), 0, 6)]
+              ((4, 5), 1, 1), ((2, 2, 1, 1, 2, 1, 2), 0, 6),
+              # even extents: 2-byte elements move as 32-bit words in 128 x 128 tiles
+              ((128, 128), 0, 1), ((130, 258), 0, 1), ((2, 4), 0, 1), ((200, 2), 0, 1), ((6, 4, 10), 0, 2),
+              ((3, 8, 6), 1, 2), ((2, 256, 3, 130), 1, 3), ((514, 126), 1, 0)]
     rng = np.random.default_rng(0)
     for shape, a, b in shapes:
         x = rng.integers(0, 255, int(np.prod(shape)) * np.dtype(elem).itemsize, dtype=np.uint8).view(elem).reshape(shape)
