@@ -57,9 +57,47 @@ DTYPE_CODES = {
 _lib = None
 
 
+THRUST_LIB_PATH = HERE / "_build" / "libcpnthrust.so"
+_thrust = None
+
+
+def thrust_local_sort(x: np.ndarray, argsort: bool, stable: bool = True, use_omp: bool = False):
+    """Baseline only (bench.py): the reference's CPU / OpenMP variant over rocThrust's host backends
+    (thrust_baseline.cpp).  Copy + index initialisation as in `SortImplBodyCpu`
+    (`src/cupynumeric/sort/sort_cpu.inl:974-1025`), then the per-row thrust calls.  Floats with NaN
+    or -0.0 do not come out in NumPy's order."""
+    global _thrust
+    if _thrust is None:
+        if not THRUST_LIB_PATH.exists():
+            build()
+        import torch  # noqa: F401  (its bundled HIP runtime must be the one the process binds, see Makefile)
+
+        _thrust = ctypes.CDLL(str(THRUST_LIB_PATH))
+        _thrust.cpn_thrust_local_sort.restype = ctypes.c_int
+        _thrust.cpn_thrust_local_sort.argtypes = [
+            ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_int, ctypes.c_int,
+        ]
+    x = np.ascontiguousarray(x)
+    seg = x.shape[-1]
+    values = x.copy()
+    indices = None
+    if argsort:
+        indices = np.ascontiguousarray(np.broadcast_to(np.arange(seg, dtype=np.int64), x.shape))
+    rc = _thrust.cpn_thrust_local_sort(
+        DTYPE_CODES[x.dtype], values.ctypes.data, indices.ctypes.data if argsort else None, x.size, seg,
+        int(stable), int(use_omp),
+    )
+    if rc != 0:
+        raise RuntimeError(f"cpn_thrust_local_sort failed: {rc}")
+    return indices if argsort else values
+
+
 def build(force: bool = False) -> Path:
-    """Compile sort_oracle.c with gcc (see Makefile)."""
-    if force or not LIB_PATH.exists() or LIB_PATH.stat().st_mtime < (HERE / "sort_oracle.c").stat().st_mtime:
+    """Compile sort_oracle.c with gcc and thrust_baseline.cpp with hipcc (see Makefile)."""
+    sources = [HERE / "sort_oracle.c", HERE / "thrust_baseline.cpp"]
+    stale = any(not lib.exists() or lib.stat().st_mtime < src.stat().st_mtime
+                for lib, src in zip([LIB_PATH, THRUST_LIB_PATH], sources))
+    if force or stale:
         subprocess.run(["make", "-C", str(HERE), "-B" if force else "-s"], check=True, capture_output=True)
     return LIB_PATH
 

@@ -282,3 +282,19 @@ def test_searchsorted_common_type_and_errors():
         oracle.searchsorted(np.arange(100), np.arange(10), sorter=np.arange(10))
     with pytest.raises(TypeError):
         oracle.searchsorted([2, 3, 10, 9], None)
+
+
+def test_thrust_baseline_matches_numpy_on_plain_data():
+    """The second CPU baseline of bench.py (the reference's per-row thrust calls over rocThrust's host
+    backends) is only a timing baseline; on data without NaN and -0.0, where bit-pattern order and
+    NumPy's order coincide, its output is checked here."""
+    rng = np.random.default_rng(21)
+    for dtype in (np.int32, np.int64, np.uint8, np.float32, np.float64):
+        if np.dtype(dtype).kind == "f":
+            x = rng.standard_normal((7, 3001)).astype(dtype)
+        else:
+            info = np.iinfo(dtype)
+            x = rng.integers(info.min, info.max, (7, 3001), dtype=dtype, endpoint=True)
+        for use_omp in (False, True):
+            assert np.array_equal(oracle.thrust_local_sort(x, False, use_omp=use_omp), np.sort(x, axis=-1, kind="stable"))
+            assert np.array_equal(oracle.thrust_local_sort(x, True, use_omp=use_omp), np.argsort(x, axis=-1, kind="stable"))
