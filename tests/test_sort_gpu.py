@@ -421,3 +421,38 @@ def test_complex_integration_cases():
                 assert np.array_equal(
                     num.argsort(arr_num, axis=axis, kind="stable"), np.argsort(arr_np, axis=axis, kind="stable")
                 )
+
+
+# ---- seeded random sweep over shapes, axes, dtypes and entry points -----------------------------------
+@pytest.mark.parametrize("seed", range(8))
+def test_random_shapes_axes_dtypes(seed):
+    """40 random cases per seed through the public API: 1-3 dimensions, any axis (or None), every dtype,
+    sort / argsort / in-place sort, rows from empty to tens of thousands of elements, so that every row
+    kernel and the global path meet odd lengths and odd batch counts."""
+    rng = np.random.default_rng(1000 + seed)
+    for case in range(40):
+        dtype = ALL_DTYPES[int(rng.integers(len(ALL_DTYPES)))]
+        ndim = int(rng.integers(1, 4))
+        budget = int(rng.choice([64, 3000, 60_000, 200_000]))
+        shape = []
+        for d in range(ndim):
+            hi = max(1, int(budget ** (1.0 / (ndim - d))))
+            n = int(rng.integers(0 if rng.random() < 0.03 else 1, hi + 1))
+            shape.append(n)
+            budget = max(1, budget // max(n, 1))
+        rng.shuffle(shape)
+        shape = tuple(int(s) for s in shape)
+        axis = None if rng.random() < 0.15 else int(rng.integers(-ndim, ndim))
+        x = make_input(dtype, shape, seed=seed * 100 + case)
+        a = num.array(x)
+        what = f"seed={seed} case={case} {np.dtype(dtype)} {shape} axis={axis}"
+        op = int(rng.integers(3))
+        if op == 0:
+            assert_same_bits(np.asarray(num.sort(a, axis=axis)), oracle.sort(x, axis=axis), what + " sort")
+        elif op == 1:
+            got = num.argsort(a, axis=axis, kind="stable")
+            want = oracle.argsort(x, axis=axis, kind="stable")
+            assert got.shape == want.shape and np.array_equal(np.asarray(got), want), what + " argsort"
+        else:
+            a.sort(axis=axis)
+            assert_same_bits(np.asarray(a), oracle.sort(x, axis=axis), what + " in place")
