@@ -22,29 +22,9 @@
 #include <stdint.h>
 
 #include "radix_common.h"
+#include "wave_row_sort.h"  // wave_all_and / wave_all_or
 
 namespace cpn {
-
-template <typename T>
-__device__ __forceinline__ T wave_reduce_and(T v)
-{
-#pragma unroll
-  for (int delta = WAVE / 2; delta > 0; delta >>= 1) {
-    v &= __shfl_xor(v, delta, WAVE);
-  }
-  return v;
-}
-template <typename T>
-__device__ __forceinline__ T wave_reduce_or(T v)
-{
-#pragma unroll
-  for (int delta = WAVE / 2; delta > 0; delta >>= 1) {
-    v |= __shfl_xor(v, delta, WAVE);
-  }
-  return v;
-}
-
-using SkipWord = unsigned long long;  // a key's digits, eight to a word, as shuffled across the wave
 
 template <typename KeyT, int CODEC, bool HAS_IDX, int BLOCK, int ITEMS>
 __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in,
@@ -60,7 +40,7 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
   constexpr int PASSES = KT::PASSES;
   constexpr int NW     = KT::NWORDS;
   using DT             = DigitThreads<BLOCK>;
-  using SW             = SkipWord;
+  using SW             = unsigned long long;  // a key's digits, eight to a word, as shuffled across the wave
   using IdxS           = uint16_t;  // row position while staged in LDS
   static_assert(TILE <= 65536, "row positions are staged as 16 bits");
 
@@ -107,8 +87,8 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
   // bits on which the keys of the row differ
 #pragma unroll
   for (int n = 0; n < NW; ++n) {
-    all_and[n] = wave_reduce_and(all_and[n]);
-    all_or[n]  = wave_reduce_or(all_or[n]);
+    all_and[n] = wave_all_and(all_and[n]);
+    all_or[n]  = wave_all_or(all_or[n]);
     if (lane == 0) {
       s_red[(2 * wave) * NW + n]     = all_and[n];
       s_red[(2 * wave + 1) * NW + n] = all_or[n];
