@@ -117,3 +117,12 @@ def make_input(dtype, shape, seed: int, special: bool = True, duplicates: bool =
             x[rng.integers(0, n, max(n // 50, 1))] = info.min
             x[rng.integers(0, n, max(n // 50, 1))] = info.max
     return x.reshape(shape)
+
+
+# tests/cpp/integration/test_unique.cc:34-68: (input, shape, expected distinct values)
+UNIQUE_GOLDEN = [
+    ([1, 1, 2, 2, 3, 3], (6,), [1, 2, 3], np.int32),
+    ([1, 1, 2, 3], (2, 2), [1, 2, 3], np.int32),
+    ([1, 2, 1, 1, 3, 3, 3, 4, 5, 4], (10,), [1, 2, 3, 4, 5], np.int32),
+    ([99], (1,), [99], np.int64),
+]

@@ -191,6 +191,11 @@ def numpy_unique(x: np.ndarray) -> np.ndarray:
 
 
 def test_unique_reference_cases():
+    from conftest import UNIQUE_GOLDEN
+
+    for values, shape, expected, dtype in UNIQUE_GOLDEN:  # tests/cpp/integration/test_unique.cc:34-68
+        got = num.unique(num.array(np.array(values, dtype=dtype).reshape(shape)))
+        assert got.dtype == np.dtype(dtype) and np.asarray(got).tolist() == expected
     # tests/integration/test_unique.py:23-39
     a = np.nonzero(np.array([1, 1, 0, 0]))[0]
     assert np.array_equal(np.asarray(num.unique(num.array(a))), np.unique(a))

@@ -298,3 +298,11 @@ def test_thrust_baseline_matches_numpy_on_plain_data():
         for use_omp in (False, True):
             assert np.array_equal(oracle.thrust_local_sort(x, False, use_omp=use_omp), np.sort(x, axis=-1, kind="stable"))
             assert np.array_equal(oracle.thrust_local_sort(x, True, use_omp=use_omp), np.argsort(x, axis=-1, kind="stable"))
+
+
+def test_unique_reference_golden_vectors():
+    from conftest import UNIQUE_GOLDEN
+
+    for values, shape, expected, dtype in UNIQUE_GOLDEN:
+        got = oracle.unique(np.array(values, dtype=dtype).reshape(shape))
+        assert got.dtype == np.dtype(dtype) and got.tolist() == expected
