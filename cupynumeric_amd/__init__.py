@@ -19,7 +19,8 @@ from ._array import convert_to_ndarray, ndarray
 from ._thunk import SUPPORTED_DTYPES, DeviceArray, check_dtype
 
 __all__ = [
-    "ndarray", "array", "asarray", "sort", "argsort", "sort_complex", "partition", "argpartition", "lexsort", "searchsorted", "unique", "random",
+    "ndarray", "array", "asarray", "sort", "argsort", "sort_complex", "partition", "argpartition", "lexsort", "searchsorted", "unique", "take_along_axis",
+    "random",
     "SUPPORTED_DTYPES",
 ]
 
@@ -178,6 +179,47 @@ def unique(
     if any((return_index, return_inverse, return_counts)) or axis is not None:
         raise NotImplementedError("Keyword arguments for `unique` are not yet supported")
     return ar.unique()
+
+
+def take_along_axis(a: Any, indices: Any, axis: int | None) -> ndarray:
+    """Values of `a` at `indices` along `axis` (`cupynumeric/_module/indexing.py:657-770`), for the
+    case the reference's TAKE task covers: every dimension other than `axis` agrees between `a`
+    and `indices` (no broadcasting).  `axis=None` flattens `a` and wants 1-D indices.  Indices out
+    of range raise IndexError."""
+    from numpy.lib.array_utils import normalize_axis_index
+
+    a = convert_to_ndarray(a)
+    indices = convert_to_ndarray(indices)
+    if not np.issubdtype(indices.dtype, np.integer):
+        raise TypeError("`indices` must be an integer array")
+
+    computed_axis = 0
+    if axis is None:
+        if indices.ndim != 1:
+            raise ValueError("indices must be 1D if axis=None")
+        if a.ndim > 1:
+            a = ndarray((a.size,), a.dtype, thunk=a._thunk.reshape((a.size,)))
+    else:
+        computed_axis = normalize_axis_index(axis, a.ndim)
+
+    if a.ndim != indices.ndim:
+        raise ValueError("`indices` and `a` must have the same number of dimensions")
+    others_a = a.shape[:computed_axis] + a.shape[computed_axis + 1 :]
+    others_i = indices.shape[:computed_axis] + indices.shape[computed_axis + 1 :]
+    if others_a != others_i:
+        raise NotImplementedError("take_along_axis: broadcasting between `a` and `indices` is not supported")
+    if indices.dtype != np.dtype(np.int64):
+        indices = indices.astype(np.int64)
+
+    last = a.ndim - 1
+    src, idx = a._thunk, indices._thunk
+    if computed_axis != last:
+        src = src.swapaxes_copy(computed_axis, last)
+        idx = idx.swapaxes_copy(computed_axis, last)
+    out = src.take_along_last_axis(idx)
+    if computed_axis != last:
+        out = out.swapaxes_copy(last, computed_axis)
+    return ndarray(out.shape, out.dtype, thunk=out)
 
 
 def _split_first_axis(a: ndarray) -> list[ndarray]:

@@ -143,3 +143,34 @@ def test_lexsort_pack_c_abi():
     assert lib.cpn_lexsort_pack(4, dtypes, ptrs, None, 4, out.data_ptr(), rows, seg, stream) == -3  # 8 bytes into 4
     cdt = (ctypes.c_int * 1)(_lib.DTYPE_CODES[np.dtype(np.complex64)])
     assert lib.cpn_lexsort_pack(1, cdt, ptrs, None, 8, out.data_ptr(), rows, seg, stream) == -1
+
+
+def test_take_along_axis_public():
+    """tests/integration/test_take_along_axis.py in the no-broadcast form: argsort indices reproduce the
+    sort, every axis, negative indices, flattened form, error cases."""
+    rng = np.random.default_rng(10)
+    for shape in [(7,), (5, 9), (3, 4, 6), (2, 3, 4, 5)]:
+        x = rng.standard_normal(shape).astype(np.float32)
+        a = num.array(x)
+        for axis in range(-len(shape), len(shape)):
+            idx = num.argsort(a, axis=axis, kind="stable")
+            got = num.take_along_axis(a, idx, axis)
+            assert np.array_equal(np.asarray(got), np.sort(x, axis=axis))
+            k = rng.integers(-shape[axis], shape[axis], shape).astype(np.int32)  # other integer type, negatives
+            assert np.array_equal(np.asarray(num.take_along_axis(a, k, axis)), np.take_along_axis(x, k.astype(np.int64), axis))
+        short = tuple(2 if d == len(shape) - 1 else s for d, s in enumerate(shape))  # fewer picks than elements
+        k = rng.integers(0, shape[-1], short)
+        assert np.array_equal(np.asarray(num.take_along_axis(a, k, -1)), np.take_along_axis(x, k, -1))
+    x = rng.integers(0, 100, (4, 5))
+    k = rng.integers(0, 20, 7)
+    assert np.array_equal(np.asarray(num.take_along_axis(num.array(x), k, None)), np.take_along_axis(x, k, None))
+    with pytest.raises(TypeError):
+        num.take_along_axis(x, np.zeros((4, 5)), 0)
+    with pytest.raises(ValueError):
+        num.take_along_axis(x, np.zeros((4, 5), dtype=int), None)
+    with pytest.raises(ValueError):
+        num.take_along_axis(x, np.zeros(3, dtype=int), 0)
+    with pytest.raises(IndexError):
+        num.take_along_axis(x, np.full((4, 5), 5), 1)
+    with pytest.raises(np.exceptions.AxisError):
+        num.take_along_axis(x, np.zeros((4, 5), dtype=int), 2)
