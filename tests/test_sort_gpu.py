@@ -504,3 +504,47 @@ def test_sort_call_is_capturable_into_a_graph(lib, torch_cuda):
         # eager work between the replays
         v, i = abi_sort(lib, torch, x[:5000], want_values=True, want_indices=True)
         assert np.array_equal(i, oracle.local_sort(x[:5000], argsort=True))
+
+
+# ---- concurrent callers ------------------------------------------------------------------------------------
+def test_concurrent_streams_and_threads(lib, torch_cuda):
+    """Two host threads, each with its own stream, buffers and workspace, sort at the same time: the
+    library keeps no shared mutable state between calls (the tunables aside)."""
+    import threading
+
+    torch = torch_cuda
+    dev = torch.device("cuda")
+    errors: list[str] = []
+
+    def worker(tid: int) -> None:
+        try:
+            rng = np.random.default_rng(50 + tid)
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for it in range(6):
+                    n = int(rng.integers(20_000, 400_000))
+                    dtype = [np.float32, np.int64, np.uint16][(tid + it) % 3]
+                    x = make_input(dtype, (n,), seed=tid * 100 + it)
+                    code = _lib.DTYPE_CODES[np.dtype(dtype)]
+                    d_in = torch.from_numpy(x.view(np.uint8).copy()).to(dev, non_blocking=False)
+                    d_idx = torch.empty(n, dtype=torch.int64, device=dev)
+                    tb = lib.cpn_local_sort_temp_bytes(code, n, n, 0, 1, 0)
+                    temp = torch.empty(tb, dtype=torch.uint8, device=dev)
+                    h = ctypes.c_void_p(stream.cuda_stream)
+                    rc = lib.cpn_local_sort(code, d_in.data_ptr(), None, d_idx.data_ptr(), n, n, 0, 1, temp.data_ptr(), tb, h)
+                    if rc != 0 or lib.cpn_local_sort_check(temp.data_ptr(), h) != 0:
+                        errors.append(f"thread {tid} iteration {it}: status {rc}")
+                        return
+                    stream.synchronize()
+                    if not np.array_equal(d_idx.cpu().numpy(), oracle.local_sort(x, argsort=True)):
+                        errors.append(f"thread {tid} iteration {it}: wrong result ({np.dtype(dtype)}, n={n})")
+                        return
+        except Exception as exc:  # surfaced below; an exception in a thread would otherwise be lost
+            errors.append(f"thread {tid}: {exc!r}")
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
