@@ -550,8 +550,8 @@ def main() -> None:
     for label, ms in records:
         by_label.setdefault(label, []).append(ms)
     alg = algorithmic_bytes(cfg, job.uses_lds_rows)
-    if job.uses_lds_rows:  # one wavefront per row up to 1024 elements, one workgroup per row above
-        dominant = "wave_row_sort" if "wave_row_sort" in by_label else "lds_row_sort"
+    if job.uses_lds_rows:  # whichever of the per-row kernels the row length selects
+        dominant = next(k for k in ("tiny_row_sort", "wave_row_sort", "lds_row_sort") if k in by_label)
         alg[dominant] = alg["lds_row_sort"]
     else:
         dominant = "onesweep"
