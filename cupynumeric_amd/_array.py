@@ -71,7 +71,8 @@ class ndarray:
         """Dense 1-D copy (C order)."""
         if order not in ("C", "K", "A"):
             raise NotImplementedError("only C-order flatten is supported")
-        return convert_to_ndarray(self.__array__().reshape(-1))
+        thunk = self._thunk.copy().reshape((self.size,))
+        return ndarray(thunk.shape, thunk.dtype, thunk=thunk)
 
     def setflags(self, write: bool | None = None) -> None:
         if write is not None:

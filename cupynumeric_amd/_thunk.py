@@ -98,6 +98,16 @@ class DeviceArray:
             raise ValueError("cannot reshape array: sizes differ")
         return out
 
+    def copy(self) -> "DeviceArray":
+        """Dense copy with storage of its own (`DeferredArray.copy(deep=True)`, `cupynumeric/_thunk/deferred.py:394-398`);
+        host data that has not been uploaded yet is copied on the host."""
+        if self.base._dev is None and self.base._host is not None:
+            return DeviceArray.from_numpy(np.asarray(self.base._host).reshape(self.shape))
+        sub = Storage(self.size * self.dtype.itemsize)
+        if self.size:
+            sub._dev = self.base.device()[: sub.nbytes].clone()
+        return DeviceArray(self.shape, self.dtype, sub)
+
     def slice_first_axis(self, i: int, count: int, shape: tuple[int, ...]) -> "DeviceArray":
         """`self[i]` as an array of `shape` (`count` elements) over the same memory: rows of a
         dense row-major buffer are themselves dense."""
