@@ -300,3 +300,60 @@ def test_astype_matches_numpy(src):
             want = x.astype(dst)
         assert got.dtype == want.dtype and got.shape == want.shape
         assert_same_bits(np.asarray(got), want, f"{np.dtype(src)}->{np.dtype(dst)}")
+
+
+# ---- seeded random sweep ------------------------------------------------------------------------------
+@pytest.mark.parametrize("seed", range(6))
+def test_random_consumers(seed):
+    """Random dtypes, sizes and duplicate rates for unique and searchsorted (NumPy is the expectation) and
+    random key sets for lexsort (the oracle, itself pinned on np.lexsort, is the expectation)."""
+    rng = np.random.default_rng(2000 + seed)
+    dtypes = ALL_REAL_DTYPES + COMPLEX_DTYPES
+    for case in range(25):
+        dtype = dtypes[int(rng.integers(len(dtypes)))]
+        kind = np.dtype(dtype).kind
+        n = int(rng.choice([1, 7, 300, 5000, 70_000]))
+        spread = float(rng.choice([1, 5, 200, 1e6]))
+
+        def draw(k):
+            if kind == "b":
+                return rng.integers(0, 2, k).astype(dtype)
+            if kind in "iu":
+                info = np.iinfo(dtype)
+                return rng.integers(max(info.min, -int(spread)), min(info.max, int(spread)) + 1, k).astype(dtype)
+            with np.errstate(all="ignore"):
+                base = np.round(rng.standard_normal(k) * spread)
+                if kind == "c":
+                    base = base + 1j * np.round(rng.standard_normal(k) * 2)
+                x = base.astype(dtype)
+            x[rng.random(k) < 0.02] = np.nan
+            return x
+
+        x = draw(n)
+        what = f"seed={seed} case={case} {np.dtype(dtype)} n={n} spread={spread}"
+        got = num.unique(num.array(x))
+        want = numpy_unique(x)
+        assert got.shape == want.shape and np.array_equal(np.asarray(got), want, equal_nan=True), what + " unique"
+        srt = np.sort(x, kind="stable")
+        v = draw(int(rng.choice([1, 50, 3000])))
+        side = "left" if rng.random() < 0.5 else "right"
+        got = np.asarray(num.searchsorted(num.array(srt), num.array(v), side=side))
+        assert np.array_equal(got, np.searchsorted(srt, v, side=side)), what + f" searchsorted {side}"
+        # lexsort: 1-4 keys of random types over a random 1-3 dimensional shape
+        ndim = int(rng.integers(1, 4))
+        shape = tuple(int(rng.integers(1, 30)) for _ in range(ndim - 1)) + (int(rng.choice([1, 9, 400, 9000])),)
+        axis = int(rng.integers(-ndim, ndim))
+        keys = []
+        for _ in range(int(rng.integers(1, 5))):
+            kd = dtypes[int(rng.integers(len(dtypes)))]
+            if np.dtype(kd).kind == "b":
+                keys.append(rng.integers(0, 2, shape).astype(kd))
+            elif np.dtype(kd).kind in "iu":
+                keys.append(rng.integers(0, 6, shape).astype(kd))
+            else:
+                with np.errstate(all="ignore"):
+                    k = np.round(rng.standard_normal(shape) * 2).astype(kd)
+                k[rng.random(shape) < 0.05] = np.nan
+                keys.append(k)
+        got = np.asarray(num.lexsort(tuple(num.array(k) for k in keys), axis=axis))
+        assert np.array_equal(got, oracle.lexsort(tuple(keys), axis=axis)), what + f" lexsort {shape} axis={axis}"
