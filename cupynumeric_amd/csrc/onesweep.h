@@ -48,6 +48,9 @@ struct DescBits {
 // Upper bound on polls of one descriptor before a tile gives up and flags an error, so
 // that every wave exits even if a predecessor never publishes.
 constexpr uint32_t LOOKBACK_SPIN_LIMIT = 1u << 22;
+// The limit in force: LOOKBACK_SPIN_LIMIT unless changed by cpn_set_lookback_spin_limit (tests of
+// the failure path set it to 1, so that a tile gives up at its first unanswered poll).
+uint32_t lookback_spin_limit();
 
 // Predecessor descriptors each look-back round reads at once.
 #ifndef CPN_LOOKBACK_WINDOW
@@ -348,6 +351,7 @@ struct SweepArgs {
   uint32_t num_tiles;
   int pass;                // which 8-bit digit this pass sorts by
   int idx_final;           // idx_out is the caller's int64 array
+  uint32_t spin_limit;     // polls of one descriptor before the tile gives up (LOOKBACK_SPIN_LIMIT)
 };
 
 #ifndef CPN_ONESWEEP_WAVES_PER_EU
@@ -509,7 +513,7 @@ __device__ __forceinline__ void onesweep_tile(
               const OffT* dp   = a.desc + static_cast<uint64_t>(t) * RADIX + tid;
               uint32_t spins   = 0;
               do {
-                if (++spins >= LOOKBACK_SPIN_LIMIT) {
+                if (++spins >= a.spin_limit) {
                   failed = true;
                   break;
                 }
@@ -657,7 +661,14 @@ void onesweep_kernel(const SweepArgs<BIG> a_in)
   // Tiles are handed out in launch order of the workgroups that are actually running, so
   // every tile a look-back waits for belongs to a resident workgroup.
   if (tid == 0) {
-    sh.tile = __hip_atomic_fetch_add(a.ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // Once a tile of an earlier pass has given up, the keys in flight no longer match the
+    // histograms the offsets come from, and a pass working on them could write past a row:
+    // nothing more is sorted then.  (An ordinary load: what earlier launches wrote is visible
+    // at the start of this one.  A failure inside this pass leaves its input consistent, every
+    // offset stays inside the row, and waiting tiles notice the status word and drain.)
+    const uint32_t ticket = __hip_atomic_fetch_add(a.ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint32_t failed = *a.status;
+    sh.tile               = (failed != 0) ? 0xFFFFFFFFu : ticket;
   }
   for (int j = tid; j < WAVES * RADIX; j += BLOCK) {
     sh.ctr[j] = 0;
@@ -665,7 +676,7 @@ void onesweep_kernel(const SweepArgs<BIG> a_in)
   __syncthreads();
   const uint32_t tile = sh.tile;
   if (tile >= a.num_tiles) {
-    return;  // uniform per block; cannot happen when grid == num_tiles
+    return;  // uniform per block: the sort has failed, see above (grid == num_tiles otherwise)
   }
   const uint64_t row    = tile / a.tiles_per_row;
   const uint32_t trow   = tile - static_cast<uint32_t>(row * a.tiles_per_row);

@@ -41,6 +41,10 @@ uint64_t wide_row_threshold()
   return (t < 0 || static_cast<uint64_t>(t) > BIG_ROW_ELEMENTS) ? BIG_ROW_ELEMENTS : static_cast<uint64_t>(t);
 }
 
+static std::atomic<long long> g_spin_limit{static_cast<long long>(LOOKBACK_SPIN_LIMIT)};
+
+uint32_t lookback_spin_limit() { return static_cast<uint32_t>(g_spin_limit.load(std::memory_order_relaxed)); }
+
 uint64_t wave_row_limit()
 {
   const long long limit = g_wave_row_limit.load(std::memory_order_relaxed);
@@ -89,6 +93,12 @@ int64_t cpn_set_lds_row_limit(int64_t limit)
 int64_t cpn_set_wide_row_threshold(int64_t elements)
 {
   return static_cast<int64_t>(cpn::g_wide_row_threshold.exchange(elements < 0 ? -1ll : static_cast<long long>(elements)));
+}
+
+int64_t cpn_set_lookback_spin_limit(int64_t polls)
+{
+  const long long v = (polls < 1 || polls > (1ll << 31)) ? static_cast<long long>(cpn::LOOKBACK_SPIN_LIMIT) : polls;
+  return static_cast<int64_t>(cpn::g_spin_limit.exchange(v));
 }
 
 int64_t cpn_set_wave_row_limit(int64_t limit)

@@ -31,12 +31,13 @@ extern thread_local int g_last_hip_error;
   } while (0)
 
 constexpr uint64_t WORKSPACE_ALIGN  = 256;
-// Workspace header: [0] status word, [64..) tile tickets, [192..) per-pass "digit varies" flags,
-// [320..) the device-side SortPlan.
+// Workspace header: [0] status word, [128..) tile tickets, [256..) per-pass "digit varies" flags,
+// [384..) the device-side SortPlan.  The status word has a 128-byte line to itself: every tile
+// reads it with an ordinary load, and the tickets next door are under constant atomic traffic.
 constexpr uint64_t HEADER_BYTES     = 1024;
-constexpr uint64_t HEADER_TICKETS   = 64;
-constexpr uint64_t HEADER_VARYING   = 192;
-constexpr uint64_t HEADER_PLAN      = 320;
+constexpr uint64_t HEADER_TICKETS   = 128;
+constexpr uint64_t HEADER_VARYING   = 256;
+constexpr uint64_t HEADER_PLAN      = 384;
 static_assert(HEADER_TICKETS + 4 * MAX_PASSES <= HEADER_VARYING, "tickets overlap the flags");
 static_assert(HEADER_VARYING + 4 * MAX_PASSES <= HEADER_PLAN, "flags overlap the plan");
 static_assert(HEADER_PLAN + sizeof(SortPlan) <= HEADER_BYTES, "plan does not fit the header");
@@ -428,6 +429,7 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
     a.tiles_per_row      = L.tiles_per_row;
     a.num_tiles          = static_cast<uint32_t>(L.num_tiles);
     a.pass               = p;
+    a.spin_limit         = lookback_spin_limit();
     {
       ProfileScope prof("onesweep", r.stream);
       const dim3 grid(static_cast<uint32_t>(L.num_tiles));

@@ -97,6 +97,15 @@ int64_t cpn_set_wave_row_limit(int64_t limit);
  */
 int64_t cpn_set_wide_row_threshold(int64_t elements);
 
+/*
+ * Process-wide tunable: how many times a tile of the global path polls the descriptor of a
+ * predecessor before it gives up, sets the device status word (CPN_ERR_DEVICE from
+ * cpn_local_sort_check) and lets every kernel run to its end with invalid output.  The default
+ * (2^22 polls, restored by a value below 1) is far above any real wait; tests of the failure
+ * path set 1.  The previous setting is returned.
+ */
+int64_t cpn_set_lookback_spin_limit(int64_t polls);
+
 /* Size in bytes of one element of `dtype`, or 0 for an unknown code. */
 uint64_t cpn_dtype_size(int dtype);
 

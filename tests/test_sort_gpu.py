@@ -548,3 +548,48 @@ def test_concurrent_streams_and_threads(lib, torch_cuda):
     for t in threads:
         t.join()
     assert not errors, errors
+
+
+# ---- failure path of the bounded look-back wait -------------------------------------------------------
+def test_lookback_gives_up_cleanly(lib, torch_cuda):
+    """With the spin limit forced to one poll, a tile whose predecessor has not answered yet gives up:
+    every kernel still runs to its end, nothing is written out of bounds, and the device status word
+    reports the failure (CPN_ERR_DEVICE) instead of a hang or a silently wrong result.  Whether a given
+    run hits an unanswered poll depends on timing, so a clean run must be fully correct and at least
+    one of several runs over a thousand tiles is expected to report the failure."""
+    torch = torch_cuda
+    dev = torch.device("cuda")
+    n = 1 << 24
+    rng = np.random.default_rng(6)
+    x = rng.integers(0, 1 << 31, n).astype(np.int32)
+    code = _lib.DTYPE_CODES[np.dtype(np.int32)]
+    d_in = torch.from_numpy(x).to(dev)
+    guard = 4096
+    d_out = torch.full((n + 2 * guard,), -1, dtype=torch.int32, device=dev)  # canaries on both sides
+    out = d_out[guard : guard + n]
+    tb = lib.cpn_local_sort_temp_bytes(code, n, n, 1, 0, 0)
+    temp = torch.empty(tb, dtype=torch.uint8, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    want = None
+    seen_failure = False
+    prev = lib.cpn_set_lookback_spin_limit(1)
+    try:
+        for _ in range(5):
+            rc = lib.cpn_local_sort(code, d_in.data_ptr(), out.data_ptr(), None, n, n, 0, 1, temp.data_ptr(), tb, stream)
+            assert rc == 0
+            status = lib.cpn_local_sort_check(temp.data_ptr(), stream)
+            assert status in (0, _lib.CPN_ERR_DEVICE)
+            assert bool((d_out[:guard] == -1).all()) and bool((d_out[guard + n :] == -1).all()), "wrote outside the output"
+            if status == 0:
+                if want is None:
+                    want = np.sort(x, kind="stable")
+                assert np.array_equal(out.cpu().numpy(), want)
+            else:
+                seen_failure = True
+    finally:
+        assert lib.cpn_set_lookback_spin_limit(prev) == 1
+    assert seen_failure, "no run reported a failed look-back although tiles were told not to wait"
+    # back at the default limit the same call succeeds
+    assert lib.cpn_local_sort(code, d_in.data_ptr(), out.data_ptr(), None, n, n, 0, 1, temp.data_ptr(), tb, stream) == 0
+    assert lib.cpn_local_sort_check(temp.data_ptr(), stream) == 0
+    assert np.array_equal(out.cpu().numpy(), np.sort(x, kind="stable") if want is None else want)
