@@ -116,6 +116,17 @@ def algorithmic_bytes(cfg: dict, lds_limit_rows: bool) -> dict:
         out["onesweep_per_pass"] = per_pass
         out["onesweep"] = sum(per_pass) / passes  # average launch
         out["histogram"] = n * kb
+        # the same passes counted with the baseline's formula, which carries the payload at its final
+        # width (vb = 8) through every pass: r_1 = kb, r_p = w_p = kb + vb, w_P = vb for index-only output
+        vb = 8 if argsort else 0
+        formula = []
+        for p in range(passes):
+            first, last = p == 0, p == passes - 1
+            r = kb if first else kb + vb
+            w = vb if (last and argsort) else kb + vb
+            formula.append(n * (r + w))
+        out["onesweep_baseline_formula"] = sum(formula) / passes
+        out["whole_baseline_formula"] = n * kb + sum(formula)
     if cfg["axis"] == 0:
         out["transpose_last"] = n * 2 * kb
     return out
@@ -575,6 +586,12 @@ def main() -> None:
         "avg_launch_ms": avg_ms,
         "launches_per_step": len(by_label[dominant]) / args.steps,
     }
+    if "onesweep_baseline_formula" in alg and dominant == "onesweep":
+        # for comparison only: the baseline's accounting moves an 8-byte payload in every pass, this
+        # build moves 4-byte row positions, so `achieved` above is the smaller, real figure
+        fb = alg["onesweep_baseline_formula"]
+        roofline["baseline_formula"] = {"bytes_per_launch": fb, "achieved": fb / (avg_ms * 1e-3) / 1e9,
+                                        "frac": fb / (avg_ms * 1e-3) / HBM_PEAK_BYTES_PER_S}
     step_bytes = sum(alg.get(k, 0) * len(v) / args.steps for k, v in by_label.items() if k in alg)
 
     line = {
@@ -596,7 +613,10 @@ def main() -> None:
                    "workspace_bytes": int(job.temp_bytes)},
         "roofline": roofline,
         "whole_step": {"algorithmic_bytes": step_bytes, "GBps": step_bytes / (elapsed / args.steps) / 1e9,
-                       "frac_of_hbm_peak": step_bytes / (elapsed / args.steps) / HBM_PEAK_BYTES_PER_S},
+                       "frac_of_hbm_peak": step_bytes / (elapsed / args.steps) / HBM_PEAK_BYTES_PER_S,
+                       **({"baseline_formula_bytes": alg["whole_baseline_formula"],
+                           "baseline_formula_frac": alg["whole_baseline_formula"] / (elapsed / args.steps)
+                           / HBM_PEAK_BYTES_PER_S} if "whole_baseline_formula" in alg else {})},
         "kernels": kernels,
         "verify": verify_sample(job, cfg),
     }

@@ -27,6 +27,8 @@ def test_algorithmic_bytes_of_the_headline_workload():
     assert alg["onesweep"] == n * 15 and alg["histogram"] == n * 4
     total = alg["histogram"] + sum(alg["onesweep_per_pass"])
     assert total == n * 64
+    # the baseline's own accounting (8-byte payload in every pass): N*88 for this workload
+    assert alg["whole_baseline_formula"] == n * 88 and alg["onesweep_baseline_formula"] == n * 21
     # keys-only int32 sort: every pass reads and writes the key
     alg1 = bench.algorithmic_bytes(bench.make_config("c1", log2n=16), lds_limit_rows=False)
     assert alg1["onesweep_per_pass"] == [(1 << 16) * 8] * 4
