@@ -20,6 +20,7 @@
 #include <stdint.h>
 
 #include "radix_common.h"
+#include "virtual_digits.h"
 
 namespace cpn {
 
@@ -189,8 +190,14 @@ template <typename OffT>
 __global__ __launch_bounds__(RADIX) void histogram_scan_kernel(OffT* __restrict__ hist,
                                                                uint32_t* __restrict__ varying,
                                                                uint64_t seg,
-                                                               uint32_t passes)
+                                                               uint32_t passes,
+                                                               const VirtPlan* __restrict__ vplan)
 {
+  // second use, after vplan_kernel: scans the histograms of the virtual digits (one row, block =
+  // group) and nothing when the plan stayed disabled
+  if (vplan != nullptr && (vplan->enabled == 0 || blockIdx.x >= vplan->n_groups)) {
+    return;
+  }
   __shared__ OffT s_wsum[RADIX / WAVE];
   const int tid  = threadIdx.x;
   const int lane = tid & (WAVE - 1);
@@ -352,6 +359,7 @@ struct SweepArgs {
   int pass;                // which 8-bit digit this pass sorts by
   int idx_final;           // idx_out is the caller's int64 array
   uint32_t spin_limit;     // polls of one descriptor before the tile gives up (LOOKBACK_SPIN_LIMIT)
+  const VirtPlan* vplan;   // virtual digits (virtual_digits.h), nullptr when the request cannot use them
 };
 
 #ifndef CPN_ONESWEEP_WAVES_PER_EU
@@ -376,9 +384,12 @@ struct SweepShared {
 // unsigned image as soon as they are loaded and writes them out that way; every pass extracts
 // digits with the identity codec, so the key transform is paid once per key instead of twice
 // per pass.  The values themselves are never returned in that case.
-template <typename KeyT, int CODEC, bool XFORM, bool BIG, bool HAS_IDX, int BLOCK, int ITEMS, bool FULL>
+template <typename KeyT, int CODEC, bool XFORM, bool BIG, bool HAS_IDX, int BLOCK, int ITEMS, bool FULL, bool VIRT>
 __device__ __forceinline__ void onesweep_tile(
   const SweepArgs<BIG>& a,
+  const uint32_t vcount,    // VIRT: positions in this pass's group, their bit offsets (8 bits each)
+  const uint64_t voffsets,  //       and their shifted lookup tables in LDS (virtual_digits.h)
+  const uint8_t* vlut,
   SweepShared<KeyT, typename RowWidth<BIG>::off_t, BLOCK / WAVE, BLOCK * ITEMS,
               ((HAS_IDX && sizeof(typename RowWidth<BIG>::off_t) > sizeof(KeyT)) ? sizeof(typename RowWidth<BIG>::off_t)
                                                                                 : sizeof(KeyT))>& sh,
@@ -427,7 +438,14 @@ __device__ __forceinline__ void onesweep_tile(
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const bool valid = FULL || (woff + i * WAVE < count);
-    const uint32_t d = KeyTraits<DCODEC, KeyT>::digit(key[i], a.pass);
+    uint32_t d;
+    if constexpr (VIRT) {
+      uint64_t ow[KeyTraits<DCODEC, KeyT>::NWORDS];
+      KeyTraits<DCODEC, KeyT>::words(key[i], ow);
+      d = virtual_digit(ow[0], vcount, voffsets, vlut);
+    } else {
+      d = KeyTraits<DCODEC, KeyT>::digit(key[i], a.pass);
+    }
     dpk[i / 4]       = (i % 4 == 0) ? d : (dpk[i / 4] | (d << (8 * (i % 4))));
     const uint32_t r = wave_match_rank(d, valid, wctr) & 0xFFFFu;
     rnk2[i / 2]      = (i % 2 == 0) ? r : (rnk2[i / 2] | (r << 16));
@@ -571,7 +589,14 @@ __device__ __forceinline__ void onesweep_tile(
     }
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
-      const uint32_t d = KeyTraits<DCODEC, KeyT>::digit(kk[k], a.pass);
+      uint32_t d;
+      if constexpr (VIRT) {
+        uint64_t ow[KeyTraits<DCODEC, KeyT>::NWORDS];
+        KeyTraits<DCODEC, KeyT>::words(kk[k], ow);
+        d = virtual_digit(ow[0], vcount, voffsets, vlut);
+      } else {
+        d = KeyTraits<DCODEC, KeyT>::digit(kk[k], a.pass);
+      }
       dq[k / 4]        = (k % 4 == 0) ? d : (dq[k / 4] | (d << (8 * (k % 4))));
     }
     if (a.keys_out != nullptr) {
@@ -631,10 +656,16 @@ __device__ __forceinline__ void onesweep_tile(
   }
 }
 
-template <typename KeyT, int CODEC, bool XFORM, bool BIG, bool HAS_IDX, int BLOCK, int ITEMS>
+template <typename KeyT, int CODEC, bool XFORM, bool BIG, bool HAS_IDX, int BLOCK, int ITEMS, bool VIRT = false>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(CPN_ONESWEEP_WAVES_PER_EU)))
 void onesweep_kernel(const SweepArgs<BIG> a_in)
 {
+  static_assert(!VIRT || (KeyTraits<CODEC, KeyT>::NWORDS == 1 && sizeof(KeyT) <= 8), "virtual digits: one ordered word");
+  // VIRT kernels can do both: the device-side plan says whether this sort runs on virtual digits
+  bool virt_on = false;
+  if constexpr (VIRT) {
+    virt_on = (a_in.vplan != nullptr) && (a_in.vplan->enabled != 0);
+  }
   using OffT = typename RowWidth<BIG>::off_t;
   static_assert(BLOCK >= RADIX, "one thread per digit is needed for the look-back");
   static_assert(ITEMS % 4 == 0, "digits are cached four to a register");
@@ -644,10 +675,26 @@ void onesweep_kernel(const SweepArgs<BIG> a_in)
   static_assert(TILE <= 65536, "positions inside a tile are kept in 16 bits");
 
   __shared__ SweepShared<KeyT, OffT, WAVES, TILE, STAGE_ELEM> sh;
+  __shared__ uint8_t s_vlut[VIRT ? VIRT_MAX_POSITIONS * RADIX : 1];
+  uint32_t vcount   = 0;
+  uint64_t voffsets = 0;
 
   const PassPlan pp = a_in.plan->pass[a_in.pass];
   if (pp.active == 0) {
     return;  // every key of every row has the same digit here
+  }
+  if (VIRT && virt_on) {
+    // this pass's group: the tables of its byte positions, codes shifted into place (made visible
+    // by the barrier below), and the bit offsets of the bytes
+    const VirtGroup& g = a_in.vplan->group[a_in.pass];
+    vcount             = g.count;
+    for (uint32_t j = 0; j < vcount; ++j) {
+      voffsets |= static_cast<uint64_t>(g.pos[j] * RADIX_BITS) << (8 * j);
+    }
+    for (uint32_t j = threadIdx.x; j < vcount * RADIX; j += BLOCK) {
+      const uint32_t which = j / RADIX;
+      s_vlut[j] = static_cast<uint8_t>(a_in.vplan->lut[g.pos[which]][j % RADIX] << g.shift[which]);
+    }
   }
   SweepArgs<BIG> a = a_in;
   a.keys_in        = a_in.key_buf[pp.key_src];
@@ -681,10 +728,21 @@ void onesweep_kernel(const SweepArgs<BIG> a_in)
   const uint64_t row    = tile / a.tiles_per_row;
   const uint32_t trow   = tile - static_cast<uint32_t>(row * a.tiles_per_row);
   const uint64_t remain = a.seg - static_cast<uint64_t>(trow) * TILE;
+  if (VIRT && virt_on) {  // uniform for the launch
+    if (remain >= static_cast<uint64_t>(TILE)) {
+      onesweep_tile<KeyT, CODEC, XFORM, BIG, HAS_IDX, BLOCK, ITEMS, true, VIRT>(a, vcount, voffsets, s_vlut, sh, tile, row,
+                                                                               trow, TILE);
+    } else {
+      onesweep_tile<KeyT, CODEC, XFORM, BIG, HAS_IDX, BLOCK, ITEMS, false, VIRT>(a, vcount, voffsets, s_vlut, sh, tile, row,
+                                                                                trow, static_cast<uint32_t>(remain));
+    }
+    return;
+  }
   if (remain >= static_cast<uint64_t>(TILE)) {
-    onesweep_tile<KeyT, CODEC, XFORM, BIG, HAS_IDX, BLOCK, ITEMS, true>(a, sh, tile, row, trow, TILE);
+    onesweep_tile<KeyT, CODEC, XFORM, BIG, HAS_IDX, BLOCK, ITEMS, true, false>(a, 0u, 0ull, nullptr, sh, tile, row, trow, TILE);
   } else {
-    onesweep_tile<KeyT, CODEC, XFORM, BIG, HAS_IDX, BLOCK, ITEMS, false>(a, sh, tile, row, trow, static_cast<uint32_t>(remain));
+    onesweep_tile<KeyT, CODEC, XFORM, BIG, HAS_IDX, BLOCK, ITEMS, false, false>(a, 0u, 0ull, nullptr, sh, tile, row, trow,
+                                                                                static_cast<uint32_t>(remain));
   }
 }
 

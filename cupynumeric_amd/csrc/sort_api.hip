@@ -45,6 +45,13 @@ static std::atomic<long long> g_spin_limit{static_cast<long long>(LOOKBACK_SPIN_
 
 uint32_t lookback_spin_limit() { return static_cast<uint32_t>(g_spin_limit.load(std::memory_order_relaxed)); }
 
+static std::atomic<long long> g_virt_threshold{[] {
+  const char* e = getenv("CPN_SORT_VIRTUAL_DIGIT_THRESHOLD");
+  return (e != nullptr && *e != 0) ? atoll(e) : static_cast<long long>(VIRT_MIN_ROW_ELEMENTS);
+}()};
+
+uint64_t virtual_digit_threshold() { return static_cast<uint64_t>(g_virt_threshold.load(std::memory_order_relaxed)); }
+
 uint64_t wave_row_limit()
 {
   const long long limit = g_wave_row_limit.load(std::memory_order_relaxed);
@@ -93,6 +100,12 @@ int64_t cpn_set_lds_row_limit(int64_t limit)
 int64_t cpn_set_wide_row_threshold(int64_t elements)
 {
   return static_cast<int64_t>(cpn::g_wide_row_threshold.exchange(elements < 0 ? -1ll : static_cast<long long>(elements)));
+}
+
+int64_t cpn_set_virtual_digit_threshold(int64_t elements)
+{
+  const long long v = elements < 0 ? static_cast<long long>(cpn::VIRT_MIN_ROW_ELEMENTS) : static_cast<long long>(elements);
+  return static_cast<int64_t>(cpn::g_virt_threshold.exchange(v));
 }
 
 int64_t cpn_set_lookback_spin_limit(int64_t polls)

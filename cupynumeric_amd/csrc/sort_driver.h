@@ -42,6 +42,11 @@ static_assert(HEADER_TICKETS + 4 * MAX_PASSES <= HEADER_VARYING, "tickets overla
 static_assert(HEADER_VARYING + 4 * MAX_PASSES <= HEADER_PLAN, "flags overlap the plan");
 static_assert(HEADER_PLAN + sizeof(SortPlan) <= HEADER_BYTES, "plan does not fit the header");
 constexpr uint64_t BIG_ROW_ELEMENTS = 1ull << 30;
+// Shortest row for which virtual digits are considered: their extra launches (three small kernels
+// and an early-exiting twin of every pass) cost about 0.1 ms, 2 % of a 2^26-key sort of 8-byte keys.
+constexpr uint64_t VIRT_MIN_ROW_ELEMENTS = 1ull << 26;
+// The threshold in force (cpn_set_virtual_digit_threshold; tests lower it).
+uint64_t virtual_digit_threshold();
 // Rows of at least this many elements use 64-bit counts, descriptors and row positions:
 // BIG_ROW_ELEMENTS unless lowered by cpn_set_wide_row_threshold / CPN_SORT_WIDE_ROW_THRESHOLD
 // (for tests that exercise the 64-bit kernels without a 2^30-element row).
@@ -130,6 +135,8 @@ struct SortRequest {
 // Workspace layout of the global path.  Everything in [0, zero_bytes) is cleared per call.
 struct GlobalLayout {
   bool big;
+  bool virt;          // the request may use virtual digits (virtual_digits.h): a VirtPlan slot follows the header
+  uint64_t off_virt;
   int passes;
   uint64_t rows;
   uint32_t tiles_per_row;
@@ -156,7 +163,12 @@ inline GlobalLayout global_layout(int key_bytes, int passes, uint64_t volume, ui
   L.valid             = (tpr < (1ull << 32)) && (L.num_tiles < (1ull << 32));
   L.tiles_per_row     = static_cast<uint32_t>(tpr);
   const uint64_t ow   = L.big ? 8 : 4;
-  L.off_hist          = HEADER_BYTES;
+  // virtual digits: one long row of real 8-byte keys.  Their extra launches (three small kernels
+  // and one early-exiting twin per pass, about 10 us each at this grid size) cost a 2^28-key sort
+  // of 4-byte keys 2 %, more than four passes can win back on average; eight passes can.
+  L.virt     = (L.rows == 1) && !L.big && (key_bytes == 8) && (passes == key_bytes) && (seg >= virtual_digit_threshold());
+  L.off_virt = L.virt ? HEADER_BYTES : 0;
+  L.off_hist          = HEADER_BYTES + (L.virt ? VIRT_PLAN_BYTES : 0);
   L.hist_bytes        = align_up(L.rows * L.passes * RADIX * ow, WORKSPACE_ALIGN);
   L.off_desc          = L.off_hist + L.hist_bytes;
   L.desc_bytes_per_pass = align_up(L.num_tiles * RADIX * ow, WORKSPACE_ALIGN);
@@ -364,6 +376,8 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
   uint32_t* tickets = reinterpret_cast<uint32_t*>(ws + HEADER_TICKETS);
   uint32_t* varying = reinterpret_cast<uint32_t*>(ws + HEADER_VARYING);
   SortPlan* plan    = reinterpret_cast<SortPlan*>(ws + HEADER_PLAN);
+  constexpr bool VIRT_OK = !BIG && KB == 8 && KeyTraits<CODEC, KeyT>::PASSES == KB;
+  VirtPlan* vplan   = L.virt ? reinterpret_cast<VirtPlan*>(ws + L.off_virt) : nullptr;
   OffT* hist        = reinterpret_cast<OffT*>(ws + L.off_hist);
   static_assert(PASSES <= MAX_PASSES, "plan table too small");
   PlanRequest rq{};
@@ -400,9 +414,35 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
     {
       ProfileScope prof("histogram_scan", r.stream);
       hipLaunchKernelGGL((histogram_scan_kernel<OffT>), dim3(static_cast<uint32_t>(L.rows * PASSES)),
-                         dim3(RADIX), 0, r.stream, hist, varying, r.seg, static_cast<uint32_t>(PASSES));
+                         dim3(RADIX), 0, r.stream, hist, varying, r.seg, static_cast<uint32_t>(PASSES),
+                         static_cast<const VirtPlan*>(nullptr));
     }
     CPN_HIP_TRY(hipGetLastError());
+    if constexpr (VIRT_OK) {
+      if (L.virt) {
+        // may replace the byte passes by fewer passes on virtual digits (decided on the device)
+        {
+          ProfileScope prof("virtual_plan", r.stream);
+          hipLaunchKernelGGL((vplan_kernel<OffT>), dim3(1), dim3(RADIX), 0, r.stream, hist, varying, vplan, r.seg,
+                             static_cast<uint32_t>(PASSES));
+        }
+        CPN_HIP_TRY(hipGetLastError());
+        {
+          const uint64_t vchunk = 65536;
+          const uint64_t vgrid  = (r.seg + vchunk - 1) / vchunk;
+          ProfileScope prof("virtual_histogram", r.stream);
+          hipLaunchKernelGGL((vhist_kernel<KeyT, CODEC, OffT>), dim3(static_cast<uint32_t>(vgrid)), dim3(VHIST_BLOCK), 0,
+                             r.stream, static_cast<const KeyT*>(r.values_in), hist, vplan, r.seg, vchunk);
+        }
+        CPN_HIP_TRY(hipGetLastError());
+        {
+          ProfileScope prof("virtual_scan", r.stream);
+          hipLaunchKernelGGL((histogram_scan_kernel<OffT>), dim3(static_cast<uint32_t>(PASSES)), dim3(RADIX), 0,
+                             r.stream, hist, varying, r.seg, static_cast<uint32_t>(PASSES), vplan);
+        }
+        CPN_HIP_TRY(hipGetLastError());
+      }
+    }
     {
       ProfileScope prof("plan", r.stream);
       hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(WAVE), 0, r.stream, varying, plan, rq);
@@ -442,12 +482,31 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
     a.num_tiles          = static_cast<uint32_t>(L.num_tiles);
     a.pass               = p;
     a.spin_limit         = lookback_spin_limit();
+    a.vplan              = vplan;
     {
       ProfileScope prof("onesweep", r.stream);
       const dim3 grid(static_cast<uint32_t>(L.num_tiles));
+      // requests that may run on virtual digits get the kernel that can do both (the device-side
+      // plan decides); everything else the plain one
       bool launched = false;
+      if constexpr (VIRT_OK) {
+        if (L.virt) {
+          if constexpr (CAN_ORDER_KEYS) {
+            if (ordered_keys) {
+              hipLaunchKernelGGL((onesweep_kernel<KeyT, CODEC, true, BIG, HAS_IDX, BLOCK, ITEMS, true>), grid,
+                                 dim3(BLOCK), 0, r.stream, a);
+              launched = true;
+            }
+          }
+          if (!launched) {
+            hipLaunchKernelGGL((onesweep_kernel<KeyT, CODEC, false, BIG, HAS_IDX, BLOCK, ITEMS, true>), grid,
+                               dim3(BLOCK), 0, r.stream, a);
+            launched = true;
+          }
+        }
+      }
       if constexpr (CAN_ORDER_KEYS) {
-        if (ordered_keys) {
+        if (!launched && ordered_keys) {
           hipLaunchKernelGGL((onesweep_kernel<KeyT, CODEC, true, BIG, HAS_IDX, BLOCK, ITEMS>), grid, dim3(BLOCK), 0,
                              r.stream, a);
           launched = true;

@@ -106,6 +106,18 @@ int64_t cpn_set_wide_row_threshold(int64_t elements);
  */
 int64_t cpn_set_lookback_spin_limit(int64_t polls);
 
+/*
+ * Process-wide tunable: a 1-D sort of real 8-byte keys with at least `elements` elements lets
+ * the device replace its eight byte passes by fewer passes on "virtual digits" when the
+ * histograms show that the bytes of the keys take few distinct values (several bytes then
+ * share one 8-bit digit; cupynumeric_amd/csrc/virtual_digits.h).  Results do not depend on
+ * it.  The default is 2^26 (below that the extra launches outweigh the average gain); a
+ * negative value restores it and the previous setting is returned.  It changes workspace
+ * sizes by 4096 bytes (cpn_local_sort_temp_bytes follows).  Also initialised from the
+ * environment variable CPN_SORT_VIRTUAL_DIGIT_THRESHOLD.
+ */
+int64_t cpn_set_virtual_digit_threshold(int64_t elements);
+
 /* Size in bytes of one element of `dtype`, or 0 for an unknown code. */
 uint64_t cpn_dtype_size(int dtype);
 

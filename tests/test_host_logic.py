@@ -92,6 +92,7 @@ def test_temp_bytes_layout(lib):
     assert tb(f32, 1 << 20, 1024, 1, 1, 0) == header  # rows that fit LDS need only the header
     n = 1 << 24
     tiles = n // 16384  # 512 threads x 32 keys per tile for keys of up to 4 bytes
+
     fixed = header + 4 * 256 * 4 + 4 * tiles * 256 * 4
     assert tb(f32, n, n, 1, 0, 0) == fixed + 4 * n  # one key buffer
     assert tb(f32, n, n, 1, 0, 1) == fixed + 2 * 4 * n  # in place: a second buffer, in case an odd number of passes runs

@@ -595,3 +595,59 @@ def test_lookback_gives_up_cleanly(lib, torch_cuda):
     assert np.array_equal(out.cpu().numpy(), np.sort(x, kind="stable") if want is None else want)
     if not seen_failure:  # timing: every poll of every tile happened to be answered at once
         pytest.skip("no look-back had to wait in five runs, the failure path was not reached")
+
+
+# ---- virtual digits: fewer passes for keys whose bytes take few distinct values ---------------------
+def _few_values(rng, dtype, n, distinct):
+    """n keys drawn from `distinct` arbitrary values of `dtype` (every byte position busy, few values each)."""
+    dt = np.dtype(dtype)
+    if dt.kind == "f":
+        pool = rng.standard_normal(distinct).astype(dtype) * dtype(1000.0)
+        pool[: min(3, distinct)] = [np.nan, -0.0, 0.0][: min(3, distinct)]
+    else:
+        info = np.iinfo(dtype)
+        pool = rng.integers(info.min, info.max, distinct, dtype=dtype, endpoint=True)
+    return pool[rng.integers(0, distinct, n)]
+
+
+@pytest.fixture()
+def virtual_digits_from_2_to_20(lib):
+    """Virtual digits are considered from 2^26 elements on by default; the tests lower that."""
+    prev = lib.cpn_set_virtual_digit_threshold(1 << 20)
+    yield
+    lib.cpn_set_virtual_digit_threshold(prev)
+
+
+@pytest.mark.parametrize("dtype", [np.int64, np.uint64, np.float64, np.int32, np.float32])
+def test_virtual_digits(lib, torch_cuda, virtual_digits_from_2_to_20, dtype):
+    """One long row of 8-byte keys (4-byte keys run alongside: they never use virtual digits and must
+    not be disturbed): with 16 distinct values every byte
+    carries 4 bits and pairs of bytes are sorted in one pass; with 3 distinct values four bytes share a
+    pass; with 300 values some bytes are too busy to share; random keys keep the ordinary passes.  Every
+    output form is compared with the oracle bit for bit."""
+    rng = np.random.default_rng(np.dtype(dtype).num)
+    n = (1 << 21) + 1234
+    for distinct in (16, 3, 300, 2):
+        x = _few_values(rng, dtype, n, distinct)
+        want_v = oracle.local_sort(x, argsort=False, threads=8)
+        want_i = oracle.local_sort(x, argsort=True, threads=8)
+        v, _ = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=False)
+        assert_same_bits(v, want_v, f"{np.dtype(dtype)} {distinct} values, sort")
+        _, i = abi_sort(lib, torch_cuda, x, want_values=False, want_indices=True)
+        assert_same_bits(i, want_i, f"{np.dtype(dtype)} {distinct} values, argsort")
+        if distinct == 16:
+            v, i = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=True, in_place=True, offset=5)
+            assert_same_bits(v, want_v, "in place + indices")
+            assert_same_bits(i, want_i + 5, "in place + indices")
+            v, _ = abi_sort(lib, torch_cuda, x, want_values=True, in_place=True)
+            assert_same_bits(v, want_v, "in place")
+    # bytes with few values next to bytes with all 256: only some positions share a pass
+    if np.dtype(dtype).kind != "f":
+        hi = rng.integers(0, 7, n).astype(np.uint64) << np.uint64(8 * (np.dtype(dtype).itemsize - 1) - 1)
+        lo = rng.integers(0, 1 << 16, n).astype(np.uint64)
+        x = (hi | lo).astype(np.dtype(dtype).str.replace("i", "u")).view(dtype)
+        _, i = abi_sort(lib, torch_cuda, x, want_values=False, want_indices=True)
+        assert_same_bits(i, oracle.local_sort(x, argsort=True, threads=8), "mixed busy and quiet bytes")
+    # short rows and several rows never use virtual digits; same answers
+    x = _few_values(rng, dtype, 3 * 100_000, 16).reshape(3, 100_000)
+    check_rows(lib, torch_cuda, x, f"{np.dtype(dtype)} short rows of few values")
