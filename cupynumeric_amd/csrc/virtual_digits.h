@@ -157,10 +157,14 @@ __global__ __launch_bounds__(VHIST_BLOCK) void vhist_kernel(const KeyT* __restri
                                                              uint64_t seg,
                                                              uint64_t chunk)
 {
-  constexpr int COPIES = 4;
+  constexpr int COPIES    = 4;
+  constexpr int POSITIONS = static_cast<int>(sizeof(KeyT));  // byte positions of the ordered key
+  static_assert(POSITIONS <= VIRT_MAX_POSITIONS, "keys of at most 8 bytes");
   __shared__ uint32_t s_hist[VIRT_MAX_POSITIONS * RADIX * COPIES];
-  __shared__ uint8_t s_lut[VIRT_MAX_POSITIONS * RADIX];  // [byte position][256]
-  __shared__ VirtGroup s_group[VIRT_MAX_POSITIONS];
+  // per byte position: byte value -> code, already shifted to its place inside the digit of its
+  // group (all zero for positions that belong to no group)
+  __shared__ uint8_t s_tab[VIRT_MAX_POSITIONS * RADIX];
+  __shared__ uint32_t s_ends;  // bit p: position p is the last one of its group
   if (plan->enabled == 0) {
     return;
   }
@@ -170,12 +174,24 @@ __global__ __launch_bounds__(VHIST_BLOCK) void vhist_kernel(const KeyT* __restri
     s_hist[j] = 0;
   }
   for (int j = tid; j < VIRT_MAX_POSITIONS * RADIX; j += VHIST_BLOCK) {
-    s_lut[j] = plan->lut[j / RADIX][j % RADIX];
-  }
-  if (tid < static_cast<int>(groups)) {
-    s_group[tid] = plan->group[tid];
+    s_tab[j] = 0;
   }
   __syncthreads();
+  uint32_t ends = 0;
+  for (uint32_t g = 0; g < groups; ++g) {
+    const VirtGroup& grp = plan->group[g];
+    for (uint32_t j = 0; j < grp.count; ++j) {
+      const uint32_t p = grp.pos[j];
+      s_tab[p * RADIX + tid] = static_cast<uint8_t>(plan->lut[p][tid] << grp.shift[j]);  // VHIST_BLOCK == RADIX
+    }
+    ends |= 1u << grp.pos[grp.count - 1];
+  }
+  static_assert(VHIST_BLOCK == RADIX, "one thread per table entry");
+  if (tid == 0) {
+    s_ends = ends;
+  }
+  __syncthreads();
+  ends = s_ends;
   const uint64_t begin = static_cast<uint64_t>(blockIdx.x) * chunk;
   uint64_t end         = begin + chunk;
   if (end > seg) {
@@ -187,14 +203,15 @@ __global__ __launch_bounds__(VHIST_BLOCK) void vhist_kernel(const KeyT* __restri
   auto count_key = [&](KeyT raw) {
     uint64_t w[1];
     KeyTraits<CODEC, KeyT>::words(raw, w);
-    for (uint32_t g = 0; g < groups; ++g) {
-      uint32_t d = 0;
-      for (uint32_t j = 0; j < s_group[g].count; ++j) {
-        const uint32_t p    = s_group[g].pos[j];
-        const uint32_t byte = static_cast<uint32_t>(w[0] >> (p * RADIX_BITS)) & 0xFFu;
-        d |= static_cast<uint32_t>(s_lut[p * RADIX + byte]) << s_group[g].shift[j];
+    uint32_t acc = 0, g = 0;
+#pragma unroll
+    for (int p = 0; p < POSITIONS; ++p) {
+      acc |= s_tab[p * RADIX + (static_cast<uint32_t>(w[0] >> (p * RADIX_BITS)) & 0xFFu)];
+      if ((ends >> p) & 1u) {  // uniform
+        atomicAdd(&s_hist[(g * RADIX + acc) * COPIES + copy], 1u);
+        acc = 0;
+        ++g;
       }
-      atomicAdd(&s_hist[(g * RADIX + d) * COPIES + copy], 1u);
     }
   };
   // four keys per thread and step, their loads issued together
