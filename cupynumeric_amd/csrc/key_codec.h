@@ -71,6 +71,21 @@ __host__ __device__ __forceinline__ U ordered_bits(U raw)
   }
 }
 
+// The float image without the NaN and zero rules, and its inverse: a bijection of the bits that
+// agrees with ordered_bits<CODEC_FLOAT> on every value except NaNs and -0.0.
+template <typename U>
+__host__ __device__ __forceinline__ U sign_flip(U raw)
+{
+  constexpr U sign = FloatLayout<U>::sign;
+  return (raw & sign) ? static_cast<U>(~raw) : static_cast<U>(raw | sign);
+}
+template <typename U>
+__host__ __device__ __forceinline__ U sign_unflip(U image)
+{
+  constexpr U sign = FloatLayout<U>::sign;
+  return (image & sign) ? static_cast<U>(image ^ sign) : static_cast<U>(~image);
+}
+
 template <int CODEC, typename U>
 __host__ __device__ __forceinline__ uint32_t radix_digit(U raw, int shift)
 {

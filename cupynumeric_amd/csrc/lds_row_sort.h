@@ -14,15 +14,23 @@
 // varying bits.  When more passes than that are due, the kernel first runs only the passes of
 // the most significant varying digits, then checks that every neighbouring pair of the result
 // is in order on the whole key.  If so the row is sorted (stably: ties on the leading digits
-// whose remaining digits also tie kept their input order).  If not, all passes are run, from
-// the state reached, which is still a stable sort of the input.
+// whose remaining digits also tie kept their input order).  If a few pairs are not, rounds of
+// odd-even transposition between neighbours repair them; if that does not finish within
+// FIXUP_ROUNDS, all passes are run, from the state reached, which is still a stable sort of
+// the input.
+//
+// Floating-point rows without NaN and without -0.0 (found during the same reduction): on such
+// a row the ordered image of a key is a bijection of its bits, so the keys are replaced by
+// their images once, the passes take plain bytes of them, and the images are mapped back
+// before the store.  Rows with a NaN or a -0.0 keep the raw bits and apply the codec per pass
+// (so do all float16 rows and the rows sorted by 1024 threads).
 #pragma once
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
 #include "radix_common.h"
-#include "wave_row_sort.h"  // wave_all_and / wave_all_or
+#include "wave_row_sort.h"  // wave_all_and / wave_all_or, FIXUP_ROUNDS
 
 namespace cpn {
 
@@ -43,6 +51,9 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
   using SW             = unsigned long long;  // a key's digits, eight to a word, as shuffled across the wave
   using IdxS           = uint16_t;  // row position while staged in LDS
   static_assert(TILE <= 65536, "row positions are staged as 16 bits");
+  // not for 2-byte keys (their codec is cheap) nor for 1024 threads: there the second code path
+  // costs registers beyond the 64 that let two workgroups share a CU
+  constexpr bool IMAGES_OK = (CODEC == CODEC_FLOAT) && sizeof(KeyT) >= 4 && BLOCK <= 512;
 
   __shared__ __align__(16) KeyT s_keys[TILE];
   __shared__ IdxS s_idx[HAS_IDX ? TILE : 1];
@@ -60,6 +71,7 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
   KeyT key[ITEMS];
   uint32_t idx[HAS_IDX ? ITEMS : 1];
   SW all_and[NW], all_or[NW];
+  int special = 0;  // float keys: the row holds a NaN or a -0.0
 #pragma unroll
   for (int n = 0; n < NW; ++n) {
     all_and[n] = ~static_cast<SW>(0);
@@ -76,6 +88,9 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
       for (int n = 0; n < NW; ++n) {
         all_and[n] &= w[n];
         all_or[n] |= w[n];
+      }
+      if constexpr (IMAGES_OK) {
+        special |= (static_cast<KeyT>(w[0]) != sign_flip(key[i])) ? 1 : 0;
       }
     } else {
       key[i] = KeyT{};
@@ -94,7 +109,8 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
       s_red[(2 * wave + 1) * NW + n] = all_or[n];
     }
   }
-  __syncthreads();
+  const int any_special = __syncthreads_or(special);
+  const bool images     = IMAGES_OK && (any_special == 0);
   SW varying[NW];
 #pragma unroll
   for (int n = 0; n < NW; ++n) {
@@ -132,6 +148,32 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
   }
 
   uint32_t* wctr = s_ctr + wave * RADIX;
+  // float rows held as images take plain bytes; `images` is uniform, so the choice is a scalar branch
+  auto digit_of = [&](KeyT k, int pass) -> uint32_t {
+    if constexpr (IMAGES_OK) {
+      if (images) {
+        return KeyTraits<CODEC_UNSIGNED, KeyT>::digit(k, pass);
+      }
+    }
+    return KT::digit(k, pass);
+  };
+  auto words_of = [&](KeyT k, uint64_t (&w)[NW]) {
+    if constexpr (IMAGES_OK) {
+      if (images) {
+        w[0] = static_cast<uint64_t>(k);
+        return;
+      }
+    }
+    KT::words(k, w);
+  };
+  if constexpr (IMAGES_OK) {
+    if (images) {
+#pragma unroll
+      for (int i = 0; i < ITEMS; ++i) {
+        key[i] = sign_flip(key[i]);
+      }
+    }
+  }
   for (;;) {
   for (int pass = 0; pass < PASSES; ++pass) {
     if (((todo >> pass) & 1u) == 0) {
@@ -146,7 +188,7 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
 #pragma unroll
     for (int i = 0; i < ITEMS; ++i) {
       const bool valid = full || (woff + i * WAVE < seg);
-      const uint32_t d = KT::digit(key[i], pass);
+      const uint32_t d = digit_of(key[i], pass);
       dpk[i / 4]       = (i % 4 == 0) ? d : (dpk[i / 4] | (d << (8 * (i % 4))));
       rnk[i]           = wave_match_rank(d, valid, wctr);
     }
@@ -213,28 +255,77 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
       break;
     }
     // s_keys holds the row as ordered by the leading digits: is every neighbouring pair in order?
-    int bad = 0;
+    // A few pairs that are not (keys that tie on the leading digits) are put right by rounds of
+    // odd-even transposition in LDS, which exchanges strictly misordered neighbours only and so
+    // keeps equal keys in input order.
+    auto misordered = [&](KeyT first, KeyT second) -> bool {
+      uint64_t a[NW], b[NW];
+      words_of(first, a);
+      words_of(second, b);
+      bool gt = false, eq = true;  // a > b, most significant word first
 #pragma unroll
-    for (int i = 0; i < ITEMS; ++i) {
-      const uint32_t o = woff + i * WAVE;
-      if (o + 1 < seg) {
-        uint64_t a[NW], b[NW];
-        KT::words(key[i], a);
-        KT::words(s_keys[o + 1], b);
-        bool gt = false, eq = true;  // a > b, most significant word first
+      for (int n = NW - 1; n >= 0; --n) {
+        gt = gt || (eq && a[n] > b[n]);
+        eq = eq && (a[n] == b[n]);
+      }
+      return gt;
+    };
+    bool in_order = false;
+    for (int round = 0;; ++round) {
+      int bad = 0;
 #pragma unroll
-        for (int n = NW - 1; n >= 0; --n) {
-          gt = gt || (eq && a[n] > b[n]);
-          eq = eq && (a[n] == b[n]);
+      for (int i = 0; i < ITEMS; ++i) {
+        const uint32_t o = woff + i * WAVE;
+        if (o + 1 < seg) {
+          bad |= misordered(key[i], s_keys[o + 1]) ? 1 : 0;
         }
-        bad |= gt ? 1 : 0;
+      }
+      if (__syncthreads_or(bad) == 0) {
+        in_order = true;
+        break;
+      }
+      if (round == FIXUP_ROUNDS) {
+        break;
+      }
+      for (uint32_t phase = 0; phase < 2; ++phase) {
+        for (uint32_t p = 2 * tid + phase; p + 1 < seg; p += 2 * BLOCK) {
+          const KeyT first = s_keys[p], second = s_keys[p + 1];
+          if (misordered(first, second)) {
+            s_keys[p]     = second;
+            s_keys[p + 1] = first;
+            if constexpr (HAS_IDX) {
+              const IdxS t = s_idx[p];
+              s_idx[p]     = s_idx[p + 1];
+              s_idx[p + 1] = t;
+            }
+          }
+        }
+        __syncthreads();
+      }
+#pragma unroll
+      for (int i = 0; i < ITEMS; ++i) {
+        const uint32_t o = woff + i * WAVE;
+        if (full || o < seg) {
+          key[i] = s_keys[o];
+          if constexpr (HAS_IDX) {
+            idx[i] = s_idx[o];
+          }
+        }
       }
     }
-    if (__syncthreads_or(bad) == 0) {
+    if (in_order) {
       break;
     }
     shortcut = false;
     todo     = active;
+  }
+  if constexpr (IMAGES_OK) {
+    if (images) {
+#pragma unroll
+      for (int i = 0; i < ITEMS; ++i) {
+        key[i] = sign_unflip(key[i]);
+      }
+    }
   }
 
 #pragma unroll

@@ -20,6 +20,9 @@
 
 namespace cpn {
 
+// odd-even transposition rounds tried after the leading-digit shortcut of the row kernels
+constexpr int FIXUP_ROUNDS = 4;
+
 // The ordered key of one element as 32-bit words, least significant first; digit p is byte
 // p%4 of word p/4.
 template <int CODEC, typename KeyT>
@@ -156,8 +159,9 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
   }
 
   // Wide keys: run the passes of the leading varying digits only (2*log2(n) + 4 bits put n keys
-  // in order almost always), then check every neighbouring pair on the whole key; if one is
-  // out of order, run all passes from the state reached (still a stable sort of the input).
+  // in order almost always), then check every neighbouring pair on the whole key; pairs out of
+  // order are repaired by a few rounds of odd-even transposition, and if that does not finish,
+  // all passes run from the state reached (still a stable sort of the input).
   uint32_t todo = active;
   bool shortcut = false;
   if constexpr (PASSES >= 5) {
@@ -254,23 +258,77 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
     if (!shortcut) {
       break;
     }
-    // s_words holds the row as ordered by the leading digits
-    bool bad = false;
+    // s_words holds the row as ordered by the leading digits; a few misordered neighbours (keys
+    // that tie on those digits) are repaired by rounds of odd-even transposition, which only
+    // exchanges strictly misordered pairs and so keeps equal keys in input order
+    bool in_order = false;
+    for (int round = 0;; ++round) {
+      bool bad = false;
 #pragma unroll
-    for (int i = 0; i < ITEMS; ++i) {
-      const uint32_t o = i * WAVE + lane;
-      if (o + 1 < seg) {
-        bool gt = false, eq = true;  // this key > its right neighbour, most significant word first
+      for (int i = 0; i < ITEMS; ++i) {
+        const uint32_t o = i * WAVE + lane;
+        if (o + 1 < seg) {
+          bool gt = false, eq = true;  // this key > its right neighbour, most significant word first
 #pragma unroll
-        for (int n = NW - 1; n >= 0; --n) {
-          const uint32_t b = s_words[wave][n][o + 1];
-          gt               = gt || (eq && w[i][n] > b);
-          eq               = eq && (w[i][n] == b);
+          for (int n = NW - 1; n >= 0; --n) {
+            const uint32_t b = s_words[wave][n][o + 1];
+            gt               = gt || (eq && w[i][n] > b);
+            eq               = eq && (w[i][n] == b);
+          }
+          bad = bad || gt;
         }
-        bad = bad || gt;
       }
+      if (__builtin_amdgcn_ballot_w64(bad) == 0) {
+        in_order = true;
+        break;
+      }
+      if (round == FIXUP_ROUNDS) {
+        break;
+      }
+      __builtin_amdgcn_wave_barrier();
+      for (uint32_t phase = 0; phase < 2; ++phase) {
+        for (uint32_t q = 2 * lane + phase; q + 1 < seg; q += 2 * WAVE) {
+          uint32_t a[NW], b[NW];
+          bool gt = false, eq = true;
+#pragma unroll
+          for (int n = NW - 1; n >= 0; --n) {
+            a[n] = s_words[wave][n][q];
+            b[n] = s_words[wave][n][q + 1];
+            gt   = gt || (eq && a[n] > b[n]);
+            eq   = eq && (a[n] == b[n]);
+          }
+          if (gt) {
+#pragma unroll
+            for (int n = 0; n < NW; ++n) {
+              s_words[wave][n][q]     = b[n];
+              s_words[wave][n][q + 1] = a[n];
+            }
+            if constexpr (CARRY) {
+              const uint16_t t   = s_pos[wave][q];
+              s_pos[wave][q]     = s_pos[wave][q + 1];
+              s_pos[wave][q + 1] = t;
+            }
+          }
+        }
+        __builtin_amdgcn_wave_barrier();
+      }
+#pragma unroll
+      for (int i = 0; i < ITEMS; ++i) {
+        const uint32_t o = i * WAVE + lane;
+        if (full || o < seg) {
+#pragma unroll
+          for (int n = 0; n < NW; ++n) {
+            w[i][n] = s_words[wave][n][o];
+          }
+          if constexpr (CARRY) {
+            const uint32_t q = s_pos[wave][o];
+            pos2[i / 2]      = (i % 2 == 0) ? q : (pos2[i / 2] | (q << 16));
+          }
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
     }
-    if (__builtin_amdgcn_ballot_w64(bad) == 0) {
+    if (in_order) {
       break;
     }
     shortcut = false;

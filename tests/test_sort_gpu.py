@@ -213,6 +213,31 @@ def test_lds_rows_leading_digit_shortcut(lib, torch_cuda, dtype, seg):
     assert_same_bits(i, oracle.local_sort(x, argsort=True), "in place indices")
 
 
+@pytest.mark.parametrize("dtype", [np.int64, np.float64, np.complex128])
+@pytest.mark.parametrize("seg", [200, 512, 1024, 3000])
+def test_row_shortcut_repairs_short_tie_runs(lib, torch_cuda, dtype, seg):
+    """After the leading-digit passes the row kernels repair short runs of ties with odd-even
+    transposition and fall back to every pass for long ones.  Each row holds runs of one length
+    whose low digits descend (a run of L needs L exchange phases), with repeated keys inside the
+    runs so that stability shows; runs of 2..8 are repaired, 9 and more take the fallback."""
+    lengths = [2, 3, 5, 8, 9, 12, 40]
+    pos = np.arange(seg, dtype=np.uint64)
+    rows = []
+    for L in lengths:
+        run, k = pos // np.uint64(L), pos % np.uint64(L)
+        lead = (run * np.uint64(0x010101)) << np.uint64(24) | (run & np.uint64(0xFF)) << np.uint64(16)
+        for low in ((np.uint64(L) - k), (np.uint64(L) - k) // np.uint64(2)):
+            rows.append(lead | low * np.uint64(0x0101))
+    bits = np.stack(rows)
+    if np.dtype(dtype).kind == "i":
+        x = bits.view(np.int64)
+    else:
+        x = (bits | np.uint64(0x3FF0) << np.uint64(48)).view(np.float64)  # positive normal numbers, same order
+        if np.dtype(dtype).kind == "c":
+            x = x + 0j
+    check_rows(lib, torch_cuda, np.ascontiguousarray(x), f"{np.dtype(dtype)} seg={seg} tie runs")
+
+
 # ---- global onesweep path ---------------------------------------------------------------------------
 GLOBAL_LENGTHS = [1, 2, 100, 4097, 8191, 8192, 8193, 16383, 16384, 16385, 3 * 16384 + 5, 100003]
 
