@@ -164,9 +164,12 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
   // all passes run from the state reached (still a stable sort of the input).
   uint32_t todo = active;
   bool shortcut = false;
-  if constexpr (PASSES >= 5) {
+  // 4-byte keys: worth it for rows of up to 256 elements (2 or 3 leading digits instead of 4)
+  constexpr bool SHORTCUT_OK = PASSES >= 5 || (PASSES == 4 && ITEMS <= 4);
+  constexpr int MARGIN       = (PASSES == 4) ? 1 : 2;  // passes the shortcut must save to be tried
+  if constexpr (SHORTCUT_OK) {
     const int lead = (2 * (32 - __builtin_clz(seg - 1 | 1u)) + 4 + RADIX_BITS - 1) / RADIX_BITS;
-    if (__builtin_popcount(active) >= lead + 2) {
+    if (__builtin_popcount(active) >= lead + MARGIN) {
       uint32_t rem = active;
       todo         = 0;
       for (int t = 0; t < lead; ++t) {

@@ -238,6 +238,26 @@ def test_row_shortcut_repairs_short_tie_runs(lib, torch_cuda, dtype, seg):
     check_rows(lib, torch_cuda, np.ascontiguousarray(x), f"{np.dtype(dtype)} seg={seg} tie runs")
 
 
+@pytest.mark.parametrize("dtype", [np.int32, np.uint32, np.float32])
+@pytest.mark.parametrize("seg", [40, 64, 130, 256])
+def test_short_rows_of_4_byte_keys_take_the_shortcut(lib, torch_cuda, dtype, seg):
+    """Rows of up to 256 four-byte keys sort by their 2 or 3 leading digits first; ties there
+    (runs of 2..40 keys whose last byte descends, with repeats) are repaired or take every pass."""
+    pos = np.arange(seg, dtype=np.uint32)
+    rows = []
+    for L in [2, 3, 5, 8, 9, 12, 40]:
+        run, k = pos // np.uint32(L), pos % np.uint32(L)
+        lead = (run * np.uint32(0x0101)) << np.uint32(16) | (run & np.uint32(0xFF)) << np.uint32(8)
+        rows.append(lead | (np.uint32(L) - k))
+        rows.append(lead | (np.uint32(L) - k) // np.uint32(2))
+    rng = np.random.default_rng(seg)
+    rows.append(rng.integers(0, 1 << 32, seg, dtype=np.uint64).astype(np.uint32))  # no ties to speak of
+    x = np.ascontiguousarray(np.stack(rows).view(dtype))
+    check_rows(lib, torch_cuda, x, f"{np.dtype(dtype)} seg={seg} tie runs")
+    many = make_input(dtype, (500, seg), seed=seg)
+    check_rows(lib, torch_cuda, many, f"{np.dtype(dtype)} seg={seg} random rows")
+
+
 # ---- global onesweep path ---------------------------------------------------------------------------
 GLOBAL_LENGTHS = [1, 2, 100, 4097, 8191, 8192, 8193, 16383, 16384, 16385, 3 * 16384 + 5, 100003]
 
