@@ -102,17 +102,29 @@ __device__ __forceinline__ void hist_accumulate(uint32_t* s_hist, KeyT raw, uint
 
 // grid = rows * blocks_per_row; block b of a row covers elements [b*chunk, min(seg, (b+1)*chunk)).
 // 128-bit loads over the 16-byte aligned middle of the chunk, scalar head and tail.
-template <typename KeyT, int CODEC, typename OffT>
+// DISTINCT (single rows of keys with one ordered word): the different keys of the row and their
+// counts are collected on the way, as long as there are at most 256 of them (virtual_digits.h).
+template <typename KeyT, int CODEC, typename OffT, bool DISTINCT = false>
 __global__ __launch_bounds__(HIST_BLOCK) void histogram_kernel(const KeyT* __restrict__ keys,
                                                                  OffT* __restrict__ hist,
                                                                  uint64_t seg,
                                                                  uint32_t blocks_per_row,
-                                                                 uint64_t chunk)
+                                                                 uint64_t chunk,
+                                                                 DistinctTable* __restrict__ table)
 {
   constexpr int PASSES      = KeyTraits<CODEC, KeyT>::PASSES;
   constexpr int VEC         = 16 / sizeof(KeyT);
   constexpr int HIST_COPIES = hist_copies(PASSES);
+  static_assert(!DISTINCT || KeyTraits<CODEC, KeyT>::NWORDS == 1, "distinct keys: one ordered word");
+  // a request that may sort on distinct keys launches both forms of this kernel; the sample
+  // taken before says which of them does the work
+  if (table != nullptr && (table->sample_many != 0) == DISTINCT) {
+    return;
+  }
   __shared__ uint32_t s_hist[PASSES * RADIX * HIST_COPIES];
+  __shared__ uint64_t s_dkeys[DISTINCT ? DISTINCT_LOCAL : 1];
+  __shared__ uint32_t s_dcounts[DISTINCT ? DISTINCT_LOCAL * DISTINCT_COPIES : 1];
+  __shared__ uint32_t s_dstate[3];  // slots taken, gave up, occurrences of image 0
 
   const int tid        = threadIdx.x;
   const uint32_t copy  = tid % HIST_COPIES;
@@ -126,7 +138,38 @@ __global__ __launch_bounds__(HIST_BLOCK) void histogram_kernel(const KeyT* __res
   for (int j = tid; j < PASSES * RADIX * HIST_COPIES; j += HIST_BLOCK) {
     s_hist[j] = 0;
   }
+  if constexpr (DISTINCT) {
+    for (int j = tid; j < static_cast<int>(DISTINCT_LOCAL); j += HIST_BLOCK) {
+      s_dkeys[j] = 0;
+    }
+    for (int j = tid; j < static_cast<int>(DISTINCT_LOCAL * DISTINCT_COPIES); j += HIST_BLOCK) {
+      s_dcounts[j] = 0;
+    }
+    if (tid == 0) {
+      s_dstate[0] = 0;
+      s_dstate[1] = __hip_atomic_load(&table->overflow, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_dstate[2] = 0;
+    }
+  }
   __syncthreads();
+  // histograms of one key; DISTINCT and `collecting`: and the key into the table
+  auto count_key = [&](KeyT raw, bool collecting) {
+    hist_accumulate<KeyT, CODEC, PASSES>(s_hist, raw, copy);
+    if constexpr (DISTINCT) {
+      if (collecting) {
+        uint64_t w[KeyTraits<CODEC, KeyT>::NWORDS];
+        KeyTraits<CODEC, KeyT>::words(raw, w);
+        distinct_collect(w[0], s_dkeys, s_dcounts, s_dstate, tid % DISTINCT_COPIES, &table->overflow);
+      }
+    }
+  };
+  // has the workgroup given up collecting?  Asked once per batch of keys.
+  auto still_collecting = [&]() -> bool {
+    if constexpr (DISTINCT) {
+      return *static_cast<volatile uint32_t*>(&s_dstate[1]) == 0;
+    }
+    return false;
+  };
 
   if (begin < end) {
     const KeyT* p = keys + row * seg;
@@ -137,7 +180,7 @@ __global__ __launch_bounds__(HIST_BLOCK) void histogram_kernel(const KeyT* __res
       head = end - begin;
     }
     for (uint64_t i = tid; i < head; i += HIST_BLOCK) {
-      hist_accumulate<KeyT, CODEC, PASSES>(s_hist, p[begin + i], copy);
+      count_key(p[begin + i], still_collecting());
     }
     const uint64_t vbegin = begin + head;
     const uint64_t nvec   = (end - vbegin) / VEC;
@@ -150,22 +193,24 @@ __global__ __launch_bounds__(HIST_BLOCK) void histogram_kernel(const KeyT* __res
       KeyT k[2 * VEC];
       __builtin_memcpy(k, &q0, 16);
       __builtin_memcpy(k + VEC, &q1, 16);
+      const bool collecting = still_collecting();
 #pragma unroll
       for (int j = 0; j < 2 * VEC; ++j) {
-        hist_accumulate<KeyT, CODEC, PASSES>(s_hist, k[j], copy);
+        count_key(k[j], collecting);
       }
     }
     for (; v < nvec; v += HIST_BLOCK) {
       const uint4 q = vp[v];
       KeyT k[VEC];
       __builtin_memcpy(k, &q, 16);
+      const bool collecting = still_collecting();
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
-        hist_accumulate<KeyT, CODEC, PASSES>(s_hist, k[j], copy);
+        count_key(k[j], collecting);
       }
     }
     for (uint64_t i = vbegin + nvec * VEC + tid; i < end; i += HIST_BLOCK) {
-      hist_accumulate<KeyT, CODEC, PASSES>(s_hist, p[i], copy);
+      count_key(p[i], still_collecting());
     }
   }
   __syncthreads();
@@ -181,6 +226,28 @@ __global__ __launch_bounds__(HIST_BLOCK) void histogram_kernel(const KeyT* __res
       __hip_atomic_fetch_add(&out[j], static_cast<OffT>(c), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
+  if constexpr (DISTINCT) {
+    // the workgroup's keys into the table of the whole row, or the news that there are too many
+    if (s_dstate[1] != 0) {
+      if (tid == 0) {
+        __hip_atomic_store(&table->overflow, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    } else {
+      for (int j = tid; j < static_cast<int>(DISTINCT_LOCAL); j += HIST_BLOCK) {
+        if (s_dkeys[j] != 0) {
+          uint32_t c = 0;
+#pragma unroll
+          for (uint32_t r = 0; r < DISTINCT_COPIES; ++r) {
+            c += s_dcounts[j * DISTINCT_COPIES + r];
+          }
+          distinct_merge(s_dkeys[j], c, table);
+        }
+      }
+      if (tid == 0 && s_dstate[2] != 0) {
+        atomicAdd(&table->zero_count, s_dstate[2]);
+      }
+    }
+  }
 }
 
 // One block per (row, pass): exclusive scan of 256 counts in place.  A pass on whose digit
@@ -193,9 +260,9 @@ __global__ __launch_bounds__(RADIX) void histogram_scan_kernel(OffT* __restrict_
                                                                uint32_t passes,
                                                                const VirtPlan* __restrict__ vplan)
 {
-  // second use, after vplan_kernel: scans the histograms of the virtual digits (one row, block =
-  // group) and nothing when the plan stayed disabled
-  if (vplan != nullptr && (vplan->enabled == 0 || blockIdx.x >= vplan->n_groups)) {
+  // second use, after vplan_kernel: scans the histograms of the grouped virtual digits (one row,
+  // block = group) and nothing when the plan stayed disabled or runs on distinct keys
+  if (vplan != nullptr && (vplan->enabled != VIRT_GROUPS || blockIdx.x >= vplan->n_groups)) {
     return;
   }
   __shared__ OffT s_wsum[RADIX / WAVE];
@@ -360,6 +427,7 @@ struct SweepArgs {
   int idx_final;           // idx_out is the caller's int64 array
   uint32_t spin_limit;     // polls of one descriptor before the tile gives up (LOOKBACK_SPIN_LIMIT)
   const VirtPlan* vplan;   // virtual digits (virtual_digits.h), nullptr when the request cannot use them
+  const DistinctTable* dtable;  // with vplan: the row's different keys when there are at most 256
 };
 
 #ifndef CPN_ONESWEEP_WAVES_PER_EU
@@ -664,7 +732,7 @@ void onesweep_kernel(const SweepArgs<BIG> a_in)
   // VIRT kernels can do both: the device-side plan says whether this sort runs on virtual digits
   bool virt_on = false;
   if constexpr (VIRT) {
-    virt_on = (a_in.vplan != nullptr) && (a_in.vplan->enabled != 0);
+    virt_on = (a_in.vplan != nullptr) && (a_in.vplan->enabled != VIRT_OFF);
   }
   using OffT = typename RowWidth<BIG>::off_t;
   static_assert(BLOCK >= RADIX, "one thread per digit is needed for the look-back");
@@ -675,7 +743,7 @@ void onesweep_kernel(const SweepArgs<BIG> a_in)
   static_assert(TILE <= 65536, "positions inside a tile are kept in 16 bits");
 
   __shared__ SweepShared<KeyT, OffT, WAVES, TILE, STAGE_ELEM> sh;
-  __shared__ uint8_t s_vlut[VIRT ? VIRT_MAX_POSITIONS * RADIX : 1];
+  __shared__ __align__(8) uint8_t s_vlut[VIRT ? VIRT_LDS_BYTES : 1];
   uint32_t vcount   = 0;
   uint64_t voffsets = 0;
 
@@ -683,7 +751,16 @@ void onesweep_kernel(const SweepArgs<BIG> a_in)
   if (pp.active == 0) {
     return;  // every key of every row has the same digit here
   }
-  if (VIRT && virt_on) {
+  if (VIRT && virt_on && a_in.vplan->enabled == VIRT_DISTINCT) {
+    // the one pass on the ranks of the row's different keys: their lookup table into LDS
+    vcount                 = VIRT_COUNT_DISTINCT;
+    const DistinctTable* t = a_in.dtable;
+    uint64_t* lk           = reinterpret_cast<uint64_t*>(s_vlut);
+    for (uint32_t j = threadIdx.x; j < DISTINCT_LOOKUP; j += BLOCK) {
+      lk[j]                           = t->lookup_keys[j];
+      s_vlut[DISTINCT_LOOKUP * 8 + j] = t->lookup_rank[j];
+    }
+  } else if (VIRT && virt_on) {
     // this pass's group: the tables of its byte positions, codes shifted into place (made visible
     // by the barrier below), and the bit offsets of the bytes
     const VirtGroup& g = a_in.vplan->group[a_in.pass];

@@ -168,7 +168,7 @@ inline GlobalLayout global_layout(int key_bytes, int passes, uint64_t volume, ui
   // of 4-byte keys 2 %, more than four passes can win back on average; eight passes can.
   L.virt     = (L.rows == 1) && !L.big && (key_bytes == 8) && (passes == key_bytes) && (seg >= virtual_digit_threshold());
   L.off_virt = L.virt ? HEADER_BYTES : 0;
-  L.off_hist          = HEADER_BYTES + (L.virt ? VIRT_PLAN_BYTES : 0);
+  L.off_hist          = HEADER_BYTES + (L.virt ? VIRT_WORKSPACE_BYTES : 0);
   L.hist_bytes        = align_up(L.rows * L.passes * RADIX * ow, WORKSPACE_ALIGN);
   L.off_desc          = L.off_hist + L.hist_bytes;
   L.desc_bytes_per_pass = align_up(L.num_tiles * RADIX * ow, WORKSPACE_ALIGN);
@@ -378,6 +378,7 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
   SortPlan* plan    = reinterpret_cast<SortPlan*>(ws + HEADER_PLAN);
   constexpr bool VIRT_OK = !BIG && KB == 8 && KeyTraits<CODEC, KeyT>::PASSES == KB;
   VirtPlan* vplan   = L.virt ? reinterpret_cast<VirtPlan*>(ws + L.off_virt) : nullptr;
+  DistinctTable* dtable = L.virt ? reinterpret_cast<DistinctTable*>(ws + L.off_virt + VIRT_PLAN_BYTES) : nullptr;
   OffT* hist        = reinterpret_cast<OffT*>(ws + L.off_hist);
   static_assert(PASSES <= MAX_PASSES, "plan table too small");
   PlanRequest rq{};
@@ -406,9 +407,20 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
     }
     {
       ProfileScope prof("histogram", r.stream);
+      if constexpr (VIRT_OK) {
+        if (L.virt) {
+          // a sample of the row decides whether the sweep also collects the row's different keys:
+          // of the two sweeps launched, the one the sample did not choose exits at once
+          hipLaunchKernelGGL((distinct_sample_kernel<KeyT, CODEC>), dim3(1), dim3(RADIX), 0, r.stream,
+                             static_cast<const KeyT*>(r.values_in), r.seg, dtable);
+          hipLaunchKernelGGL((histogram_kernel<KeyT, CODEC, OffT, true>), dim3(static_cast<uint32_t>(grid)),
+                             dim3(HIST_BLOCK), 0, r.stream, static_cast<const KeyT*>(r.values_in), hist, r.seg,
+                             static_cast<uint32_t>(bpr), chunk, dtable);
+        }
+      }
       hipLaunchKernelGGL((histogram_kernel<KeyT, CODEC, OffT>), dim3(static_cast<uint32_t>(grid)),
                          dim3(HIST_BLOCK), 0, r.stream, static_cast<const KeyT*>(r.values_in), hist, r.seg,
-                         static_cast<uint32_t>(bpr), chunk);
+                         static_cast<uint32_t>(bpr), chunk, dtable);
     }
     CPN_HIP_TRY(hipGetLastError());
     {
@@ -423,8 +435,8 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
         // may replace the byte passes by fewer passes on virtual digits (decided on the device)
         {
           ProfileScope prof("virtual_plan", r.stream);
-          hipLaunchKernelGGL((vplan_kernel<OffT>), dim3(1), dim3(RADIX), 0, r.stream, hist, varying, vplan, r.seg,
-                             static_cast<uint32_t>(PASSES));
+          hipLaunchKernelGGL((vplan_kernel<OffT>), dim3(1), dim3(RADIX), 0, r.stream, hist, varying, vplan, dtable,
+                             r.seg, static_cast<uint32_t>(PASSES));
         }
         CPN_HIP_TRY(hipGetLastError());
         {
@@ -483,6 +495,7 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
     a.pass               = p;
     a.spin_limit         = lookback_spin_limit();
     a.vplan              = vplan;
+    a.dtable             = dtable;
     {
       ProfileScope prof("onesweep", r.stream);
       const dim3 grid(static_cast<uint32_t>(L.num_tiles));

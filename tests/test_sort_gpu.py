@@ -693,6 +693,62 @@ def test_virtual_digits(lib, torch_cuda, virtual_digits_from_2_to_20, dtype):
         x = (hi | lo).astype(np.dtype(dtype).str.replace("i", "u")).view(dtype)
         _, i = abi_sort(lib, torch_cuda, x, want_values=False, want_indices=True)
         assert_same_bits(i, oracle.local_sort(x, argsort=True, threads=8), "mixed busy and quiet bytes")
+    # more than 256 different keys whose bytes take 4 values each: bytes share passes (grouped digits)
+    if np.dtype(dtype).kind != "f":
+        width = np.dtype(dtype).itemsize
+        x = np.zeros(n, dtype=np.uint64)
+        for b in range(width):
+            vals = rng.integers(0, 256, 4).astype(np.uint64)
+            x |= vals[rng.integers(0, 4, n)] << np.uint64(8 * b)
+        x = x.astype(np.dtype(dtype).str.replace("i", "u")).view(dtype)
+        _, i = abi_sort(lib, torch_cuda, x, want_values=False, want_indices=True)
+        assert_same_bits(i, oracle.local_sort(x, argsort=True, threads=8), "4 values per byte")
+        v, _ = abi_sort(lib, torch_cuda, x, want_values=True)
+        assert_same_bits(v, oracle.local_sort(x, argsort=False, threads=8), "4 values per byte, sort")
     # short rows and several rows never use virtual digits; same answers
     x = _few_values(rng, dtype, 3 * 100_000, 16).reshape(3, 100_000)
     check_rows(lib, torch_cuda, x, f"{np.dtype(dtype)} short rows of few values")
+
+
+@pytest.mark.parametrize("dtype", [np.int64, np.uint64, np.float64])
+def test_rows_of_at_most_256_different_keys(lib, torch_cuda, virtual_digits_from_2_to_20, dtype):
+    """A long row of 8-byte keys with at most 256 different values is sorted by one pass on the rank of
+    each key among them; 257 and more fall back to the other plans.  The smallest key of the type (its
+    ordered image is the marker of an empty table slot) and, for floats, NaNs of several payloads and both
+    zeros take part."""
+    rng = np.random.default_rng(7 + np.dtype(dtype).num)
+    n = (1 << 20) + 4321
+    dt = np.dtype(dtype)
+    for distinct in (1, 2, 255, 256, 257, 1000):
+        if dt.kind == "f":
+            pool = rng.standard_normal(distinct) * 1e3
+            bits = pool.view(np.uint64)
+            if distinct >= 6:
+                bits[:6] = [0x7FF8000000000000, 0x7FF8000000000123, 0xFFF8000000000000, 0x8000000000000000, 0,
+                            0xFFF0000000000000]  # three NaNs (one key), -0.0 and 0.0 (one key), -inf
+            pool = bits.view(np.float64)
+        else:
+            info = np.iinfo(dtype)
+            pool = rng.integers(info.min, info.max, distinct, dtype=dtype, endpoint=True)
+            if distinct >= 2:
+                pool[0] = info.min
+                pool[1] = info.max
+        x = pool[rng.integers(0, distinct, n)]
+        want_i = oracle.local_sort(x, argsort=True, threads=8)
+        want_v = oracle.local_sort(x, argsort=False, threads=8)
+        _, i = abi_sort(lib, torch_cuda, x, want_values=False, want_indices=True)
+        assert_same_bits(i, want_i, f"{dt} {distinct} different keys, argsort")
+        v, i = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=True, offset=3)
+        assert_same_bits(v, want_v, f"{dt} {distinct} different keys, values")
+        assert_same_bits(i, want_i + 3, f"{dt} {distinct} different keys, indices")
+        v, _ = abi_sort(lib, torch_cuda, x, want_values=True, in_place=True)
+        assert_same_bits(v, want_v, f"{dt} {distinct} different keys, in place")
+    # few keys in most of the row, many in one corner: the workgroup that meets them reports it
+    x = pool[:16][rng.integers(0, 16, n)]
+    x[n // 3 : n // 3 + 5000] = pool[rng.integers(0, 1000, 5000)]
+    _, i = abi_sort(lib, torch_cuda, x, want_values=False, want_indices=True)
+    assert_same_bits(i, oracle.local_sort(x, argsort=True, threads=8), f"{dt} crowded corner")
+    # sorted input with long runs: every workgroup sees few keys, the row holds many
+    x = np.sort(pool[rng.integers(0, 1000, n)])
+    _, i = abi_sort(lib, torch_cuda, x, want_values=False, want_indices=True)
+    assert_same_bits(i, oracle.local_sort(x, argsort=True, threads=8), f"{dt} sorted runs")
