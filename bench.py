@@ -120,6 +120,7 @@ def algorithmic_bytes(cfg: dict, lds_limit_rows: bool, passes_run: int | None = 
         out["onesweep"] = sum(per_pass) / passes  # average launch
         out["histogram"] = n * kb
         out["virtual_histogram"] = n * kb
+        out["distinct_sweep"] = n * kb
         # the same passes counted with the baseline's formula, which carries the payload at its final
         # width (vb = 8) through every pass: r_1 = kb, r_p = w_p = kb + vb, w_P = vb for index-only output
         vb = 8 if argsort else 0
@@ -572,8 +573,10 @@ def main() -> None:
         if skipped:
             by_label["onesweep_skipped"] = skipped
         passes_run = round(len(by_label["onesweep"]) / args.steps)
-    if "virtual_histogram" in by_label and max(by_label["virtual_histogram"]) < 0.02:
-        by_label["virtual_histogram_skipped"] = by_label.pop("virtual_histogram")  # plan not enabled: early exit
+    # sweeps whose launch exits at once because the device-side plan has no use for them
+    for label in ("histogram", "virtual_histogram", "distinct_sweep"):
+        if label in by_label and cfg["x"].nbytes >= (1 << 26) and max(by_label[label]) < 0.02:
+            by_label[label + "_skipped"] = by_label.pop(label)
     alg = algorithmic_bytes(cfg, job.uses_lds_rows, passes_run)
     if job.uses_lds_rows:  # whichever of the per-row kernels the row length selects
         dominant = next(k for k in ("tiny_row_sort", "wave_row_sort", "lds_row_sort") if k in by_label)

@@ -102,29 +102,23 @@ __device__ __forceinline__ void hist_accumulate(uint32_t* s_hist, KeyT raw, uint
 
 // grid = rows * blocks_per_row; block b of a row covers elements [b*chunk, min(seg, (b+1)*chunk)).
 // 128-bit loads over the 16-byte aligned middle of the chunk, scalar head and tail.
-// DISTINCT (single rows of keys with one ordered word): the different keys of the row and their
-// counts are collected on the way, as long as there are at most 256 of them (virtual_digits.h).
-template <typename KeyT, int CODEC, typename OffT, bool DISTINCT = false>
+// `vplan` (may be null): nothing to do when the sort already runs on the ranks of the row's
+// different keys (virtual_digits.h).
+template <typename KeyT, int CODEC, typename OffT>
 __global__ __launch_bounds__(HIST_BLOCK) void histogram_kernel(const KeyT* __restrict__ keys,
                                                                  OffT* __restrict__ hist,
                                                                  uint64_t seg,
                                                                  uint32_t blocks_per_row,
                                                                  uint64_t chunk,
-                                                                 DistinctTable* __restrict__ table)
+                                                                 const VirtPlan* __restrict__ vplan)
 {
   constexpr int PASSES      = KeyTraits<CODEC, KeyT>::PASSES;
   constexpr int VEC         = 16 / sizeof(KeyT);
   constexpr int HIST_COPIES = hist_copies(PASSES);
-  static_assert(!DISTINCT || KeyTraits<CODEC, KeyT>::NWORDS == 1, "distinct keys: one ordered word");
-  // a request that may sort on distinct keys launches both forms of this kernel; the sample
-  // taken before says which of them does the work
-  if (table != nullptr && (table->sample_many != 0) == DISTINCT) {
+  if (vplan != nullptr && vplan->enabled == VIRT_DISTINCT) {
     return;
   }
   __shared__ uint32_t s_hist[PASSES * RADIX * HIST_COPIES];
-  __shared__ uint64_t s_dkeys[DISTINCT ? DISTINCT_LOCAL : 1];
-  __shared__ uint32_t s_dcounts[DISTINCT ? DISTINCT_LOCAL * DISTINCT_COPIES : 1];
-  __shared__ uint32_t s_dstate[3];  // slots taken, gave up, occurrences of image 0
 
   const int tid        = threadIdx.x;
   const uint32_t copy  = tid % HIST_COPIES;
@@ -138,38 +132,7 @@ __global__ __launch_bounds__(HIST_BLOCK) void histogram_kernel(const KeyT* __res
   for (int j = tid; j < PASSES * RADIX * HIST_COPIES; j += HIST_BLOCK) {
     s_hist[j] = 0;
   }
-  if constexpr (DISTINCT) {
-    for (int j = tid; j < static_cast<int>(DISTINCT_LOCAL); j += HIST_BLOCK) {
-      s_dkeys[j] = 0;
-    }
-    for (int j = tid; j < static_cast<int>(DISTINCT_LOCAL * DISTINCT_COPIES); j += HIST_BLOCK) {
-      s_dcounts[j] = 0;
-    }
-    if (tid == 0) {
-      s_dstate[0] = 0;
-      s_dstate[1] = __hip_atomic_load(&table->overflow, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      s_dstate[2] = 0;
-    }
-  }
   __syncthreads();
-  // histograms of one key; DISTINCT and `collecting`: and the key into the table
-  auto count_key = [&](KeyT raw, bool collecting) {
-    hist_accumulate<KeyT, CODEC, PASSES>(s_hist, raw, copy);
-    if constexpr (DISTINCT) {
-      if (collecting) {
-        uint64_t w[KeyTraits<CODEC, KeyT>::NWORDS];
-        KeyTraits<CODEC, KeyT>::words(raw, w);
-        distinct_collect(w[0], s_dkeys, s_dcounts, s_dstate, tid % DISTINCT_COPIES, &table->overflow);
-      }
-    }
-  };
-  // has the workgroup given up collecting?  Asked once per batch of keys.
-  auto still_collecting = [&]() -> bool {
-    if constexpr (DISTINCT) {
-      return *static_cast<volatile uint32_t*>(&s_dstate[1]) == 0;
-    }
-    return false;
-  };
 
   if (begin < end) {
     const KeyT* p = keys + row * seg;
@@ -180,7 +143,7 @@ __global__ __launch_bounds__(HIST_BLOCK) void histogram_kernel(const KeyT* __res
       head = end - begin;
     }
     for (uint64_t i = tid; i < head; i += HIST_BLOCK) {
-      count_key(p[begin + i], still_collecting());
+      hist_accumulate<KeyT, CODEC, PASSES>(s_hist, p[begin + i], copy);
     }
     const uint64_t vbegin = begin + head;
     const uint64_t nvec   = (end - vbegin) / VEC;
@@ -193,24 +156,22 @@ __global__ __launch_bounds__(HIST_BLOCK) void histogram_kernel(const KeyT* __res
       KeyT k[2 * VEC];
       __builtin_memcpy(k, &q0, 16);
       __builtin_memcpy(k + VEC, &q1, 16);
-      const bool collecting = still_collecting();
 #pragma unroll
       for (int j = 0; j < 2 * VEC; ++j) {
-        count_key(k[j], collecting);
+        hist_accumulate<KeyT, CODEC, PASSES>(s_hist, k[j], copy);
       }
     }
     for (; v < nvec; v += HIST_BLOCK) {
       const uint4 q = vp[v];
       KeyT k[VEC];
       __builtin_memcpy(k, &q, 16);
-      const bool collecting = still_collecting();
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
-        count_key(k[j], collecting);
+        hist_accumulate<KeyT, CODEC, PASSES>(s_hist, k[j], copy);
       }
     }
     for (uint64_t i = vbegin + nvec * VEC + tid; i < end; i += HIST_BLOCK) {
-      count_key(p[i], still_collecting());
+      hist_accumulate<KeyT, CODEC, PASSES>(s_hist, p[i], copy);
     }
   }
   __syncthreads();
@@ -226,28 +187,6 @@ __global__ __launch_bounds__(HIST_BLOCK) void histogram_kernel(const KeyT* __res
       __hip_atomic_fetch_add(&out[j], static_cast<OffT>(c), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
-  if constexpr (DISTINCT) {
-    // the workgroup's keys into the table of the whole row, or the news that there are too many
-    if (s_dstate[1] != 0) {
-      if (tid == 0) {
-        __hip_atomic_store(&table->overflow, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-    } else {
-      for (int j = tid; j < static_cast<int>(DISTINCT_LOCAL); j += HIST_BLOCK) {
-        if (s_dkeys[j] != 0) {
-          uint32_t c = 0;
-#pragma unroll
-          for (uint32_t r = 0; r < DISTINCT_COPIES; ++r) {
-            c += s_dcounts[j * DISTINCT_COPIES + r];
-          }
-          distinct_merge(s_dkeys[j], c, table);
-        }
-      }
-      if (tid == 0 && s_dstate[2] != 0) {
-        atomicAdd(&table->zero_count, s_dstate[2]);
-      }
-    }
-  }
 }
 
 // One block per (row, pass): exclusive scan of 256 counts in place.  A pass on whose digit
@@ -258,12 +197,17 @@ __global__ __launch_bounds__(RADIX) void histogram_scan_kernel(OffT* __restrict_
                                                                uint32_t* __restrict__ varying,
                                                                uint64_t seg,
                                                                uint32_t passes,
-                                                               const VirtPlan* __restrict__ vplan)
+                                                               const VirtPlan* __restrict__ vplan,
+                                                               uint32_t second)
 {
-  // second use, after vplan_kernel: scans the histograms of the grouped virtual digits (one row,
-  // block = group) and nothing when the plan stayed disabled or runs on distinct keys
-  if (vplan != nullptr && (vplan->enabled != VIRT_GROUPS || blockIdx.x >= vplan->n_groups)) {
-    return;
+  // first use (`second` == 0): nothing when the sort already runs on the ranks of the row's
+  // different keys.  Second use, after vplan_kernel: scans the histograms of the grouped virtual
+  // digits (one row, block = group) and nothing when that plan is not in force.
+  if (vplan != nullptr) {
+    const uint32_t mode = vplan->enabled;
+    if (second == 0 ? (mode == VIRT_DISTINCT) : (mode != VIRT_GROUPS || blockIdx.x >= vplan->n_groups)) {
+      return;
+    }
   }
   __shared__ OffT s_wsum[RADIX / WAVE];
   const int tid  = threadIdx.x;
@@ -567,13 +511,20 @@ __device__ __forceinline__ void onesweep_tile(
   __syncthreads();
 
   // ---- scatter into LDS: counter = first position of this wave's keys with that digit ----
+  // VIRT kernels, passes that store no keys (the last pass of an index-only sort): only the digits
+  // travel, one byte each, and the table lookups for the second use of the digit fall away
+  const bool digits_only = VIRT && (a.keys_out == nullptr);
   uint32_t pos2[ITEMS / 2];  // positions in the sorted tile, two per register
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t d   = (dpk[i / 4] >> (8 * (i % 4))) & 0xFFu;
     const uint32_t pos = (wctr[d] + ((rnk2[i / 2] >> (16 * (i % 2))) & 0xFFFFu)) & 0xFFFFu;
     if (FULL || (woff + i * WAVE < count)) {
-      s_keys[pos] = key[i];
+      if (VIRT && digits_only) {
+        reinterpret_cast<uint8_t*>(s_keys)[pos] = static_cast<uint8_t>(d);
+      } else {
+        s_keys[pos] = key[i];
+      }
     }
     pos2[i / 2] = (i % 2 == 0) ? pos : (pos2[i / 2] | (pos << 16));
   }
@@ -648,7 +599,15 @@ __device__ __forceinline__ void onesweep_tile(
   //      to row offset gbase[its digit] + p.  The digits of this thread's output positions
   //      are kept (four per register) for the payload, which goes the same way. ----
   uint32_t dq[ITEMS / 4];
-  {
+  if (VIRT && digits_only) {
+    const uint8_t* s_digits = reinterpret_cast<const uint8_t*>(s_keys);
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+      const uint32_t p = tid + k * BLOCK;
+      const uint32_t d = (FULL || p < count) ? s_digits[p] : 0u;
+      dq[k / 4]        = (k % 4 == 0) ? d : (dq[k / 4] | (d << (8 * (k % 4))));
+    }
+  } else {
     KeyT kk[ITEMS];
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {

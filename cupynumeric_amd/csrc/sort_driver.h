@@ -405,29 +405,45 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
     if (grid >= (1ull << 31)) {
       return CPN_ERR_UNSUPPORTED;
     }
-    {
-      ProfileScope prof("histogram", r.stream);
-      if constexpr (VIRT_OK) {
-        if (L.virt) {
-          // a sample of the row decides whether the sweep also collects the row's different keys:
-          // of the two sweeps launched, the one the sample did not choose exits at once
+    if constexpr (VIRT_OK) {
+      if (L.virt) {
+        // At most 256 different keys in the row?  A sample decides whether it is worth finding out;
+        // if so a sweep collects the keys and a plan kernel sets up the one pass on their ranks,
+        // and the histogram sweep and the other plan kernels below then exit at once.
+        {
+          ProfileScope prof("distinct_sample", r.stream);
           hipLaunchKernelGGL((distinct_sample_kernel<KeyT, CODEC>), dim3(1), dim3(RADIX), 0, r.stream,
                              static_cast<const KeyT*>(r.values_in), r.seg, dtable);
-          hipLaunchKernelGGL((histogram_kernel<KeyT, CODEC, OffT, true>), dim3(static_cast<uint32_t>(grid)),
-                             dim3(HIST_BLOCK), 0, r.stream, static_cast<const KeyT*>(r.values_in), hist, r.seg,
-                             static_cast<uint32_t>(bpr), chunk, dtable);
         }
+        CPN_HIP_TRY(hipGetLastError());
+        {
+          const uint64_t dchunk = 65536;
+          const uint64_t dgrid  = (r.seg + dchunk - 1) / dchunk;
+          ProfileScope prof("distinct_sweep", r.stream);
+          hipLaunchKernelGGL((distinct_sweep_kernel<KeyT, CODEC>), dim3(static_cast<uint32_t>(dgrid)), dim3(DSWEEP_BLOCK),
+                             0, r.stream, static_cast<const KeyT*>(r.values_in), r.seg, dchunk, dtable);
+        }
+        CPN_HIP_TRY(hipGetLastError());
+        {
+          ProfileScope prof("distinct_plan", r.stream);
+          hipLaunchKernelGGL((distinct_plan_kernel<OffT>), dim3(1), dim3(RADIX), 0, r.stream, hist, varying, vplan,
+                             dtable, static_cast<uint32_t>(PASSES));
+        }
+        CPN_HIP_TRY(hipGetLastError());
       }
+    }
+    {
+      ProfileScope prof("histogram", r.stream);
       hipLaunchKernelGGL((histogram_kernel<KeyT, CODEC, OffT>), dim3(static_cast<uint32_t>(grid)),
                          dim3(HIST_BLOCK), 0, r.stream, static_cast<const KeyT*>(r.values_in), hist, r.seg,
-                         static_cast<uint32_t>(bpr), chunk, dtable);
+                         static_cast<uint32_t>(bpr), chunk, static_cast<const VirtPlan*>(vplan));
     }
     CPN_HIP_TRY(hipGetLastError());
     {
       ProfileScope prof("histogram_scan", r.stream);
       hipLaunchKernelGGL((histogram_scan_kernel<OffT>), dim3(static_cast<uint32_t>(L.rows * PASSES)),
                          dim3(RADIX), 0, r.stream, hist, varying, r.seg, static_cast<uint32_t>(PASSES),
-                         static_cast<const VirtPlan*>(nullptr));
+                         static_cast<const VirtPlan*>(vplan), 0u);
     }
     CPN_HIP_TRY(hipGetLastError());
     if constexpr (VIRT_OK) {
@@ -435,8 +451,8 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
         // may replace the byte passes by fewer passes on virtual digits (decided on the device)
         {
           ProfileScope prof("virtual_plan", r.stream);
-          hipLaunchKernelGGL((vplan_kernel<OffT>), dim3(1), dim3(RADIX), 0, r.stream, hist, varying, vplan, dtable,
-                             r.seg, static_cast<uint32_t>(PASSES));
+          hipLaunchKernelGGL((vplan_kernel<OffT>), dim3(1), dim3(RADIX), 0, r.stream, hist, varying, vplan, r.seg,
+                             static_cast<uint32_t>(PASSES));
         }
         CPN_HIP_TRY(hipGetLastError());
         {
@@ -450,7 +466,7 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
         {
           ProfileScope prof("virtual_scan", r.stream);
           hipLaunchKernelGGL((histogram_scan_kernel<OffT>), dim3(static_cast<uint32_t>(PASSES)), dim3(RADIX), 0,
-                             r.stream, hist, varying, r.seg, static_cast<uint32_t>(PASSES), vplan);
+                             r.stream, hist, varying, r.seg, static_cast<uint32_t>(PASSES), vplan, 1u);
         }
         CPN_HIP_TRY(hipGetLastError());
       }

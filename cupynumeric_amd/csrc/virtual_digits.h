@@ -18,13 +18,14 @@
 // real keys of at most 8 bytes only.
 //
 // Distinct keys: when the whole row holds at most 256 different keys, ONE pass sorts it, on
-// the rank of each key among the different keys.  The histogram sweep collects the different
-// keys and their counts in a hash table as it goes (per workgroup in LDS, merged into a table
-// in the workspace; it stops at the 257th key), vplan_kernel ranks them and writes the
-// offsets of the one pass, and the scatter pass looks every key's rank up in a copy of the
-// table in LDS.  No second sweep is needed.  Collecting costs the sweep LDS and time, so a
-// sample of 4096 keys is looked at first (distinct_sample_kernel) and rows whose sample already
-// holds more than 256 different keys get the plain sweep.
+// the rank of each key among the different keys.  Before the histogram sweep a sample of 4096
+// keys is looked at (distinct_sample_kernel); unless it already holds more than 256 different
+// keys, a sweep of its own collects the different keys and their counts in a hash table
+// (distinct_sweep_kernel: per workgroup in LDS, merged into a table in the workspace; it stops
+// at the 257th key) and distinct_plan_kernel ranks them, writes the offsets of the one pass
+// and the lookup table in which the scatter pass finds every key's rank (copied into LDS).
+// The histogram sweep and the other plan kernels then exit at once; when the table stays
+// incomplete they run as if nothing had happened.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -176,7 +177,7 @@ __device__ __forceinline__ void distinct_merge(uint64_t image, uint32_t count, D
   }
 }
 
-// One workgroup: DISTINCT_SAMPLE keys spread evenly over the row; more than DISTINCT_MAX different
+// One workgroup: DISTINCT_SAMPLE keys from all over the row; more than DISTINCT_MAX different
 // ones among them raise table->sample_many.
 constexpr uint32_t DISTINCT_SAMPLE = 4096;
 template <typename KeyT, int CODEC>
@@ -198,14 +199,16 @@ __global__ __launch_bounds__(RADIX) void distinct_sample_kernel(const KeyT* __re
     s_state[tid] = 0;
   }
   __syncthreads();
+  // DISTINCT_SAMPLE / WAVE runs of WAVE neighbouring keys, the runs spread evenly over the row (few
+  // memory pages are touched, every wave reads one run per step)
   const uint64_t n      = seg < DISTINCT_SAMPLE ? seg : DISTINCT_SAMPLE;
-  const uint64_t stride = seg / n;
+  const uint64_t stride = (seg / n) * WAVE;  // from run to run
   constexpr int PER_THREAD = DISTINCT_SAMPLE / RADIX;
   KeyT mine[PER_THREAD];  // all loads of a thread are issued before the first key is looked at
 #pragma unroll
   for (int j = 0; j < PER_THREAD; ++j) {
     const uint64_t i = static_cast<uint64_t>(j) * RADIX + tid;
-    mine[j]          = (i < n) ? keys[i * stride] : KeyT{};
+    mine[j]          = (i < n) ? keys[(i / WAVE) * stride + (i % WAVE)] : KeyT{};
   }
 #pragma unroll
   for (int j = 0; j < PER_THREAD; ++j) {
@@ -218,30 +221,217 @@ __global__ __launch_bounds__(RADIX) void distinct_sample_kernel(const KeyT* __re
   }
 }
 
+// The collecting sweep: every workgroup gathers the different keys of its chunk of the row (and how
+// often each occurs) in LDS and merges them into the row's table.  Exits at once when the sample
+// already found too many; workgroups that start after one has given up do not try either.
+constexpr int DSWEEP_BLOCK = 256;
+template <typename KeyT, int CODEC>
+__global__ __launch_bounds__(DSWEEP_BLOCK) void distinct_sweep_kernel(const KeyT* __restrict__ keys,
+                                                                       uint64_t seg,
+                                                                       uint64_t chunk,
+                                                                       DistinctTable* __restrict__ table)
+{
+  static_assert(KeyTraits<CODEC, KeyT>::NWORDS == 1, "distinct keys: one ordered word");
+  if (table->sample_many != 0) {
+    return;
+  }
+  __shared__ uint64_t s_keys[DISTINCT_LOCAL];
+  __shared__ uint32_t s_counts[DISTINCT_LOCAL * DISTINCT_COPIES];
+  __shared__ uint32_t s_state[3];  // slots taken, gave up, occurrences of image 0
+  const uint32_t tid = threadIdx.x;
+  for (uint32_t j = tid; j < DISTINCT_LOCAL; j += DSWEEP_BLOCK) {
+    s_keys[j] = 0;
+  }
+  for (uint32_t j = tid; j < DISTINCT_LOCAL * DISTINCT_COPIES; j += DSWEEP_BLOCK) {
+    s_counts[j] = 0;
+  }
+  if (tid == 0) {
+    s_state[0] = 0;
+    s_state[1] = __hip_atomic_load(&table->overflow, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_state[2] = 0;
+  }
+  __syncthreads();
+  const uint64_t begin = static_cast<uint64_t>(blockIdx.x) * chunk;
+  uint64_t end         = begin + chunk;
+  if (end > seg) {
+    end = seg;
+  }
+  const uint32_t copy = tid % DISTINCT_COPIES;
+  auto collect = [&](KeyT raw) {
+    uint64_t w[1];
+    KeyTraits<CODEC, KeyT>::words(raw, w);
+    distinct_collect(w[0], s_keys, s_counts, s_state, copy, &table->overflow);
+  };
+  // four keys per thread and step, their loads issued together; has the workgroup given up is
+  // asked once per step
+  uint64_t i = begin + tid;
+  for (; i + 3 * DSWEEP_BLOCK < end; i += 4 * DSWEEP_BLOCK) {
+    if (*static_cast<volatile uint32_t*>(&s_state[1]) != 0) {
+      break;
+    }
+    const KeyT k0 = keys[i], k1 = keys[i + DSWEEP_BLOCK], k2 = keys[i + 2 * DSWEEP_BLOCK], k3 = keys[i + 3 * DSWEEP_BLOCK];
+    collect(k0);
+    collect(k1);
+    collect(k2);
+    collect(k3);
+  }
+  for (; i < end; i += DSWEEP_BLOCK) {
+    if (*static_cast<volatile uint32_t*>(&s_state[1]) != 0) {
+      break;
+    }
+    collect(keys[i]);
+  }
+  __syncthreads();
+  if (s_state[1] != 0) {
+    return;  // whoever gave up has said so in the table
+  }
+  for (uint32_t j = tid; j < DISTINCT_LOCAL; j += DSWEEP_BLOCK) {
+    if (s_keys[j] != 0) {
+      uint32_t c = 0;
+#pragma unroll
+      for (uint32_t r = 0; r < DISTINCT_COPIES; ++r) {
+        c += s_counts[j * DISTINCT_COPIES + r];
+      }
+      distinct_merge(s_keys[j], c, table);
+    }
+  }
+  if (tid == 0 && s_state[2] != 0) {
+    atomicAdd(&table->zero_count, s_state[2]);
+  }
+}
+
+// One workgroup of 256 threads, after the collecting sweep.  When the table is complete (at most
+// 256 different keys): ranks them, writes the offsets of the one pass into hist[0][*], the lookup
+// table of the scatter pass, varying[] (pass 0 runs unless all keys are equal) and
+// plan->enabled = VIRT_DISTINCT, after which the histogram sweep and the other plan kernels have
+// nothing to do.  Otherwise leaves everything alone.
+template <typename OffT>
+__global__ __launch_bounds__(RADIX) void distinct_plan_kernel(OffT* __restrict__ hist,
+                                                               uint32_t* __restrict__ varying,
+                                                               VirtPlan* __restrict__ plan,
+                                                               DistinctTable* __restrict__ table,
+                                                               uint32_t passes)
+{
+  __shared__ uint64_t s_keys[DISTINCT_MAX];  // the row's different keys (other than image 0), unordered
+  __shared__ uint32_t s_slot[DISTINCT_MAX];  // where each sits in the collecting table
+  __shared__ uint32_t s_nkeys;
+  __shared__ uint64_t s_lookup_keys[DISTINCT_LOOKUP];
+  __shared__ uint8_t s_lookup_rank[DISTINCT_LOOKUP];
+  __shared__ OffT s_count[RADIX];
+  __shared__ OffT s_wsum[RADIX / WAVE];
+  __shared__ uint32_t s_use_table, s_failed, s_total;
+  const int tid  = threadIdx.x;
+  const int lane = tid & (WAVE - 1);
+  const int wave = tid / WAVE;
+  if (tid == 0) {
+    const uint32_t k = table->n_keys + (table->zero_count != 0 ? 1u : 0u);
+    s_use_table      = (table->sample_many == 0 && table->overflow == 0 && k >= 1 && k <= DISTINCT_MAX) ? 1u : 0u;
+    s_total          = k;
+    s_failed         = 0;
+    s_nkeys          = 0;
+  }
+  __syncthreads();
+  if (s_use_table == 0) {
+    return;
+  }
+  const uint32_t zero_rank = (table->zero_count != 0) ? 1u : 0u;
+  for (uint32_t j = tid; j < DISTINCT_SLOTS; j += RADIX) {
+    const uint64_t key = table->keys[j];
+    if (key != 0) {
+      const uint32_t i = atomicAdd(&s_nkeys, 1u);
+      if (i < DISTINCT_MAX) {  // n_keys <= DISTINCT_MAX was checked above
+        s_keys[i] = key;
+        s_slot[i] = j;
+      }
+    }
+  }
+  for (uint32_t j = tid; j < DISTINCT_LOOKUP; j += RADIX) {
+    s_lookup_keys[j] = 0;
+    s_lookup_rank[j] = 0;
+  }
+  s_count[tid] = (tid == 0) ? static_cast<OffT>(table->zero_count) : static_cast<OffT>(0);
+  __syncthreads();
+  const uint32_t nkeys = (s_nkeys < DISTINCT_MAX) ? s_nkeys : DISTINCT_MAX;
+  if (static_cast<uint32_t>(tid) < nkeys) {  // RADIX threads, DISTINCT_MAX == RADIX keys at most
+    const uint64_t key = s_keys[tid];
+    uint32_t rank      = zero_rank;
+    for (uint32_t i = 0; i < nkeys; ++i) {
+      rank += (s_keys[i] < key) ? 1u : 0u;
+    }
+    s_count[rank] = static_cast<OffT>(table->counts[s_slot[tid]]);  // ranks are distinct: one writer each
+    uint32_t h    = distinct_hash(key, 9);
+    bool placed   = false;
+    for (uint32_t probe = 0; probe < DISTINCT_MAX_PROBES && !placed; ++probe) {
+      const uint64_t prev =
+        atomicCAS(reinterpret_cast<unsigned long long*>(&s_lookup_keys[h]), 0ull, static_cast<unsigned long long>(key));
+      if (prev == 0) {
+        s_lookup_rank[h] = static_cast<uint8_t>(rank);
+        placed           = true;
+      } else {
+        h = (h + 1) & (DISTINCT_LOOKUP - 1);
+      }
+    }
+    if (!placed) {
+      s_failed = 1;  // a chain the scatter pass would not follow to its end
+    }
+  }
+  __syncthreads();
+  if (s_failed != 0) {
+    return;  // the byte passes take over
+  }
+  {
+    // exclusive scan of the counts by rank: the offsets of the one pass
+    const OffT c = s_count[tid];
+    OffT incl    = c;
+#pragma unroll
+    for (int delta = 1; delta < WAVE; delta <<= 1) {
+      const OffT t = __shfl_up(incl, delta, WAVE);
+      if (lane >= delta) {
+        incl += t;
+      }
+    }
+    if (lane == WAVE - 1) {
+      s_wsum[wave] = incl;
+    }
+    __syncthreads();
+    OffT prefix = 0;
+    for (int w = 0; w < wave; ++w) {
+      prefix += s_wsum[w];
+    }
+    hist[tid] = prefix + incl - c;
+    for (uint32_t j = tid; j < DISTINCT_LOOKUP; j += RADIX) {
+      table->lookup_keys[j] = s_lookup_keys[j];
+      table->lookup_rank[j] = s_lookup_rank[j];
+    }
+    if (tid < static_cast<int>(passes)) {
+      varying[tid] = (tid == 0 && s_total >= 2) ? 1u : 0u;  // one key only: nothing to sort
+    }
+    if (tid == 0) {
+      plan->enabled  = VIRT_DISTINCT;
+      plan->n_groups = 1;
+    }
+  }
+}
+
 // One workgroup of 256 threads.  `hist` holds the exclusive-scanned byte histograms of the one
 // row ([pass][256]); `varying[p]` says whether position p differs between keys at all.
 // When virtual digits save enough passes to pay for themselves: writes the plan, clears hist[g][*] for the
 // groups (vhist_kernel accumulates there) and resets varying (the second scan raises it again
-// for the groups).  Otherwise leaves everything alone with enabled == 0.
+// for the groups).  Otherwise leaves everything alone with enabled == 0.  Nothing to do when the
+// sort already runs on the ranks of the row's different keys.
 template <typename OffT>
 __global__ __launch_bounds__(RADIX) void vplan_kernel(OffT* __restrict__ hist,
                                                        uint32_t* __restrict__ varying,
                                                        VirtPlan* __restrict__ plan,
-                                                       DistinctTable* __restrict__ table,
                                                        uint64_t seg,
                                                        uint32_t passes)
 {
   __shared__ uint32_t s_wcount[RADIX / WAVE];
   __shared__ uint32_t s_distinct[VIRT_MAX_POSITIONS];
   __shared__ uint32_t s_enabled, s_groups;
-  __shared__ uint64_t s_keys[DISTINCT_MAX];   // the row's different keys (other than image 0), unordered
-  __shared__ uint32_t s_slot[DISTINCT_MAX];   // where each sits in the collecting table
-  __shared__ uint32_t s_nkeys;
-  __shared__ uint64_t s_lookup_keys[DISTINCT_LOOKUP];
-  __shared__ uint8_t s_lookup_rank[DISTINCT_LOOKUP];
-  __shared__ OffT s_count[RADIX];
-  __shared__ OffT s_wsum[RADIX / WAVE];
-  __shared__ uint32_t s_use_table, s_failed;
+  if (plan->enabled == VIRT_DISTINCT) {
+    return;  // distinct_plan_kernel has settled everything; the byte histograms were not even made
+  }
   const int tid  = threadIdx.x;
   const int lane = tid & (WAVE - 1);
   const int wave = tid / WAVE;
@@ -269,96 +459,6 @@ __global__ __launch_bounds__(RADIX) void vplan_kernel(OffT* __restrict__ hist,
       s_distinct[p] = total;
     }
     __syncthreads();
-  }
-
-  // ---- at most 256 different keys in the row: one pass on their ranks ----
-  if (tid == 0) {
-    uint32_t busy = 0;
-    for (uint32_t p = 0; p < passes; ++p) {
-      busy += (s_distinct[p] > 1) ? 1u : 0u;
-    }
-    const uint32_t k = table->n_keys + (table->zero_count != 0 ? 1u : 0u);
-    s_use_table      = (table->sample_many == 0 && table->overflow == 0 && k <= DISTINCT_MAX && busy >= 2) ? 1u : 0u;
-    s_failed         = 0;
-    s_nkeys          = 0;
-  }
-  __syncthreads();
-  if (s_use_table != 0) {
-    const uint32_t zero_rank = (table->zero_count != 0) ? 1u : 0u;
-    for (uint32_t j = tid; j < DISTINCT_SLOTS; j += RADIX) {
-      const uint64_t key = table->keys[j];
-      if (key != 0) {
-        const uint32_t i = atomicAdd(&s_nkeys, 1u);
-        if (i < DISTINCT_MAX) {  // n_keys <= DISTINCT_MAX was checked above
-          s_keys[i] = key;
-          s_slot[i] = j;
-        }
-      }
-    }
-    for (uint32_t j = tid; j < DISTINCT_LOOKUP; j += RADIX) {
-      s_lookup_keys[j] = 0;
-      s_lookup_rank[j] = 0;
-    }
-    s_count[tid] = (tid == 0) ? static_cast<OffT>(table->zero_count) : static_cast<OffT>(0);
-    __syncthreads();
-    const uint32_t nkeys = (s_nkeys < DISTINCT_MAX) ? s_nkeys : DISTINCT_MAX;
-    if (static_cast<uint32_t>(tid) < nkeys) {  // RADIX threads, DISTINCT_MAX == RADIX keys at most
-      const uint64_t key = s_keys[tid];
-      uint32_t rank      = zero_rank;
-      for (uint32_t i = 0; i < nkeys; ++i) {
-        rank += (s_keys[i] < key) ? 1u : 0u;
-      }
-      s_count[rank] = static_cast<OffT>(table->counts[s_slot[tid]]);  // ranks are distinct: one writer each
-      uint32_t h    = distinct_hash(key, 9);
-      bool placed   = false;
-      for (uint32_t probe = 0; probe < DISTINCT_MAX_PROBES && !placed; ++probe) {
-        const uint64_t prev =
-          atomicCAS(reinterpret_cast<unsigned long long*>(&s_lookup_keys[h]), 0ull, static_cast<unsigned long long>(key));
-        if (prev == 0) {
-          s_lookup_rank[h] = static_cast<uint8_t>(rank);
-          placed           = true;
-        } else {
-          h = (h + 1) & (DISTINCT_LOOKUP - 1);
-        }
-      }
-      if (!placed) {
-        s_failed = 1;  // a chain the scatter pass would not follow to its end
-      }
-    }
-    __syncthreads();
-    if (s_failed == 0) {
-      // exclusive scan of the counts by rank: the offsets of the one pass
-      const OffT c = s_count[tid];
-      OffT incl    = c;
-#pragma unroll
-      for (int delta = 1; delta < WAVE; delta <<= 1) {
-        const OffT t = __shfl_up(incl, delta, WAVE);
-        if (lane >= delta) {
-          incl += t;
-        }
-      }
-      if (lane == WAVE - 1) {
-        s_wsum[wave] = incl;
-      }
-      __syncthreads();
-      OffT prefix = 0;
-      for (int w = 0; w < wave; ++w) {
-        prefix += s_wsum[w];
-      }
-      hist[tid] = prefix + incl - c;
-      for (uint32_t j = tid; j < DISTINCT_LOOKUP; j += RADIX) {
-        table->lookup_keys[j] = s_lookup_keys[j];
-        table->lookup_rank[j] = s_lookup_rank[j];
-      }
-      if (tid < static_cast<int>(passes)) {
-        varying[tid] = (tid == 0) ? 1u : 0u;  // busy >= 2: the row holds at least two keys
-      }
-      if (tid == 0) {
-        plan->enabled  = VIRT_DISTINCT;
-        plan->n_groups = 1;
-      }
-      return;
-    }
   }
 
   if (tid == 0) {
