@@ -140,6 +140,40 @@ def algorithmic_bytes(cfg: dict, lds_limit_rows: bool, passes_run: int | None = 
 # -------------------------------------------------------------------------------------------------
 # GPU side
 # -------------------------------------------------------------------------------------------------
+def measure_device_rates(torch) -> dict:
+    """Streaming rates of the device on 1 GiB buffers with the framework's own kernels, outside the
+    timed region: a device-to-device copy (bytes read + written), a read-only reduction and a
+    write-only fill.  Reported beside the roofline so that the fraction of the published HBM peak
+    can be read against what a plain copy reaches on the same box."""
+    n = 1 << 28
+    src = torch.empty(n, dtype=torch.float32, device="cuda:0").normal_()
+    dst = torch.empty_like(src)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def best_ms(fn, reps=5, inner=5):
+        fn()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(reps):
+            e0.record()
+            for _ in range(inner):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            best = min(best, e0.elapsed_time(e1) / inner)
+        return best
+
+    nbytes = 4 * n
+    rates = {
+        "copy_GBps": 2 * nbytes / best_ms(lambda: dst.copy_(src)) / 1e6,
+        "read_GBps": nbytes / best_ms(lambda: src.sum()) / 1e6,
+        "fill_GBps": nbytes / best_ms(lambda: dst.zero_()) / 1e6,
+        "buffer_bytes": nbytes,
+    }
+    del src, dst
+    return rates
+
+
 class GpuJob:
     """Device buffers and the call sequence of one workload, through the C ABI."""
 
@@ -591,6 +625,7 @@ def main() -> None:
         for label, v in by_label.items()
     }
     traffic = MEASURED_TRAFFIC_BYTES.get((args.config, cfg["x"].size))
+    device_rates = measure_device_rates(torch)
     roofline = {
         "kernel": dominant,
         "bound": "hbm",
@@ -602,6 +637,10 @@ def main() -> None:
         "bytes_per_launch": alg[dominant],
         "avg_launch_ms": avg_ms,
         "launches_per_step": len(by_label[dominant]) / args.steps,
+        # what this device sustains on plain streaming kernels, measured in this run: the published
+        # peak is not reached by a copy either
+        "device_rates": device_rates,
+        "frac_of_device_copy": achieved / 1e9 / device_rates["copy_GBps"],
     }
     if "onesweep_baseline_formula" in alg and dominant == "onesweep":
         # for comparison only: the baseline's accounting moves an 8-byte payload in every pass, this
