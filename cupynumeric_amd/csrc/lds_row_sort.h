@@ -39,8 +39,12 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
                                                               KeyT* keys_out,
                                                               int64_t* idx_out,
                                                               uint32_t seg,
-                                                              int64_t index_offset)
+                                                              int64_t index_offset,
+                                                              uint32_t* status)
 {
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    *status = 0;  // the workspace's status word: a per-row sort cannot fail on the device
+  }
   constexpr int WAVES  = BLOCK / WAVE;
   constexpr int TILE   = BLOCK * ITEMS;
   constexpr int WTILE  = ITEMS * WAVE;

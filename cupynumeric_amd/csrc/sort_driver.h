@@ -243,7 +243,7 @@ inline int launch_lds_rows(const SortRequest& r)
     hipLaunchKernelGGL((lds_row_sort_kernel<KeyT, CODEC, HAS_IDX, BLOCK, ITEMS>),
                        dim3(static_cast<uint32_t>(rows)), dim3(BLOCK), 0, r.stream,
                        static_cast<const KeyT*>(r.values_in), static_cast<KeyT*>(r.values_out), r.indices_out,
-                       static_cast<uint32_t>(r.seg), r.index_offset);
+                       static_cast<uint32_t>(r.seg), r.index_offset, static_cast<uint32_t*>(r.temp));
   }
   CPN_HIP_TRY(hipGetLastError());
   return CPN_OK;
@@ -261,7 +261,7 @@ inline int launch_wave_rows(const SortRequest& r)
     hipLaunchKernelGGL((wave_row_sort_kernel<KeyT, CODEC, HAS_IDX, ITEMS, ROWS_PER_BLOCK>),
                        dim3(static_cast<uint32_t>(blocks)), dim3(WAVE * ROWS_PER_BLOCK), 0, r.stream,
                        static_cast<const KeyT*>(r.values_in), static_cast<KeyT*>(r.values_out), r.indices_out,
-                       static_cast<uint32_t>(r.seg), rows, r.index_offset);
+                       static_cast<uint32_t>(r.seg), rows, r.index_offset, static_cast<uint32_t*>(r.temp));
   }
   CPN_HIP_TRY(hipGetLastError());
   return CPN_OK;
@@ -277,7 +277,7 @@ inline int launch_tiny_rows(const SortRequest& r)
     ProfileScope prof("tiny_row_sort", r.stream);
     hipLaunchKernelGGL((tiny_row_sort_kernel<KeyT, CODEC, HAS_IDX, S>), dim3(static_cast<uint32_t>(blocks)), dim3(256),
                        0, r.stream, static_cast<const KeyT*>(r.values_in), static_cast<KeyT*>(r.values_out),
-                       r.indices_out, static_cast<uint32_t>(r.seg), rows, r.index_offset);
+                       r.indices_out, static_cast<uint32_t>(r.seg), rows, r.index_offset, static_cast<uint32_t*>(r.temp));
   }
   CPN_HIP_TRY(hipGetLastError());
   return CPN_OK;
@@ -577,10 +577,7 @@ int sort_typed(const SortRequest& r)
     return CPN_ERR_TEMP;
   }
   if (r.seg <= lds_row_limit(KB)) {
-    const int rc = launch_zero_fill(r.temp, HEADER_BYTES, r.stream);
-    if (rc != CPN_OK) {
-      return rc;
-    }
+    // one launch: the row kernels clear the status word of the workspace themselves
     return has_idx ? sort_rows_in_lds<KeyT, CODEC, true>(r) : sort_rows_in_lds<KeyT, CODEC, false>(r);
   }
   const GlobalLayout L = global_layout(KB, PASSES, r.volume, r.seg, r.values_out != nullptr, has_idx, in_place);

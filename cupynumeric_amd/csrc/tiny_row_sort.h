@@ -21,8 +21,12 @@ __global__ __launch_bounds__(256) void tiny_row_sort_kernel(const KeyT* keys_in,
                                                              int64_t* idx_out,
                                                              uint32_t seg,
                                                              uint64_t rows,
-                                                             int64_t index_offset)
+                                                             int64_t index_offset,
+                                                             uint32_t* status)
 {
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    *status = 0;  // the workspace's status word: a per-row sort cannot fail on the device
+  }
   using OW                = OrderedWords<CODEC, KeyT>;
   constexpr int NW        = OW::NW;
   constexpr int ROWS_WAVE = WAVE / S;

@@ -93,8 +93,12 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
                                                                               int64_t* idx_out,
                                                                               uint32_t seg,
                                                                               uint64_t rows,
-                                                                              int64_t index_offset)
+                                                                              int64_t index_offset,
+                                                                              uint32_t* status)
 {
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    *status = 0;  // the workspace's status word: a per-row sort cannot fail on the device
+  }
   using OW                = OrderedWords<CODEC, KeyT>;
   constexpr int NW        = OW::NW;
   constexpr int PASSES    = OW::PASSES;

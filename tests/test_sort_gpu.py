@@ -51,7 +51,7 @@ def abi_sort(lib, torch, x: np.ndarray, want_values=True, want_indices=False, in
     d_idx = torch.full((volume,), -7, dtype=torch.int64, device=dev) if want_indices else None
     tb = lib.cpn_local_sort_temp_bytes(code, volume, seg, int(want_values), int(want_indices), int(in_place))
     assert tb >= 1024
-    temp = torch.empty(tb, dtype=torch.uint8, device=dev)
+    temp = torch.full((tb,), 0xFF, dtype=torch.uint8, device=dev)  # a dirty workspace: the call clears what it needs
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     rc = lib.cpn_local_sort(
         code, d_in.data_ptr(), d_val.data_ptr() if want_values else None,
