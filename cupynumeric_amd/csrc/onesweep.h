@@ -189,6 +189,86 @@ __global__ __launch_bounds__(HIST_BLOCK) void histogram_kernel(const KeyT* __res
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// pass plan: which passes run and between which buffers, decided on the device
+// ---------------------------------------------------------------------------------------
+// Passes whose digit is the same for all keys of every row are skipped.  Which buffer a pass
+// reads and writes then depends on how many passes remain, which only the device knows after
+// the histogram sweep: a one-thread kernel writes one PassPlan per pass and the scatter
+// kernels look their buffers up by id.  The last running pass always writes the caller's
+// arrays; the ones before it alternate, walking backwards, between two scratch buffers.
+constexpr int MAX_PASSES = 24;
+enum KeyBuf : uint32_t { KEY_IN = 0, KEY_OUT = 1, KEY_T1 = 2, KEY_T2 = 3 };
+enum IdxBuf : uint32_t { IDX_FINAL = 1, IDX_T1 = 2, IDX_ALIAS = 3 };  // ALIAS: the int64 output used as narrow scratch
+constexpr uint32_t BUF_NONE = 0xFFu;
+
+struct PassPlan {
+  uint32_t active;   // 0: the pass exits at once
+  uint32_t key_src;  // KeyBuf
+  uint32_t key_dst;  // KeyBuf or BUF_NONE (index-only sort, last pass)
+  uint32_t idx_src;  // IdxBuf or BUF_NONE (first running pass: positions are synthesised)
+  uint32_t idx_dst;  // IdxBuf
+  uint32_t first;    // first running pass
+};
+
+struct SortPlan {
+  PassPlan pass[MAX_PASSES];
+  uint32_t n_active;
+};
+
+struct PlanRequest {
+  uint32_t passes;
+  uint32_t want_values;
+  uint32_t want_indices;
+  uint32_t in_place;
+};
+
+// One thread.  `varying` is read with device-scope loads: the flags may have been raised by other
+// workgroups of the same launch (make_plan at the end of the scan kernel).
+__device__ __forceinline__ void make_plan(const uint32_t* varying, SortPlan* __restrict__ plan, PlanRequest rq)
+{
+  uint32_t flags = 0;  // bit p: pass p runs
+  uint32_t k     = 0;
+  for (uint32_t p = 0; p < rq.passes; ++p) {
+    if (__hip_atomic_load(&varying[p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
+      flags |= 1u << p;
+      ++k;
+    }
+  }
+  plan->n_active = k;
+  // scratch partner of T1: the caller's value array when it is free to be overwritten early
+  const uint32_t key_x = (rq.want_values && !rq.in_place) ? KEY_OUT : KEY_T2;
+  uint32_t j = 0, key_prev = KEY_IN, idx_prev = BUF_NONE;
+  for (uint32_t p = 0; p < rq.passes; ++p) {
+    PassPlan e{};
+    if ((flags >> p) & 1u) {
+      ++j;
+      const uint32_t from_last = k - j;
+      e.active                 = 1;
+      e.first                  = (j == 1) ? 1u : 0u;
+      e.key_src                = key_prev;
+      e.idx_src                = idx_prev;
+      if (from_last == 0) {
+        e.key_dst = rq.want_values ? ((k == 1 && rq.in_place) ? KEY_T1 : KEY_OUT) : BUF_NONE;
+        e.idx_dst = IDX_FINAL;
+      } else {
+        e.key_dst = (from_last & 1u) ? KEY_T1 : key_x;
+        e.idx_dst = (from_last & 1u) ? IDX_T1 : IDX_ALIAS;
+      }
+      key_prev = e.key_dst;
+      idx_prev = e.idx_dst;
+    }
+    plan->pass[p] = e;
+  }
+}
+
+static __global__ void plan_kernel(const uint32_t* __restrict__ varying, SortPlan* __restrict__ plan, PlanRequest rq)
+{
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    make_plan(varying, plan, rq);
+  }
+}
+
 // One block per (row, pass): exclusive scan of 256 counts in place.  A pass on whose digit
 // all keys of a row agree (one bin holds the whole row) would be the identity permutation for
 // that row; `varying[pass]` is raised by every row for which that is not so.
@@ -198,7 +278,10 @@ __global__ __launch_bounds__(RADIX) void histogram_scan_kernel(OffT* __restrict_
                                                                uint64_t seg,
                                                                uint32_t passes,
                                                                const VirtPlan* __restrict__ vplan,
-                                                               uint32_t second)
+                                                               uint32_t second,
+                                                               uint32_t* __restrict__ blocks_done,
+                                                               SortPlan* __restrict__ plan,
+                                                               PlanRequest rq)
 {
   // first use (`second` == 0): nothing when the sort already runs on the ranks of the row's
   // different keys.  Second use, after vplan_kernel: scans the histograms of the grouped virtual
@@ -236,75 +319,18 @@ __global__ __launch_bounds__(RADIX) void histogram_scan_kernel(OffT* __restrict_
     prefix += s_wsum[w];
   }
   h[tid] = prefix + incl - c;
-}
-
-// ---------------------------------------------------------------------------------------
-// pass plan: which passes run and between which buffers, decided on the device
-// ---------------------------------------------------------------------------------------
-// Passes whose digit is the same for all keys of every row are skipped.  Which buffer a pass
-// reads and writes then depends on how many passes remain, which only the device knows after
-// the histogram sweep: a one-thread kernel writes one PassPlan per pass and the scatter
-// kernels look their buffers up by id.  The last running pass always writes the caller's
-// arrays; the ones before it alternate, walking backwards, between two scratch buffers.
-constexpr int MAX_PASSES = 24;
-enum KeyBuf : uint32_t { KEY_IN = 0, KEY_OUT = 1, KEY_T1 = 2, KEY_T2 = 3 };
-enum IdxBuf : uint32_t { IDX_FINAL = 1, IDX_T1 = 2, IDX_ALIAS = 3 };  // ALIAS: the int64 output used as narrow scratch
-constexpr uint32_t BUF_NONE = 0xFFu;
-
-struct PassPlan {
-  uint32_t active;   // 0: the pass exits at once
-  uint32_t key_src;  // KeyBuf
-  uint32_t key_dst;  // KeyBuf or BUF_NONE (index-only sort, last pass)
-  uint32_t idx_src;  // IdxBuf or BUF_NONE (first running pass: positions are synthesised)
-  uint32_t idx_dst;  // IdxBuf
-  uint32_t first;    // first running pass
-};
-
-struct SortPlan {
-  PassPlan pass[MAX_PASSES];
-  uint32_t n_active;
-};
-
-struct PlanRequest {
-  uint32_t passes;
-  uint32_t want_values;
-  uint32_t want_indices;
-  uint32_t in_place;
-};
-
-static __global__ void plan_kernel(const uint32_t* __restrict__ varying, SortPlan* __restrict__ plan, PlanRequest rq)
-{
-  if (threadIdx.x != 0 || blockIdx.x != 0) {
-    return;
-  }
-  uint32_t k = 0;
-  for (uint32_t p = 0; p < rq.passes; ++p) {
-    k += (varying[p] != 0) ? 1u : 0u;
-  }
-  plan->n_active = k;
-  // scratch partner of T1: the caller's value array when it is free to be overwritten early
-  const uint32_t key_x = (rq.want_values && !rq.in_place) ? KEY_OUT : KEY_T2;
-  uint32_t j = 0, key_prev = KEY_IN, idx_prev = BUF_NONE;
-  for (uint32_t p = 0; p < rq.passes; ++p) {
-    PassPlan e{};
-    if (varying[p] != 0) {
-      ++j;
-      const uint32_t from_last = k - j;
-      e.active                 = 1;
-      e.first                  = (j == 1) ? 1u : 0u;
-      e.key_src                = key_prev;
-      e.idx_src                = idx_prev;
-      if (from_last == 0) {
-        e.key_dst = rq.want_values ? ((k == 1 && rq.in_place) ? KEY_T1 : KEY_OUT) : BUF_NONE;
-        e.idx_dst = IDX_FINAL;
-      } else {
-        e.key_dst = (from_last & 1u) ? KEY_T1 : key_x;
-        e.idx_dst = (from_last & 1u) ? IDX_T1 : IDX_ALIAS;
+  // `blocks_done` given: the block that finishes last also makes the pass plan (saves a launch)
+  if (blocks_done != nullptr) {
+    __shared__ uint32_t s_last;
+    __syncthreads();  // this block's flag (thread 0, above) is on its way
+    if (tid == 0) {
+      __threadfence();
+      const uint32_t before = __hip_atomic_fetch_add(blocks_done, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+      s_last                = (before + 1 == gridDim.x) ? 1u : 0u;
+      if (s_last != 0) {
+        make_plan(varying, plan, rq);
       }
-      key_prev = e.key_dst;
-      idx_prev = e.idx_dst;
     }
-    plan->pass[p] = e;
   }
 }
 

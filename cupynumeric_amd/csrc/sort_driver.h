@@ -36,9 +36,10 @@ constexpr uint64_t WORKSPACE_ALIGN  = 256;
 // reads it with an ordinary load, and the tickets next door are under constant atomic traffic.
 constexpr uint64_t HEADER_BYTES     = 1024;
 constexpr uint64_t HEADER_TICKETS   = 128;
+constexpr uint64_t HEADER_SCAN_DONE = 240;  // blocks of the scan kernel that have finished
 constexpr uint64_t HEADER_VARYING   = 256;
 constexpr uint64_t HEADER_PLAN      = 384;
-static_assert(HEADER_TICKETS + 4 * MAX_PASSES <= HEADER_VARYING, "tickets overlap the flags");
+static_assert(HEADER_TICKETS + 4 * MAX_PASSES <= HEADER_SCAN_DONE, "tickets overlap the scan counter");
 static_assert(HEADER_VARYING + 4 * MAX_PASSES <= HEADER_PLAN, "flags overlap the plan");
 static_assert(HEADER_PLAN + sizeof(SortPlan) <= HEADER_BYTES, "plan does not fit the header");
 constexpr uint64_t BIG_ROW_ELEMENTS = 1ull << 30;
@@ -443,7 +444,8 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
       ProfileScope prof("histogram_scan", r.stream);
       hipLaunchKernelGGL((histogram_scan_kernel<OffT>), dim3(static_cast<uint32_t>(L.rows * PASSES)),
                          dim3(RADIX), 0, r.stream, hist, varying, r.seg, static_cast<uint32_t>(PASSES),
-                         static_cast<const VirtPlan*>(vplan), 0u);
+                         static_cast<const VirtPlan*>(vplan), 0u,
+                         L.virt ? nullptr : reinterpret_cast<uint32_t*>(ws + HEADER_SCAN_DONE), plan, rq);
     }
     CPN_HIP_TRY(hipGetLastError());
     if constexpr (VIRT_OK) {
@@ -466,16 +468,17 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
         {
           ProfileScope prof("virtual_scan", r.stream);
           hipLaunchKernelGGL((histogram_scan_kernel<OffT>), dim3(static_cast<uint32_t>(PASSES)), dim3(RADIX), 0,
-                             r.stream, hist, varying, r.seg, static_cast<uint32_t>(PASSES), vplan, 1u);
+                             r.stream, hist, varying, r.seg, static_cast<uint32_t>(PASSES), vplan, 1u,
+                             static_cast<uint32_t*>(nullptr), plan, rq);
         }
         CPN_HIP_TRY(hipGetLastError());
       }
     }
-    {
+    if (L.virt) {  // otherwise the scan kernel has made the plan
       ProfileScope prof("plan", r.stream);
       hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(WAVE), 0, r.stream, varying, plan, rq);
+      CPN_HIP_TRY(hipGetLastError());
     }
-    CPN_HIP_TRY(hipGetLastError());
   }
 
   // The buffers a pass may read or write; which ones it uses is in the device-side plan.
