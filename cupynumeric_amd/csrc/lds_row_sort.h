@@ -93,7 +93,7 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
         all_and[n] &= w[n];
         all_or[n] |= w[n];
       }
-      if constexpr (IMAGES_OK) {
+      if constexpr (CODEC == CODEC_FLOAT) {
         special |= (static_cast<KeyT>(w[0]) != sign_flip(key[i])) ? 1 : 0;
       }
     } else {
@@ -115,6 +115,14 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
   }
   const int any_special = __syncthreads_or(special);
   const bool images     = IMAGES_OK && (any_special == 0);
+  // Sorts that return keys only: the first pass to run need not be stable.  Keys that tie in every
+  // digit are the same bits (float rows with a NaN or a -0.0, where different bits tie, are left
+  // out; so are complex keys), so nothing shows in which order that pass leaves equal digits, and
+  // every later pass is stable.  Its ranks then come from one LDS atomic per key on counters
+  // shared by the workgroup instead of the ballots of the stable ranking.
+  const bool free_first = !HAS_IDX && (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED ||
+                                       (CODEC == CODEC_FLOAT && any_special == 0));
+  bool first_running    = true;
   SW varying[NW];
 #pragma unroll
   for (int n = 0; n < NW; ++n) {
@@ -194,8 +202,14 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
       const bool valid = full || (woff + i * WAVE < seg);
       const uint32_t d = digit_of(key[i], pass);
       dpk[i / 4]       = (i % 4 == 0) ? d : (dpk[i / 4] | (d << (8 * (i % 4))));
-      rnk[i]           = wave_match_rank(d, valid, wctr);
+      if (!HAS_IDX && free_first && first_running) {  // uniform
+        rnk[i] = valid ? atomicAdd(&s_ctr[d], 1u) : 0u;  // wave 0's counters serve the whole workgroup
+      } else {
+        rnk[i] = wave_match_rank(d, valid, wctr);
+      }
     }
+    const uint32_t* base = (!HAS_IDX && free_first && first_running) ? s_ctr : wctr;
+    first_running        = false;
     __syncthreads();
     // exclusive scan over (digit, wave) in digit-major order
     uint32_t tsum = 0, tincl = 0;
@@ -235,7 +249,7 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
     for (int i = 0; i < ITEMS; ++i) {
       if (full || (woff + i * WAVE < seg)) {
         const uint32_t d   = (dpk[i / 4] >> (8 * (i % 4))) & 0xFFu;
-        const uint32_t pos = wctr[d] + rnk[i];
+        const uint32_t pos = base[d] + rnk[i];
         s_keys[pos]        = key[i];
         if constexpr (HAS_IDX) {
           s_idx[pos] = static_cast<IdxS>(idx[i]);

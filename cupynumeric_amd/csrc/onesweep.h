@@ -471,6 +471,12 @@ __device__ __forceinline__ void onesweep_tile(
   }
 
   // ---- rank inside the wave (counters run from zero), count digits per wave ----
+  // Sorts of integer keys that return keys only: the first pass to run need not be stable (keys
+  // that tie in every digit are the same bits and every later pass is stable), so its ranks come
+  // from one LDS atomic per key on the counters of wave 0, which then serve the whole tile.
+  constexpr bool FREE_FIRST_OK = !HAS_IDX && !VIRT && (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED);
+  const bool free_first        = FREE_FIRST_OK && (a.first != 0);
+  const uint32_t* rank_base    = free_first ? sh.ctr : wctr;
   uint32_t dpk[ITEMS / 4];   // the digits, four per register
   uint32_t rnk2[ITEMS / 2];  // rank among the wave's keys of the same digit, two per register
 #pragma unroll
@@ -485,7 +491,12 @@ __device__ __forceinline__ void onesweep_tile(
       d = KeyTraits<DCODEC, KeyT>::digit(key[i], a.pass);
     }
     dpk[i / 4]       = (i % 4 == 0) ? d : (dpk[i / 4] | (d << (8 * (i % 4))));
-    const uint32_t r = wave_match_rank(d, valid, wctr) & 0xFFFFu;
+    uint32_t r;
+    if (FREE_FIRST_OK && free_first) {  // uniform
+      r = valid ? atomicAdd(&sh.ctr[d], 1u) : 0u;
+    } else {
+      r = wave_match_rank(d, valid, wctr) & 0xFFFFu;
+    }
     rnk2[i / 2]      = (i % 2 == 0) ? r : (rnk2[i / 2] | (r << 16));
     // the packed registers are opaque to the optimiser, which would otherwise keep every
     // digit and rank alive in a register of its own until the scatter phase
@@ -544,7 +555,7 @@ __device__ __forceinline__ void onesweep_tile(
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t d   = (dpk[i / 4] >> (8 * (i % 4))) & 0xFFu;
-    const uint32_t pos = (wctr[d] + ((rnk2[i / 2] >> (16 * (i % 2))) & 0xFFFFu)) & 0xFFFFu;
+    const uint32_t pos = (rank_base[d] + ((rnk2[i / 2] >> (16 * (i % 2))) & 0xFFFFu)) & 0xFFFFu;
     if (FULL || (woff + i * WAVE < count)) {
       if (VIRT && digits_only) {
         reinterpret_cast<uint8_t*>(s_keys)[pos] = static_cast<uint8_t>(d);

@@ -124,6 +124,7 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
   uint32_t w[ITEMS][NW];
   uint32_t pos2[CARRY ? (ITEMS + 1) / 2 : 1];  // source positions, two per register
   uint32_t vary_and[NW], vary_or[NW];
+  bool special = false;  // float keys: a NaN or a -0.0 (different bits that tie)
 #pragma unroll
   for (int n = 0; n < NW; ++n) {
     vary_and[n] = 0xFFFFFFFFu;
@@ -133,11 +134,15 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t o = i * WAVE + lane;
     if (full || o < seg) {
-      OW::encode(keys_in[base + o], w[i]);
+      const KeyT raw = keys_in[base + o];
+      OW::encode(raw, w[i]);
 #pragma unroll
       for (int n = 0; n < NW; ++n) {
         vary_and[n] &= w[i][n];
         vary_or[n] |= w[i][n];
+      }
+      if constexpr (CODEC == CODEC_FLOAT && !HAS_IDX) {
+        special = special || (ordered_bits<CODEC_FLOAT, KeyT>(raw) != sign_flip(raw));
       }
     } else {
 #pragma unroll
@@ -185,6 +190,11 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
     }
   }
 
+  // Sorts that return keys only: the first pass to run need not be stable (keys that tie in every
+  // digit are the same bits, unless a float row holds a NaN or a -0.0; complex keys are left out),
+  // so its ranks come from one LDS atomic per key instead of the ballots of the stable ranking.
+  const bool free_first = !HAS_IDX && (OW::BIJECT || (CODEC == CODEC_FLOAT && __builtin_amdgcn_ballot_w64(special) == 0));
+  bool first_running    = true;
   for (;;) {
   for (int pass = 0; pass < PASSES; ++pass) {
     if (((todo >> pass) & 1u) == 0) {
@@ -208,12 +218,19 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
         wsel = (word == n) ? w[i][n] : wsel;
       }
       const uint32_t d = (wsel >> shift) & 0xFFu;
-      const uint32_t r = wave_match_rank(d, full || (i * WAVE + lane < seg), ctr) & 0xFFFFu;
+      const bool valid = full || (i * WAVE + lane < seg);
+      uint32_t r;
+      if (!HAS_IDX && free_first && first_running) {  // uniform
+        r = valid ? atomicAdd(&ctr[d], 1u) : 0u;
+      } else {
+        r = wave_match_rank(d, valid, ctr) & 0xFFFFu;
+      }
       dpk[i / 4]       = (i % 4 == 0) ? d : (dpk[i / 4] | (d << (8 * (i % 4))));
       rnk2[i / 2]      = (i % 2 == 0) ? r : (rnk2[i / 2] | (r << 16));
       // opaque to the optimiser, which would otherwise keep one register per digit and rank
       asm volatile("" : "+v"(dpk[i / 4]), "+v"(rnk2[i / 2]));
     }
+    first_running = false;
     // ---- exclusive scan of the 256 counts: lane l owns digits 4l .. 4l+3 ----
     {
       uint32_t c[RADIX / WAVE], sum = 0;
