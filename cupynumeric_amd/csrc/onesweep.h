@@ -86,31 +86,40 @@ constexpr int HIST_BLOCK = 256;
 // (complex keys: 9 passes x 4 copies, 17 passes x 2 copies).
 __host__ __device__ constexpr int hist_copies(int passes) { return passes <= 4 ? 8 : (passes <= 9 ? 4 : 2); }
 
-template <typename KeyT, int CODEC, int PASSES>
-__device__ __forceinline__ void hist_accumulate(uint32_t* s_hist, KeyT raw, uint32_t copy)
+// Returns whether `raw` is a float key whose bits are not determined by its place in the order
+// (a NaN or a -0.0); false for every other key type.
+template <typename KeyT, int CODEC, int PASSES, bool SPECIALS>
+__device__ __forceinline__ bool hist_accumulate(uint32_t* s_hist, KeyT raw, uint32_t copy)
 {
   using KT                  = KeyTraits<CODEC, KeyT>;
   constexpr int HIST_COPIES = hist_copies(PASSES);
   uint64_t w[KT::NWORDS];
   KT::words(raw, w);
+  bool special = false;
+  if constexpr (SPECIALS) {
+    special = static_cast<KeyT>(w[0]) != sign_flip(raw);
+  }
 #pragma unroll
   for (int p = 0; p < PASSES; ++p) {
     const uint32_t d = static_cast<uint32_t>(w[p / 8] >> ((p % 8) * RADIX_BITS)) & 0xFFu;
     atomicAdd(&s_hist[(p * RADIX + d) * HIST_COPIES + copy], 1u);
   }
+  return special;
 }
 
 // grid = rows * blocks_per_row; block b of a row covers elements [b*chunk, min(seg, (b+1)*chunk)).
 // 128-bit loads over the 16-byte aligned middle of the chunk, scalar head and tail.
 // `vplan` (may be null): nothing to do when the sort already runs on the ranks of the row's
 // different keys (virtual_digits.h).
-template <typename KeyT, int CODEC, typename OffT>
+// SPECIALS (float keys, keys-only sorts): also tells through `specials` whether a NaN or a -0.0 occurs.
+template <typename KeyT, int CODEC, typename OffT, bool SPECIALS = false>
 __global__ __launch_bounds__(HIST_BLOCK) void histogram_kernel(const KeyT* __restrict__ keys,
                                                                  OffT* __restrict__ hist,
                                                                  uint64_t seg,
                                                                  uint32_t blocks_per_row,
                                                                  uint64_t chunk,
-                                                                 const VirtPlan* __restrict__ vplan)
+                                                                 const VirtPlan* __restrict__ vplan,
+                                                                 uint32_t* __restrict__ specials)
 {
   constexpr int PASSES      = KeyTraits<CODEC, KeyT>::PASSES;
   constexpr int VEC         = 16 / sizeof(KeyT);
@@ -133,6 +142,7 @@ __global__ __launch_bounds__(HIST_BLOCK) void histogram_kernel(const KeyT* __res
     s_hist[j] = 0;
   }
   __syncthreads();
+  bool special = false;  // float keys: a NaN or a -0.0 among this thread's keys
 
   if (begin < end) {
     const KeyT* p = keys + row * seg;
@@ -143,7 +153,7 @@ __global__ __launch_bounds__(HIST_BLOCK) void histogram_kernel(const KeyT* __res
       head = end - begin;
     }
     for (uint64_t i = tid; i < head; i += HIST_BLOCK) {
-      hist_accumulate<KeyT, CODEC, PASSES>(s_hist, p[begin + i], copy);
+      special |= hist_accumulate<KeyT, CODEC, PASSES, SPECIALS>(s_hist, p[begin + i], copy);
     }
     const uint64_t vbegin = begin + head;
     const uint64_t nvec   = (end - vbegin) / VEC;
@@ -158,7 +168,7 @@ __global__ __launch_bounds__(HIST_BLOCK) void histogram_kernel(const KeyT* __res
       __builtin_memcpy(k + VEC, &q1, 16);
 #pragma unroll
       for (int j = 0; j < 2 * VEC; ++j) {
-        hist_accumulate<KeyT, CODEC, PASSES>(s_hist, k[j], copy);
+        special |= hist_accumulate<KeyT, CODEC, PASSES, SPECIALS>(s_hist, k[j], copy);
       }
     }
     for (; v < nvec; v += HIST_BLOCK) {
@@ -167,14 +177,23 @@ __global__ __launch_bounds__(HIST_BLOCK) void histogram_kernel(const KeyT* __res
       __builtin_memcpy(k, &q, 16);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
-        hist_accumulate<KeyT, CODEC, PASSES>(s_hist, k[j], copy);
+        special |= hist_accumulate<KeyT, CODEC, PASSES, SPECIALS>(s_hist, k[j], copy);
       }
     }
     for (uint64_t i = vbegin + nvec * VEC + tid; i < end; i += HIST_BLOCK) {
-      hist_accumulate<KeyT, CODEC, PASSES>(s_hist, p[i], copy);
+      special |= hist_accumulate<KeyT, CODEC, PASSES, SPECIALS>(s_hist, p[i], copy);
     }
   }
-  __syncthreads();
+  // (the barrier also ends the accumulation) `specials`: does any float key of the sort tie with
+  // keys of other bits?  The first pass of a keys-only sort may ignore stability if not.
+  if constexpr (SPECIALS) {
+    const int any_special = __syncthreads_or(special ? 1 : 0);
+    if (any_special != 0 && tid == 0) {
+      __hip_atomic_store(specials, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  } else {
+    __syncthreads();
+  }
 
   OffT* out = hist + row * (PASSES * RADIX);
   for (int j = tid; j < PASSES * RADIX; j += HIST_BLOCK) {
@@ -208,8 +227,10 @@ struct PassPlan {
   uint32_t key_dst;  // KeyBuf or BUF_NONE (index-only sort, last pass)
   uint32_t idx_src;  // IdxBuf or BUF_NONE (first running pass: positions are synthesised)
   uint32_t idx_dst;  // IdxBuf
-  uint32_t first;    // first running pass
+  uint32_t first;    // bit 0: first running pass; bit 1: that pass need not be stable (PLAN_FREE_RANK)
 };
+constexpr uint32_t PLAN_FIRST     = 1u;
+constexpr uint32_t PLAN_FREE_RANK = 2u;
 
 struct SortPlan {
   PassPlan pass[MAX_PASSES];
@@ -221,6 +242,11 @@ struct PlanRequest {
   uint32_t want_values;
   uint32_t want_indices;
   uint32_t in_place;
+  // Keys-only sorts: the first running pass need not be stable when keys that tie in every digit
+  // are the same bits: always for integer keys (free_rank = 1, specials = nullptr); for float
+  // keys unless the histogram sweep met a NaN or a -0.0 (*specials != 0).
+  uint32_t free_rank;
+  const uint32_t* specials;
 };
 
 // One thread.  `varying` is read with device-scope loads: the flags may have been raised by other
@@ -245,7 +271,11 @@ __device__ __forceinline__ void make_plan(const uint32_t* varying, SortPlan* __r
       ++j;
       const uint32_t from_last = k - j;
       e.active                 = 1;
-      e.first                  = (j == 1) ? 1u : 0u;
+      e.first                  = (j == 1) ? PLAN_FIRST : 0u;
+      if (j == 1 && rq.free_rank != 0 &&
+          (rq.specials == nullptr || __hip_atomic_load(rq.specials, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)) {
+        e.first |= PLAN_FREE_RANK;
+      }
       e.key_src                = key_prev;
       e.idx_src                = idx_prev;
       if (from_last == 0) {
@@ -398,6 +428,7 @@ struct SweepArgs {
   uint32_t spin_limit;     // polls of one descriptor before the tile gives up (LOOKBACK_SPIN_LIMIT)
   const VirtPlan* vplan;   // virtual digits (virtual_digits.h), nullptr when the request cannot use them
   const DistinctTable* dtable;  // with vplan: the row's different keys when there are at most 256
+  int free_rank;                // from the plan: this pass need not be stable
 };
 
 #ifndef CPN_ONESWEEP_WAVES_PER_EU
@@ -471,11 +502,13 @@ __device__ __forceinline__ void onesweep_tile(
   }
 
   // ---- rank inside the wave (counters run from zero), count digits per wave ----
-  // Sorts of integer keys that return keys only: the first pass to run need not be stable (keys
-  // that tie in every digit are the same bits and every later pass is stable), so its ranks come
-  // from one LDS atomic per key on the counters of wave 0, which then serve the whole tile.
-  constexpr bool FREE_FIRST_OK = !HAS_IDX && !VIRT && (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED);
-  const bool free_first        = FREE_FIRST_OK && (a.first != 0);
+  // Sorts that return keys only: the first pass to run need not be stable (keys that tie in
+  // every digit are the same bits, unless float keys hold a NaN or a -0.0, which the histogram
+  // sweep has looked for; complex keys are left out; every later pass is stable), so its ranks
+  // come from one LDS atomic per key on the counters of wave 0, which then serve the whole tile.
+  constexpr bool FREE_FIRST_OK =
+    !HAS_IDX && !VIRT && (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT);
+  const bool free_first = FREE_FIRST_OK && (a.free_rank != 0);
   const uint32_t* rank_base    = free_first ? sh.ctr : wctr;
   uint32_t dpk[ITEMS / 4];   // the digits, four per register
   uint32_t rnk2[ITEMS / 2];  // rank among the wave's keys of the same digit, two per register
@@ -775,7 +808,8 @@ void onesweep_kernel(const SweepArgs<BIG> a_in)
   a.idx_in         = (pp.idx_src == BUF_NONE) ? nullptr : static_cast<const OffT*>(a_in.idx_buf[pp.idx_src]);
   a.idx_out        = a_in.idx_buf[pp.idx_dst];
   a.idx_final      = (pp.idx_dst == IDX_FINAL) ? 1 : 0;
-  a.first          = static_cast<int>(pp.first);
+  a.first          = static_cast<int>(pp.first & PLAN_FIRST);
+  a.free_rank      = static_cast<int>((pp.first & PLAN_FREE_RANK) != 0);
 
   const int tid = threadIdx.x;
   // Tiles are handed out in launch order of the workgroups that are actually running, so

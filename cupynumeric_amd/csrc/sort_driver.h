@@ -37,6 +37,7 @@ constexpr uint64_t WORKSPACE_ALIGN  = 256;
 constexpr uint64_t HEADER_BYTES     = 1024;
 constexpr uint64_t HEADER_TICKETS   = 128;
 constexpr uint64_t HEADER_SCAN_DONE = 240;  // blocks of the scan kernel that have finished
+constexpr uint64_t HEADER_SPECIALS  = 244;  // float keys: the sort holds a NaN or a -0.0
 constexpr uint64_t HEADER_VARYING   = 256;
 constexpr uint64_t HEADER_PLAN      = 384;
 static_assert(HEADER_TICKETS + 4 * MAX_PASSES <= HEADER_SCAN_DONE, "tickets overlap the scan counter");
@@ -387,6 +388,8 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
   rq.want_values  = want_vals ? 1u : 0u;
   rq.want_indices = HAS_IDX ? 1u : 0u;
   rq.in_place     = in_place ? 1u : 0u;
+  rq.free_rank    = (!HAS_IDX && (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT)) ? 1u : 0u;
+  rq.specials     = (CODEC == CODEC_FLOAT) ? reinterpret_cast<const uint32_t*>(ws + HEADER_SPECIALS) : nullptr;
 
   // histogram sweep: about 2048 blocks in total, at least one per row
   {
@@ -435,9 +438,11 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
     }
     {
       ProfileScope prof("histogram", r.stream);
-      hipLaunchKernelGGL((histogram_kernel<KeyT, CODEC, OffT>), dim3(static_cast<uint32_t>(grid)),
+      constexpr bool SPECIALS = (CODEC == CODEC_FLOAT) && !HAS_IDX;  // who may rank its first pass freely
+      hipLaunchKernelGGL((histogram_kernel<KeyT, CODEC, OffT, SPECIALS>), dim3(static_cast<uint32_t>(grid)),
                          dim3(HIST_BLOCK), 0, r.stream, static_cast<const KeyT*>(r.values_in), hist, r.seg,
-                         static_cast<uint32_t>(bpr), chunk, static_cast<const VirtPlan*>(vplan));
+                         static_cast<uint32_t>(bpr), chunk, static_cast<const VirtPlan*>(vplan),
+                         reinterpret_cast<uint32_t*>(ws + HEADER_SPECIALS));
     }
     CPN_HIP_TRY(hipGetLastError());
     {
