@@ -108,12 +108,13 @@ int64_t cpn_set_lookback_spin_limit(int64_t polls);
 
 /*
  * Process-wide tunable: a 1-D sort of real 8-byte keys with at least `elements` elements lets
- * the device replace its eight byte passes by fewer passes on "virtual digits" when the
+ * the device replace its eight byte passes by one pass on the ranks of the keys when the row
+ * holds at most 256 different keys, or by fewer passes on "virtual digits" when the
  * histograms show that the bytes of the keys take few distinct values (several bytes then
  * share one 8-bit digit; cupynumeric_amd/csrc/virtual_digits.h).  Results do not depend on
  * it.  The default is 2^26 (below that the extra launches outweigh the average gain); a
  * negative value restores it and the previous setting is returned.  It changes workspace
- * sizes by 4096 bytes (cpn_local_sort_temp_bytes follows).  Also initialised from the
+ * sizes by 24 KiB (cpn_local_sort_temp_bytes follows).  Also initialised from the
  * environment variable CPN_SORT_VIRTUAL_DIGIT_THRESHOLD.
  */
 int64_t cpn_set_virtual_digit_threshold(int64_t elements);
