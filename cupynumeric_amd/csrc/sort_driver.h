@@ -431,7 +431,7 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
         {
           ProfileScope prof("distinct_plan", r.stream);
           hipLaunchKernelGGL((distinct_plan_kernel<OffT>), dim3(1), dim3(RADIX), 0, r.stream, hist, varying, vplan,
-                             dtable, static_cast<uint32_t>(PASSES));
+                             dtable, r.seg, static_cast<uint32_t>(PASSES));
         }
         CPN_HIP_TRY(hipGetLastError());
       }

@@ -124,7 +124,7 @@ __device__ __forceinline__ void distinct_collect(uint64_t image, uint64_t* keys,
   uint32_t h = distinct_hash(image, 9);
   static_assert(DISTINCT_LOCAL == 512, "hash width");
   for (uint32_t probe = 0; probe < DISTINCT_MAX_PROBES; ++probe) {
-    uint64_t cur = keys[h];
+    uint64_t cur = __hip_atomic_load(&keys[h], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     if (cur == 0) {
       cur = atomicCAS(reinterpret_cast<unsigned long long*>(&keys[h]), 0ull, static_cast<unsigned long long>(image));
       if (cur == 0) {
@@ -304,12 +304,13 @@ __global__ __launch_bounds__(DSWEEP_BLOCK) void distinct_sweep_kernel(const KeyT
 // 256 different keys): ranks them, writes the offsets of the one pass into hist[0][*], the lookup
 // table of the scatter pass, varying[] (pass 0 runs unless all keys are equal) and
 // plan->enabled = VIRT_DISTINCT, after which the histogram sweep and the other plan kernels have
-// nothing to do.  Otherwise leaves everything alone.
+// nothing to do.  Otherwise (also when the counts do not add up to `seg`) leaves everything alone.
 template <typename OffT>
 __global__ __launch_bounds__(RADIX) void distinct_plan_kernel(OffT* __restrict__ hist,
                                                                uint32_t* __restrict__ varying,
                                                                VirtPlan* __restrict__ plan,
                                                                DistinctTable* __restrict__ table,
+                                                               uint64_t seg,
                                                                uint32_t passes)
 {
   __shared__ uint64_t s_keys[DISTINCT_MAX];  // the row's different keys (other than image 0), unordered
@@ -397,6 +398,15 @@ __global__ __launch_bounds__(RADIX) void distinct_plan_kernel(OffT* __restrict__
     OffT prefix = 0;
     for (int w = 0; w < wave; ++w) {
       prefix += s_wsum[w];
+    }
+    // the counts must add up to the row: offsets from a table that lost or doubled a key would
+    // send the scatter pass out of the row, so such a table is not used
+    if (tid == RADIX - 1 && static_cast<uint64_t>(prefix + incl) != seg) {
+      s_failed = 1;
+    }
+    __syncthreads();
+    if (s_failed != 0) {
+      return;
     }
     hist[tid] = prefix + incl - c;
     for (uint32_t j = tid; j < DISTINCT_LOOKUP; j += RADIX) {
