@@ -551,6 +551,66 @@ def test_sort_call_is_capturable_into_a_graph(lib, torch_cuda):
         assert np.array_equal(i, oracle.local_sort(x[:5000], argsort=True))
 
 
+def test_captured_sort_switches_plans_between_replays(lib, torch_cuda, virtual_digits_from_2_to_20):
+    """A captured sort of 8-byte keys whose input changes between replays from few different keys (one pass
+    on their ranks) to few values per byte (grouped digits) to random keys (byte passes) and back: every
+    decision is taken on the device from the data of that replay, and the tables in the workspace are
+    cleared by the call itself."""
+    torch = torch_cuda
+    dev = torch.device("cuda")
+    rng = np.random.default_rng(21)
+    n = (1 << 20) + 777
+    code = _lib.DTYPE_CODES[np.dtype(np.int64)]
+    d_in = torch.zeros(n, dtype=torch.int64, device=dev)
+    d_val = torch.zeros(n, dtype=torch.int64, device=dev)
+    d_idx = torch.zeros(n, dtype=torch.int64, device=dev)
+    tb = lib.cpn_local_sort_temp_bytes(code, n, n, 1, 1, 0)
+    temp = torch.full((tb,), 0xFF, dtype=torch.uint8, device=dev)
+
+    def enqueue():
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        rc = lib.cpn_local_sort(code, d_in.data_ptr(), d_val.data_ptr(), d_idx.data_ptr(), n, n, 0, 1,
+                                temp.data_ptr(), tb, stream)
+        assert rc == 0, _lib.status_string(rc)
+
+    def few_keys():
+        return _few_values(rng, np.int64, n, 16)
+
+    def few_per_byte():
+        x = np.zeros(n, dtype=np.uint64)
+        for b in range(8):
+            x |= rng.integers(0, 256, 4).astype(np.uint64)[rng.integers(0, 4, n)] << np.uint64(8 * b)
+        return x.view(np.int64)
+
+    def random_keys():
+        return rng.integers(-(2**63), 2**63 - 1, n, dtype=np.int64)
+
+    def all_equal():
+        return np.full(n, 12345, dtype=np.int64)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        enqueue()  # warm-up outside capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        enqueue()
+    for rep, make in enumerate([few_keys, few_per_byte, random_keys, few_keys, all_equal, random_keys, few_per_byte]):
+        x = make()
+        d_in.copy_(torch.from_numpy(x))
+        d_idx.fill_(-1)
+        d_val.fill_(-1)
+        graph.replay()
+        torch.cuda.synchronize()
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        assert lib.cpn_local_sort_check(temp.data_ptr(), stream) == 0
+        assert np.array_equal(d_idx.cpu().numpy(), oracle.local_sort(x, argsort=True, threads=8)), f"replay {rep} {make.__name__}"
+        assert np.array_equal(d_val.cpu().numpy(), oracle.local_sort(x, argsort=False, threads=8)), f"replay {rep} {make.__name__}"
+        abi_sort(lib, torch, x[:3000], want_values=True, want_indices=True)  # eager work between the replays
+
+
 # ---- concurrent callers ------------------------------------------------------------------------------------
 def test_concurrent_streams_and_threads(lib, torch_cuda):
     """Two host threads, each with its own stream, buffers and workspace, sort at the same time: the
