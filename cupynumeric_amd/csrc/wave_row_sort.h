@@ -41,6 +41,19 @@ struct OrderedWords {
       w[n] = static_cast<uint32_t>(q[n / 2] >> ((n % 2) * 32));
     }
   }
+  // float keys that are neither NaN nor -0.0: the image determines the bits
+  static __device__ __forceinline__ KeyT decode_plain_float(const uint32_t (&w)[NW])
+  {
+    if constexpr (CODEC == CODEC_FLOAT && sizeof(KeyT) <= 8) {
+      uint64_t v = w[0];
+      if constexpr (NW > 1) {
+        v |= static_cast<uint64_t>(w[1]) << 32;
+      }
+      return sign_unflip(static_cast<KeyT>(v));
+    } else {
+      return KeyT{};
+    }
+  }
   // only for bijective codecs
   static __device__ __forceinline__ KeyT decode(const uint32_t (&w)[NW])
   {
@@ -154,6 +167,11 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
       pos2[i / 2] = (i % 2 == 0) ? o : (pos2[i / 2] | (o << 16));
     }
   }
+  // float rows without a NaN or a -0.0 (keys-only sorts look for them): the ordered words are
+  // then a bijection of the bits, so the source positions need not travel and the keys are
+  // decoded at the end like integer keys
+  const bool plain_floats = (CODEC == CODEC_FLOAT) && !HAS_IDX && (__builtin_amdgcn_ballot_w64(special) == 0);
+  const bool carry        = CARRY && !plain_floats;
   // passes on whose digit the whole row agrees are the identity permutation: skip them
   uint32_t active = 0;
 #pragma unroll
@@ -193,7 +211,7 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
   // Sorts that return keys only: the first pass to run need not be stable (keys that tie in every
   // digit are the same bits, unless a float row holds a NaN or a -0.0; complex keys are left out),
   // so its ranks come from one LDS atomic per key instead of the ballots of the stable ranking.
-  const bool free_first = !HAS_IDX && (OW::BIJECT || (CODEC == CODEC_FLOAT && __builtin_amdgcn_ballot_w64(special) == 0));
+  const bool free_first = !HAS_IDX && (OW::BIJECT || plain_floats);
   bool first_running    = true;
   for (;;) {
   for (int pass = 0; pass < PASSES; ++pass) {
@@ -257,7 +275,7 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
         for (int n = 0; n < NW; ++n) {
           s_words[wave][n][p] = w[i][n];
         }
-        if constexpr (CARRY) {
+        if (CARRY && carry) {
           s_pos[wave][p] = static_cast<uint16_t>(pos2[i / 2] >> (16 * (i % 2)));
         }
       }
@@ -271,7 +289,7 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
         for (int n = 0; n < NW; ++n) {
           w[i][n] = s_words[wave][n][o];
         }
-        if constexpr (CARRY) {
+        if (CARRY && carry) {
           const uint32_t q = s_pos[wave][o];
           pos2[i / 2]      = (i % 2 == 0) ? q : (pos2[i / 2] | (q << 16));
         }
@@ -327,7 +345,7 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
               s_words[wave][n][q]     = b[n];
               s_words[wave][n][q + 1] = a[n];
             }
-            if constexpr (CARRY) {
+            if (CARRY && carry) {
               const uint16_t t   = s_pos[wave][q];
               s_pos[wave][q]     = s_pos[wave][q + 1];
               s_pos[wave][q + 1] = t;
@@ -344,7 +362,7 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
           for (int n = 0; n < NW; ++n) {
             w[i][n] = s_words[wave][n][o];
           }
-          if constexpr (CARRY) {
+          if (CARRY && carry) {
             const uint32_t q = s_pos[wave][o];
             pos2[i / 2]      = (i % 2 == 0) ? q : (pos2[i / 2] | (q << 16));
           }
@@ -368,6 +386,8 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
       if (full || o < seg) {
         if constexpr (OW::BIJECT) {
           v[i] = OW::decode(w[i]);
+        } else if (!carry) {
+          v[i] = OW::decode_plain_float(w[i]);
         } else {
           v[i] = keys_in[base + ((pos2[i / 2] >> (16 * (i % 2))) & 0xFFFFu)];  // every gather of the row is issued before any store
         }
@@ -375,7 +395,7 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
         v[i] = KeyT{};
       }
     }
-    if constexpr (!OW::BIJECT) {
+    if (!OW::BIJECT && carry) {
       // keys_out may alias keys_in: every gather of the row must have returned before the
       // first store overwrites it (the asm also keeps the compiler from moving either across)
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
