@@ -116,7 +116,10 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
   constexpr int NW        = OW::NW;
   constexpr int PASSES    = OW::PASSES;
   constexpr int TILE      = ITEMS * WAVE;
-  constexpr bool CARRY    = HAS_IDX || !OW::BIJECT;  // source positions travel with the keys
+  // Float keys without indices: the sorted images give back every key but NaNs and zeros, whose
+  // bits the image does not hold; those are put in place at the end from a second look at the input.
+  constexpr bool FLOAT_KEYS_ONLY = (CODEC == CODEC_FLOAT) && !HAS_IDX && sizeof(KeyT) <= 8;
+  constexpr bool CARRY           = HAS_IDX || !(OW::BIJECT || FLOAT_KEYS_ONLY);  // source positions travel with the keys
   static_assert(TILE <= 65536, "positions are 16 bits");
 
   __shared__ uint32_t s_words[ROWS_PER_BLOCK][NW][TILE];
@@ -168,10 +171,8 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
     }
   }
   // float rows without a NaN or a -0.0 (keys-only sorts look for them): the ordered words are
-  // then a bijection of the bits, so the source positions need not travel and the keys are
-  // decoded at the end like integer keys
+  // then a bijection of the bits
   const bool plain_floats = (CODEC == CODEC_FLOAT) && !HAS_IDX && (__builtin_amdgcn_ballot_w64(special) == 0);
-  const bool carry        = CARRY && !plain_floats;
   // passes on whose digit the whole row agrees are the identity permutation: skip them
   uint32_t active = 0;
 #pragma unroll
@@ -275,7 +276,7 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
         for (int n = 0; n < NW; ++n) {
           s_words[wave][n][p] = w[i][n];
         }
-        if (CARRY && carry) {
+        if constexpr (CARRY) {
           s_pos[wave][p] = static_cast<uint16_t>(pos2[i / 2] >> (16 * (i % 2)));
         }
       }
@@ -289,7 +290,7 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
         for (int n = 0; n < NW; ++n) {
           w[i][n] = s_words[wave][n][o];
         }
-        if (CARRY && carry) {
+        if constexpr (CARRY) {
           const uint32_t q = s_pos[wave][o];
           pos2[i / 2]      = (i % 2 == 0) ? q : (pos2[i / 2] | (q << 16));
         }
@@ -345,7 +346,7 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
               s_words[wave][n][q]     = b[n];
               s_words[wave][n][q + 1] = a[n];
             }
-            if (CARRY && carry) {
+            if constexpr (CARRY) {
               const uint16_t t   = s_pos[wave][q];
               s_pos[wave][q]     = s_pos[wave][q + 1];
               s_pos[wave][q + 1] = t;
@@ -362,7 +363,7 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
           for (int n = 0; n < NW; ++n) {
             w[i][n] = s_words[wave][n][o];
           }
-          if (CARRY && carry) {
+          if constexpr (CARRY) {
             const uint32_t q = s_pos[wave][o];
             pos2[i / 2]      = (i % 2 == 0) ? q : (pos2[i / 2] | (q << 16));
           }
@@ -379,6 +380,83 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
 
   // ---- results ----
   if (keys_out != nullptr) {
+    if constexpr (FLOAT_KEYS_ONLY) {
+      if (!plain_floats) {
+        // The zeros of the row (either sign) and its NaNs (any payload) form one block each in the
+        // sorted row; a stable sort leaves them there in input order.  Where the blocks start
+        // follows from the sorted images.  The images go to LDS; the input is read once more and
+        // the bits of every zero and NaN replace the image at their place; then the row is
+        // written, decoded outside the two blocks.  All reads of the input come before the first
+        // store (keys_out may alias keys_in).  A rare path: plain loops keep its registers few.
+        constexpr KeyT SIGN = FloatLayout<KeyT>::sign;
+        constexpr KeyT INF  = FloatLayout<KeyT>::inf;
+        constexpr KeyT ONES = static_cast<KeyT>(~static_cast<KeyT>(0));
+        uint32_t zero_start = 0, zero_end = 0, nan_start = 0;
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+          const uint32_t o = i * WAVE + lane;
+          const bool valid = full || o < seg;
+          uint64_t image   = w[i][0];
+          if constexpr (NW > 1) {
+            image |= static_cast<uint64_t>(w[i][1]) << 32;
+          }
+          const KeyT img = static_cast<KeyT>(image);
+          zero_start += static_cast<uint32_t>(__builtin_popcountll(__builtin_amdgcn_ballot_w64(valid && img < SIGN)));
+          zero_end += static_cast<uint32_t>(__builtin_popcountll(__builtin_amdgcn_ballot_w64(valid && img <= SIGN)));
+          nan_start += static_cast<uint32_t>(__builtin_popcountll(__builtin_amdgcn_ballot_w64(valid && img != ONES)));
+          if (valid) {
+#pragma unroll
+            for (int n = 0; n < NW; ++n) {
+              s_words[wave][n][o] = w[i][n];
+            }
+          }
+        }
+        __builtin_amdgcn_wave_barrier();
+        auto put = [&](uint32_t slot, KeyT bits) {
+          s_words[wave][0][slot] = static_cast<uint32_t>(bits);
+          if constexpr (NW > 1) {
+            s_words[wave][1][slot] = static_cast<uint32_t>(static_cast<uint64_t>(bits) >> 32);
+          }
+        };
+        uint32_t zeros_seen = 0, nans_seen = 0;
+#pragma nounroll
+        for (int i = 0; i < ITEMS; ++i) {
+          const uint32_t o   = i * WAVE + lane;
+          const bool valid   = full || o < seg;
+          const KeyT raw     = valid ? keys_in[base + o] : KeyT{};
+          const KeyT mag     = static_cast<KeyT>(raw & static_cast<KeyT>(~SIGN));
+          const bool is_zero = valid && mag == 0;
+          const bool is_nan  = valid && mag > INF;
+          const uint64_t bz  = __builtin_amdgcn_ballot_w64(is_zero);
+          const uint64_t bn  = __builtin_amdgcn_ballot_w64(is_nan);
+          if (is_zero) {
+            put(zero_start + zeros_seen + lanes_below(bz), raw);
+          }
+          if (is_nan) {
+            put(nan_start + nans_seen + lanes_below(bn), raw);
+          }
+          zeros_seen += static_cast<uint32_t>(__builtin_popcountll(bz));
+          nans_seen += static_cast<uint32_t>(__builtin_popcountll(bn));
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+#pragma nounroll
+        for (int i = 0; i < ITEMS; ++i) {
+          const uint32_t o = i * WAVE + lane;
+          if (full || o < seg) {
+            uint64_t bits = s_words[wave][0][o];
+            if constexpr (NW > 1) {
+              bits |= static_cast<uint64_t>(s_words[wave][1][o]) << 32;
+            }
+            const bool in_block = (o >= zero_start && o < zero_end) || o >= nan_start;
+            const KeyT value    = static_cast<KeyT>(bits);
+            keys_out[base + o]  = in_block ? value : sign_unflip(value);
+          }
+        }
+        return;
+      }
+    }
     KeyT v[ITEMS];
 #pragma unroll
     for (int i = 0; i < ITEMS; ++i) {
@@ -386,8 +464,8 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
       if (full || o < seg) {
         if constexpr (OW::BIJECT) {
           v[i] = OW::decode(w[i]);
-        } else if (!carry) {
-          v[i] = OW::decode_plain_float(w[i]);
+        } else if constexpr (FLOAT_KEYS_ONLY) {
+          v[i] = OW::decode_plain_float(w[i]);  // zeros come out as +0.0, NaNs as some NaN: repaired below
         } else {
           v[i] = keys_in[base + ((pos2[i / 2] >> (16 * (i % 2))) & 0xFFFFu)];  // every gather of the row is issued before any store
         }
@@ -395,7 +473,7 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
         v[i] = KeyT{};
       }
     }
-    if (!OW::BIJECT && carry) {
+    if constexpr (CARRY && !OW::BIJECT) {
       // keys_out may alias keys_in: every gather of the row must have returned before the
       // first store overwrites it (the asm also keeps the compiler from moving either across)
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");

@@ -258,6 +258,41 @@ def test_short_rows_of_4_byte_keys_take_the_shortcut(lib, torch_cuda, dtype, seg
     check_rows(lib, torch_cuda, many, f"{np.dtype(dtype)} seg={seg} random rows")
 
 
+@pytest.mark.parametrize("dtype", [np.float16, np.float32, np.float64])
+@pytest.mark.parametrize("seg", [33, 64, 100, 257, 512, 1000, 1024])
+def test_short_float_rows_keys_only_with_zeros_and_nans(lib, torch_cuda, dtype, seg):
+    """Keys-only sorts of short float rows rebuild every key from its sorted image except zeros and NaNs,
+    whose bits (signs, payloads) are put back in input order from a second look at the input: rows of
+    only zeros of both signs, only NaNs of several payloads, mixtures, rows without either, sorted out
+    of place and in place."""
+    if np.dtype(dtype).itemsize == 8 and seg > 512:
+        pytest.skip("8-byte rows of this length take the workgroup kernel")
+    dt = np.dtype(dtype)
+    ub = {2: np.uint16, 4: np.uint32, 8: np.uint64}[dt.itemsize]
+    rng = np.random.default_rng(seg * dt.itemsize)
+    rows = 24
+    x = (rng.standard_normal((rows, seg)) * 4).astype(dtype)
+    bits = x.view(ub)
+    sign = ub(1) << ub(8 * dt.itemsize - 1)
+    nan_patterns = np.array([np.array(np.nan, dtype=dtype).view(ub), np.array(np.nan, dtype=dtype).view(ub) | sign,
+                             np.array(np.nan, dtype=dtype).view(ub) | ub(1), np.array(np.nan, dtype=dtype).view(ub) | ub(5) | sign], dtype=ub)
+    bits[0] = np.where(rng.random(seg) < 0.5, sign, ub(0))                         # zeros only
+    bits[1] = nan_patterns[rng.integers(0, 4, seg)]                                # NaNs only
+    for r in range(2, 12):                                                         # mixtures of growing density
+        m = rng.random(seg)
+        p = (r - 1) / 20
+        bits[r] = np.where(m < p, np.where(rng.random(seg) < 0.5, sign, ub(0)), bits[r])
+        bits[r] = np.where(m > 1 - p, nan_patterns[rng.integers(0, 4, seg)], bits[r])
+    bits[12, ::3] = sign                                                           # -0.0 only among ordinary keys
+    bits[13, 5] = nan_patterns[3]                                                  # a single NaN
+    x = bits.view(dtype)
+    want = oracle.local_sort(x, argsort=False)
+    v, _ = abi_sort(lib, torch_cuda, x, want_values=True)
+    assert_same_bits(v, want, f"{dt} seg={seg} keys only")
+    v, _ = abi_sort(lib, torch_cuda, x.copy(), want_values=True, in_place=True)
+    assert_same_bits(v, want, f"{dt} seg={seg} keys only, in place")
+
+
 # ---- global onesweep path ---------------------------------------------------------------------------
 GLOBAL_LENGTHS = [1, 2, 100, 4097, 8191, 8192, 8193, 16383, 16384, 16385, 3 * 16384 + 5, 100003]
 
