@@ -141,10 +141,11 @@ def algorithmic_bytes(cfg: dict, lds_limit_rows: bool, passes_run: int | None = 
 # GPU side
 # -------------------------------------------------------------------------------------------------
 def measure_device_rates(torch) -> dict:
-    """Streaming rates of the device on 1 GiB buffers with the framework's own kernels, outside the
-    timed region: a device-to-device copy (bytes read + written), a read-only reduction and a
-    write-only fill.  Reported beside the roofline so that the fraction of the published HBM peak
-    can be read against what a plain copy reaches on the same box."""
+    """Streaming rates of the device on 1 GiB buffers, outside the timed region: a device-to-device
+    copy (bytes read + written), a read-only sweep and a write-only fill, each once with the
+    library's own probe kernels (cpn_stream_probe: 128-bit nontemporal accesses, many short
+    workgroups) and once with torch's copy_/sum/zero_.  Reported beside the roofline so that the
+    fraction of the published HBM peak can be read against what plain passes reach on the same box."""
     n = 1 << 28
     src = torch.empty(n, dtype=torch.float32, device="cuda:0").normal_()
     dst = torch.empty_like(src)
@@ -164,10 +165,23 @@ def measure_device_rates(torch) -> dict:
         return best
 
     nbytes = 4 * n
+    from cupynumeric_amd import _lib
+
+    lib = _lib.load()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def probe(mode):
+        rc = lib.cpn_stream_probe(mode, src.data_ptr(), dst.data_ptr(), nbytes, stream)
+        if rc != 0:
+            raise RuntimeError(f"cpn_stream_probe: {_lib.status_string(rc)}")
+
     rates = {
-        "copy_GBps": 2 * nbytes / best_ms(lambda: dst.copy_(src)) / 1e6,
-        "read_GBps": nbytes / best_ms(lambda: src.sum()) / 1e6,
-        "fill_GBps": nbytes / best_ms(lambda: dst.zero_()) / 1e6,
+        "copy_GBps": 2 * nbytes / best_ms(lambda: probe(1)) / 1e6,
+        "read_GBps": nbytes / best_ms(lambda: probe(0)) / 1e6,
+        "fill_GBps": nbytes / best_ms(lambda: probe(2)) / 1e6,
+        "torch_copy_GBps": 2 * nbytes / best_ms(lambda: dst.copy_(src)) / 1e6,
+        "torch_sum_GBps": nbytes / best_ms(lambda: src.sum()) / 1e6,
+        "torch_zero_GBps": nbytes / best_ms(lambda: dst.zero_()) / 1e6,
         "buffer_bytes": nbytes,
     }
     del src, dst

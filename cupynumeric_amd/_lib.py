@@ -79,6 +79,7 @@ PROTOTYPES: dict[str, tuple] = {
     ),
     "cpn_profile_enable": (c_int, [c_int]),
     "cpn_profile_collect": (c_int, [c_void_p, c_uint64, c_void_p, c_int]),
+    "cpn_stream_probe": (c_int, [c_int, c_void_p, c_void_p, c_uint64, c_void_p]),
     "cpn_swapaxes_copy": (c_int, [c_int, c_void_p, c_void_p, ctypes.POINTER(c_int64), c_int, c_int, c_int, c_void_p]),
 }
 

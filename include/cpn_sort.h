@@ -280,6 +280,20 @@ int cpn_lexsort_pack(int num_keys, const int* dtypes, const void* const* keys, c
 int cpn_profile_enable(int on);
 int cpn_profile_collect(char* labels, uint64_t label_stride, float* milliseconds, int max_records);
 
+/*
+ * Streaming-rate probe: one plain pass over `bytes` bytes (a multiple of 16, both pointers
+ * 16-byte aligned) on `stream`, for benchmarks that want the device's own ceilings beside a
+ * sort's rate.  mode CPN_STREAM_READ reads src (dst receives nothing unless the data holds one
+ * improbable pattern, which keeps the loads alive), CPN_STREAM_COPY copies src to dst,
+ * CPN_STREAM_FILL writes a constant to dst.  Loads and stores carry the nontemporal hint.
+ * Returns 0 or a negative status.  No counterpart in the reference (its benchmarks time
+ * whole API calls, examples/_benchmark/timer.py:199-241).
+ */
+#define CPN_STREAM_READ 0
+#define CPN_STREAM_COPY 1
+#define CPN_STREAM_FILL 2
+int cpn_stream_probe(int mode, const void* src, void* dst, uint64_t bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

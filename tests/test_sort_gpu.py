@@ -847,3 +847,37 @@ def test_rows_of_at_most_256_different_keys(lib, torch_cuda, virtual_digits_from
     x = np.sort(pool[rng.integers(0, 1000, n)])
     _, i = abi_sort(lib, torch_cuda, x, want_values=False, want_indices=True)
     assert_same_bits(i, oracle.local_sort(x, argsort=True, threads=8), f"{dt} sorted runs")
+
+
+# ---- the streaming-rate probe of the benchmark ------------------------------------------------------
+@pytest.mark.parametrize("nbytes", [0, 16, 4096 + 16, (1 << 22) + 48, 3 * (1 << 24)])
+def test_stream_probe_copies_fills_and_leaves_the_source_alone(nbytes):
+    """cpn_stream_probe: the copy moves every byte (sizes below, at and above one grid of 512-thread
+    workgroups, and above the grid cap so that threads loop), the fill writes its constant, the read
+    pass changes nothing, and bad arguments come back as status codes."""
+    import torch
+
+    lib = _lib.load()
+    dev = torch.device("cuda")
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    g = torch.Generator(device="cpu").manual_seed(nbytes)
+    host = torch.randint(0, 256, (max(nbytes, 16),), dtype=torch.uint8, generator=g)
+    src = host.to(dev)
+    dst = torch.full((max(nbytes, 16) + 32,), 0xEE, dtype=torch.uint8, device=dev)  # 32 guard bytes
+    assert lib.cpn_stream_probe(1, src.data_ptr(), dst.data_ptr(), nbytes, stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(dst[:nbytes].cpu(), host[:nbytes])
+    assert bool((dst[nbytes:] == 0xEE).all()), "the copy wrote past its size"
+    assert lib.cpn_stream_probe(0, src.data_ptr(), dst.data_ptr(), nbytes, stream) == 0
+    assert lib.cpn_stream_probe(0, src.data_ptr(), None, nbytes, stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(src.cpu(), host) and torch.equal(dst[:nbytes].cpu(), host[:nbytes])
+    assert lib.cpn_stream_probe(2, None, dst.data_ptr(), nbytes, stream) == 0
+    torch.cuda.synchronize()
+    assert bool((dst[:nbytes] == 1).all()) and bool((dst[nbytes:] == 0xEE).all())
+    # error paths: nothing is launched
+    assert lib.cpn_stream_probe(3, src.data_ptr(), dst.data_ptr(), 16, stream) == -3
+    assert lib.cpn_stream_probe(1, src.data_ptr(), dst.data_ptr(), 8, stream) == -3
+    assert lib.cpn_stream_probe(1, None, dst.data_ptr(), 16, stream) == -2
+    assert lib.cpn_stream_probe(2, None, None, 16, stream) == -2
+    assert lib.cpn_stream_probe(1, src.data_ptr() + 4, dst.data_ptr(), 16, stream) == -5
