@@ -34,15 +34,17 @@ constexpr uint64_t WORKSPACE_ALIGN  = 256;
 // Workspace header: [0] status word, [128..) tile tickets, [256..) per-pass "digit varies" flags,
 // [384..) the device-side SortPlan.  The status word has a 128-byte line to itself: every tile
 // reads it with an ordinary load, and the tickets next door are under constant atomic traffic.
-constexpr uint64_t HEADER_BYTES     = 1024;
+constexpr uint64_t HEADER_BYTES     = 2048;
 constexpr uint64_t HEADER_TICKETS   = 128;
 constexpr uint64_t HEADER_SCAN_DONE = 240;  // blocks of the scan kernel that have finished
 constexpr uint64_t HEADER_SPECIALS  = 244;  // float keys: the sort holds a NaN or a -0.0
 constexpr uint64_t HEADER_VARYING   = 256;
 constexpr uint64_t HEADER_PLAN      = 384;
+constexpr uint64_t HEADER_XCD_TICKETS = 1024;  // per pass: one tile counter per XCD (onesweep.h, claim_tile)
 static_assert(HEADER_TICKETS + 4 * MAX_PASSES <= HEADER_SCAN_DONE, "tickets overlap the scan counter");
 static_assert(HEADER_VARYING + 4 * MAX_PASSES <= HEADER_PLAN, "flags overlap the plan");
-static_assert(HEADER_PLAN + sizeof(SortPlan) <= HEADER_BYTES, "plan does not fit the header");
+static_assert(HEADER_PLAN + sizeof(SortPlan) <= HEADER_XCD_TICKETS, "plan overlaps the per-XCD tile counters");
+static_assert(HEADER_XCD_TICKETS + 4 * XCD_COUNT * MAX_PASSES <= HEADER_BYTES, "tile counters do not fit the header");
 constexpr uint64_t BIG_ROW_ELEMENTS = 1ull << 30;
 // Shortest row for which virtual digits are considered: their extra launches (three small kernels
 // and an early-exiting twin of every pass) cost about 0.1 ms, 2 % of a 2^26-key sort of 8-byte keys.
@@ -508,6 +510,7 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
     a.idx_buf[IDX_ALIAS] = r.indices_out;
     a.plan               = plan;
     a.ticket             = tickets + p;
+    a.xcd_tickets        = reinterpret_cast<uint32_t*>(ws + HEADER_XCD_TICKETS) + p * XCD_COUNT;
     a.hist_excl          = hist + p * RADIX;
     a.desc               = reinterpret_cast<OffT*>(ws + L.off_desc + L.desc_bytes_per_pass * p);
     a.status             = status;

@@ -88,7 +88,7 @@ def test_temp_bytes_layout(lib):
     assert tb(99, 100, 100, 1, 0, 0) == 0
     assert tb(f32, 100, 7, 1, 0, 0) == 0  # 7 does not divide 100
     header = tb(f32, 0, 0, 1, 0, 0)
-    assert header == 1024
+    assert header == 2048
     assert tb(f32, 1 << 20, 1024, 1, 1, 0) == header  # rows that fit LDS need only the header
     n = 1 << 24
     tiles = n // 16384  # 512 threads x 32 keys per tile for keys of up to 4 bytes
