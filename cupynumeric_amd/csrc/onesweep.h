@@ -444,7 +444,11 @@ struct SweepArgs {
 // the next XCD's groups, so every tile is taken exactly once whatever the dispatcher does, and
 // the tiles below any taken tile of an XCD's own sequence are always taken too: a tile that a
 // look-back waits for is either held by a resident workgroup or next in line on an XCD whose
-// resident workgroups hold lower tiles only, which finish without it.
+// resident workgroups hold lower tiles only, which finish without it.  What the order does
+// assume is that every XCD keeps receiving workgroups of this launch: if other work kept one XCD
+// fully occupied for seconds, tiles elsewhere would wait for that XCD's share until the bounded
+// look-back gave up and the call reported CPN_ERR_DEVICE (a single counter for all XCDs has no
+// such dependence, at the price of the split lines).
 constexpr uint32_t XCD_COUNT = 8;
 #ifndef CPN_TILE_GROUP
 #define CPN_TILE_GROUP 8
