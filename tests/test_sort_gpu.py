@@ -690,6 +690,37 @@ def test_concurrent_streams_and_threads(lib, torch_cuda):
     assert not errors, errors
 
 
+def test_global_sorts_overlapping_on_three_streams(lib, torch_cuda):
+    """Global sorts of several hundred tiles each, enqueued on three streams without a host wait in
+    between, so that their scatter passes compete for the workgroup slots of every XCD while each
+    deals its tiles per XCD: every call must finish without the look-back giving up and match the
+    oracle."""
+    torch = torch_cuda
+    dev = torch.device("cuda")
+    jobs = []
+    streams = [torch.cuda.Stream() for _ in range(3)]
+    torch.cuda.synchronize()
+    for rnd in range(3):
+        for k, stream in enumerate(streams):
+            dtype = [np.float32, np.int32, np.int64][(k + rnd) % 3]
+            n = (1 << 22) + 12345 * (k + 1) + rnd
+            x = make_input(dtype, (n,), seed=900 + 10 * rnd + k)
+            code = _lib.DTYPE_CODES[np.dtype(dtype)]
+            d_in = torch.from_numpy(x.view(np.uint8).copy()).to(dev)
+            d_idx = torch.empty(n, dtype=torch.int64, device=dev)
+            tb = lib.cpn_local_sort_temp_bytes(code, n, n, 0, 1, 0)
+            temp = torch.full((tb,), 0xFF, dtype=torch.uint8, device=dev)
+            jobs.append((x, d_in, d_idx, temp, tb, code, n, stream))
+    torch.cuda.synchronize()
+    for x, d_in, d_idx, temp, tb, code, n, stream in jobs:  # all enqueued before anything is waited for
+        h = ctypes.c_void_p(stream.cuda_stream)
+        assert lib.cpn_local_sort(code, d_in.data_ptr(), None, d_idx.data_ptr(), n, n, 0, 1, temp.data_ptr(), tb, h) == 0
+    for x, d_in, d_idx, temp, tb, code, n, stream in jobs:
+        h = ctypes.c_void_p(stream.cuda_stream)
+        assert lib.cpn_local_sort_check(temp.data_ptr(), h) == 0, f"{x.dtype} n={n}: device status"
+        assert np.array_equal(d_idx.cpu().numpy(), oracle.local_sort(x, argsort=True, threads=8)), f"{x.dtype} n={n}"
+
+
 # ---- failure path of the bounded look-back wait -------------------------------------------------------
 def test_lookback_gives_up_cleanly(lib, torch_cuda):
     """With the spin limit forced to one poll, a tile whose predecessor has not answered yet gives up:
