@@ -41,7 +41,7 @@ MEASURED_TRAFFIC_BYTES = {
     ("c1", 1 << 24): 1.44e8,    # onesweep, profiles/onesweep_c1_traffic.txt
     ("c2", 1 << 28): 4.303e9,   # onesweep, profiles/onesweep_c2_traffic.txt
     ("c3", 1 << 26): 1.074e9,   # lds_row_sort, profiles/lds_row_sort_c3_traffic.txt
-    ("c4", 1 << 27): 2.277e9,   # onesweep (the one pass on the ranks of the 16 different keys), profiles/onesweep_c4_traffic.txt
+    ("c4", 1 << 27): 2.211e9,   # onesweep (the one pass on the ranks of the 16 different keys), profiles/onesweep_c4_traffic.txt
     ("c5", 1 << 26): 2.69e8,    # lds_row_sort, profiles/lds_row_sort_c5_traffic.txt
 }
 
