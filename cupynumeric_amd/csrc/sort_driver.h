@@ -69,8 +69,9 @@ __host__ __device__ constexpr uint64_t align_up(uint64_t v, uint64_t a) { return
 // 16 384 keys like the tiles of 4-byte keys and a digit's run 64 keys on average.  Measured on 2^27
 // keys against 512 threads (8192-key tiles, two workgroups per CU): float64 sort 5.24 -> 5.02 ms,
 // argsort 6.51 -> 6.16, int64 sort 5.04 -> 4.67; the one pass of a row of 16 different int64 keys
-// 0.66 -> 0.71 ms.  4-byte keys: 512 threads x 32 keys (1024 threads: 3.94 -> 4.33 ms at 2^28).
-__host__ __device__ constexpr int global_block(int key_bytes) { return key_bytes == 8 ? 1024 : CPN_GLOBAL_BLOCK; }
+// 0.66 -> 0.71 ms.  16-byte keys likewise (1024 x 8 keys: 2^25 complex128 keys 4.91 -> 4.69 ms).
+// 4-byte keys: 512 threads x 32 keys (1024 threads: 3.94 -> 4.33 ms at 2^28).
+__host__ __device__ constexpr int global_block(int key_bytes) { return key_bytes >= 8 ? 1024 : CPN_GLOBAL_BLOCK; }
 // (64-bit keys or 64-bit row positions halve the items per thread: the LDS staging area stays at
 // 64 KiB for 512 threads, two workgroups per CU, and is 128 KiB for the 1024 threads of 8-byte keys)
 __host__ __device__ constexpr int global_items(int key_bytes, bool big)

@@ -108,7 +108,7 @@ def test_temp_bytes_layout(lib):
     # complex keys take one more pass (the NaN class) than their bytes
     c64, c128 = 12, 13
     assert tb(c64, n, n, 1, 0, 0) == header + 9 * 256 * 4 + 9 * (n // 16384) * 256 * 4 + 8 * n  # 8-byte keys: 1024 x 16
-    assert tb(c128, n, n, 1, 0, 0) == header + align256(17 * 256 * 4) + 17 * (n // 4096) * 256 * 4 + 16 * n
+    assert tb(c128, n, n, 1, 0, 0) == header + align256(17 * 256 * 4) + 17 * (n // 8192) * 256 * 4 + 16 * n
     # the row-length switch moves work to the global path
     prev = lib.cpn_set_lds_row_limit(0)
     try:

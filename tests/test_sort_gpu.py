@@ -350,7 +350,7 @@ def wide_rows(lib):
 
 @pytest.mark.parametrize("dtype", ALL_DTYPES)
 def test_global_path_wide_rows(lib, torch_cuda, wide_rows, dtype):
-    """The 64-bit variant of the global path: tiles are 8192 keys of 4 bytes or less, 16 384 keys of 8 bytes and 4096 of 16 bytes there."""
+    """The 64-bit variant of the global path: tiles are 8192 keys of 4 bytes or less, 16 384 keys of 8 bytes and 8192 of 16 bytes there."""
     for shape in [(5000,), (8192,), (8193,), (3, 20011), (100003,), (2, 4 * 8192)]:
         x = make_input(dtype, shape, seed=shape[-1])
         check_rows(lib, torch_cuda, x, f"{np.dtype(dtype)} {shape} (wide rows)")
