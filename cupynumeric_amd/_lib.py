@@ -43,6 +43,10 @@ CPN_ERR_ALIGN = -5
 CPN_ERR_HIP = -6
 CPN_ERR_DEVICE = -7
 CPN_ERR_UNSUPPORTED = -8
+CPN_ERR_SCRATCH = -9
+
+# include/cpn_sort.h: workspace of cpn_local_sort_static
+STATIC_SCRATCH_BYTES = 64 << 20
 
 # name -> (restype, argtypes); every symbol include/cpn_sort.h declares
 PROTOTYPES: dict[str, tuple] = {
@@ -60,6 +64,9 @@ PROTOTYPES: dict[str, tuple] = {
     "cpn_local_sort": (
         c_int,
         [c_int, c_void_p, c_void_p, c_void_p, c_uint64, c_uint64, c_int64, c_int, c_void_p, c_uint64, c_void_p],
+    ),
+    "cpn_local_sort_static": (
+        c_int, [c_int, c_void_p, c_void_p, c_void_p, c_uint64, c_uint64, c_int64, c_int, c_void_p, c_void_p]
     ),
     "cpn_local_sort_check": (c_int, [c_void_p, c_void_p]),
     "cpn_real_to_complex": (c_int, [c_int, c_void_p, c_int, c_void_p, c_uint64, c_void_p]),

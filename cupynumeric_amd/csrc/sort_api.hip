@@ -7,8 +7,15 @@
 #include <stdlib.h>
 
 #include <atomic>
+#include <mutex>
 
 #include "sort_driver.h"
+
+// Device memory for cpn_local_sort_static: the workspace of a sort that may not allocate.  One
+// copy of the array exists on every GPU that loads this library, for the life of the process.
+// In host code the name below is only a handle for hipGetSymbolAddress; kernels and HIP calls
+// receive the per-device address kept in g_static_scratch.
+static __device__ __align__(256) unsigned char scratch[CPN_STATIC_SCRATCH_BYTES];
 
 namespace cpn {
 
@@ -68,6 +75,40 @@ uint64_t lds_row_limit(int key_bytes)
   return cap;
 }
 
+// Address of `scratch` on every device seen so far (looked up once per device, with that device
+// current).
+constexpr int MAX_DEVICES = 64;
+static void* g_static_scratch[MAX_DEVICES];
+static std::mutex g_static_scratch_mutex;
+
+static int static_scratch_of_current_device(void** out)
+{
+  int dev = -1;
+  CPN_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= MAX_DEVICES) {
+    return CPN_ERR_UNSUPPORTED;
+  }
+  std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+  if (g_static_scratch[dev] == nullptr) {
+    void* ptr = nullptr;
+    CPN_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (ptr == nullptr || (reinterpret_cast<uintptr_t>(ptr) % WORKSPACE_ALIGN) != 0) {
+      return CPN_ERR_TEMP;
+    }
+    g_static_scratch[dev] = ptr;
+  }
+  *out = g_static_scratch[dev];
+  return CPN_OK;
+}
+
+// one thread: hands the status word of a finished sort to the caller's device memory
+static __global__ void copy_status_kernel(const uint32_t* __restrict__ status, uint32_t* __restrict__ out)
+{
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    *out = *status;
+  }
+}
+
 }  // namespace cpn
 
 extern "C" {
@@ -86,6 +127,7 @@ const char* cpn_status_string(int status)
     case CPN_ERR_HIP: return "HIP runtime call failed";
     case CPN_ERR_DEVICE: return "kernel reported an internal failure";
     case CPN_ERR_UNSUPPORTED: return "request not implemented by this build";
+    case CPN_ERR_SCRATCH: return "request needs more workspace than the static scratch holds";
     default: return "unknown status";
   }
 }
@@ -203,6 +245,39 @@ int cpn_local_sort(int dtype, const void* values_in, void* values_out, int64_t* 
     case 16: return cpn::sort_keys128(k.codec, r);
     default: return CPN_ERR_UNSUPPORTED;
   }
+}
+
+int cpn_local_sort_static(int dtype, const void* values_in, void* values_out, int64_t* indices_out, uint64_t volume,
+                          uint64_t sort_dim_size, int64_t index_offset, int stable, uint32_t* status_out, void* stream)
+{
+  if ((reinterpret_cast<uintptr_t>(status_out) & 3u) != 0) {
+    return CPN_ERR_ALIGN;
+  }
+  const cpn::KeyKind k = cpn::key_kind(dtype);
+  if (k.bytes != 0 && k.codec >= 0 && volume != 0 && sort_dim_size != 0 && volume % sort_dim_size == 0) {
+    // a well-formed request: does its workspace fit?  (everything else gets cpn_local_sort's own answer)
+    const uint64_t need = cpn_local_sort_temp_bytes(dtype, volume, sort_dim_size, values_out != nullptr,
+                                                    indices_out != nullptr, values_out == values_in);
+    if (need > CPN_STATIC_SCRATCH_BYTES) {
+      return CPN_ERR_SCRATCH;
+    }
+  }
+  void* ws = nullptr;
+  if (volume != 0) {
+    const int rc = cpn::static_scratch_of_current_device(&ws);
+    if (rc != CPN_OK) {
+      return rc;
+    }
+  }
+  const int rc = cpn_local_sort(dtype, values_in, values_out, indices_out, volume, sort_dim_size, index_offset, stable,
+                                ws, CPN_STATIC_SCRATCH_BYTES, stream);
+  if (rc != CPN_OK || status_out == nullptr || volume == 0) {
+    return rc;
+  }
+  hipLaunchKernelGGL(cpn::copy_status_kernel, dim3(1), dim3(cpn::WAVE), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint32_t*>(ws), status_out);
+  CPN_HIP_TRY(hipGetLastError());
+  return CPN_OK;
 }
 
 int cpn_local_sort_check(const void* temp, void* stream)

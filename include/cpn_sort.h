@@ -56,7 +56,9 @@ typedef enum cpn_status {
   CPN_ERR_ALIGN       = -5, /* a data pointer is not aligned to its element size       */
   CPN_ERR_HIP         = -6, /* a HIP runtime call failed (see cpn_last_hip_error)      */
   CPN_ERR_DEVICE      = -7, /* a kernel flagged an internal failure (bounded wait hit) */
-  CPN_ERR_UNSUPPORTED = -8  /* valid request that this build does not implement        */
+  CPN_ERR_UNSUPPORTED = -8, /* valid request that this build does not implement        */
+  CPN_ERR_SCRATCH     = -9  /* cpn_local_sort_static: the request needs more workspace
+                               than CPN_STATIC_SCRATCH_BYTES                            */
 } cpn_status;
 
 /* Library version, (major << 16) | minor. */
@@ -167,6 +169,33 @@ uint64_t cpn_local_sort_temp_bytes(int dtype, uint64_t volume, uint64_t sort_dim
 int cpn_local_sort(int dtype, const void* values_in, void* values_out, int64_t* indices_out,
                    uint64_t volume, uint64_t sort_dim_size, int64_t index_offset, int stable,
                    void* temp, uint64_t temp_bytes, void* stream);
+
+/*
+ * cpn_local_sort for callers that cannot allocate device memory or pass a workspace: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference, whose sort always draws its temporaries from a Legate pool
+ * (src/cupynumeric/sort/cub_sort.cuh:48,62-63).
+ *
+ * Same arguments, results and ordering as cpn_local_sort, without `temp`: the workspace is a
+ * static array of CPN_STATIC_SCRATCH_BYTES bytes of device memory inside the library, one copy
+ * per GPU, held until the process ends.  The call allocates and frees nothing (no hipMalloc,
+ * hipFree or allocating library routine) and launches the same kernels as cpn_local_sort.
+ *
+ *   - a request whose cpn_local_sort_temp_bytes exceeds CPN_STATIC_SCRATCH_BYTES returns
+ *     CPN_ERR_SCRATCH and launches nothing (row sorts that fit the per-row kernels need 2 KiB
+ *     whatever their volume; a 1-D argsort of 4-byte keys fits up to about 5.4 million keys);
+ *   - status_out (device memory, 4-byte aligned, may be NULL) receives the sort's device status
+ *     word when the sort has finished: 0, or non-zero when a bounded wait inside a kernel ran out
+ *     and the output is invalid (what cpn_local_sort_check reports for cpn_local_sort);
+ *   - every call on one GPU uses that GPU's one array, whatever its stream: calls that overlap in
+ *     time on one GPU race.  Order them on one stream, or with events;
+ *   - the first call on a device looks up the array's address on that device
+ *     (hipGetSymbolAddress); make that call outside graph capture.
+ */
+#define CPN_STATIC_SCRATCH_BYTES (64ull << 20)
+int cpn_local_sort_static(int dtype, const void* values_in, void* values_out, int64_t* indices_out,
+                          uint64_t volume, uint64_t sort_dim_size, int64_t index_offset, int stable,
+                          uint32_t* status_out, void* stream);
 
 /*
  * Blocks until `stream` has finished, then reports what the kernels of the last

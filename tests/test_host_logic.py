@@ -43,7 +43,7 @@ def test_dtype_codes_match_header():
 def test_version_status_strings_and_sizes(lib):
     assert lib.cpn_sort_version() >= 1
     assert lib.cpn_status_string(0) == b"ok"
-    for status in range(-8, 0):
+    for status in range(-9, 0):
         assert lib.cpn_status_string(status) not in (b"ok", b"unknown status")
     assert lib.cpn_status_string(-99) == b"unknown status"
     for dt, code in _lib.DTYPE_CODES.items():

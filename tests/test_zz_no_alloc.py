@@ -1,0 +1,111 @@
+"""cpn_local_sort_static (the entry point that allocates nothing: its workspace is a static device
+array inside the library) against cpn_local_sort on the same inputs, through the C ABI.  Results
+must be bit-identical.  Collected last on purpose: a failure here must not hide other tests."""
+from __future__ import annotations
+
+import ctypes
+
+import numpy as np
+import pytest
+from conftest import make_input
+
+from cupynumeric_amd import _lib
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return _lib.load()
+
+
+@pytest.fixture(scope="module")
+def torch_cuda():
+    import torch
+
+    assert torch.cuda.is_available(), "these tests need a HIP device"
+    return torch
+
+
+def run_both(lib, torch, x: np.ndarray, want_values: bool, want_indices: bool, in_place: bool = False, offset: int = 0):
+    """Sorts x with cpn_local_sort (caller's workspace) and with cpn_local_sort_static; every
+    buffer the static call touches is allocated before it is made."""
+    dev = torch.device("cuda")
+    seg, volume = x.shape[-1], x.size
+    code = _lib.DTYPE_CODES[x.dtype]
+    raw = np.ascontiguousarray(x).reshape(-1).view(np.uint8)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def buffers():
+        d_in = torch.from_numpy(raw.copy()).to(dev)
+        d_val = d_in if in_place else (torch.full_like(d_in, 0x5A) if want_values else None)
+        d_idx = torch.full((volume,), -7, dtype=torch.int64, device=dev) if want_indices else None
+        return d_in, d_val, d_idx
+
+    tb = lib.cpn_local_sort_temp_bytes(code, volume, seg, int(want_values), int(want_indices), int(in_place))
+    assert 0 < tb <= _lib.STATIC_SCRATCH_BYTES
+    a_in, a_val, a_idx = buffers()
+    temp = torch.full((tb,), 0xFF, dtype=torch.uint8, device=dev)
+    rc = lib.cpn_local_sort(code, a_in.data_ptr(), a_val.data_ptr() if want_values else None,
+                            a_idx.data_ptr() if want_indices else None, volume, seg, offset, 1,
+                            temp.data_ptr(), tb, stream)
+    assert rc == 0, _lib.status_string(rc)
+    assert lib.cpn_local_sort_check(temp.data_ptr(), stream) == 0
+
+    b_in, b_val, b_idx = buffers()
+    status = torch.full((1,), 77, dtype=torch.int32, device=dev)
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_stats()["allocation.all.allocated"]
+    rc = lib.cpn_local_sort_static(code, b_in.data_ptr(), b_val.data_ptr() if want_values else None,
+                                   b_idx.data_ptr() if want_indices else None, volume, seg, offset, 1,
+                                   status.data_ptr(), stream)
+    assert rc == 0, _lib.status_string(rc)
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
+    assert int(status.item()) == 0
+    if want_values:
+        assert torch.equal(a_val, b_val), "values differ"
+    if want_indices:
+        assert torch.equal(a_idx, b_idx), "indices differ"
+    if not in_place:
+        assert np.array_equal(b_in.cpu().numpy(), raw), "input was modified"
+
+
+def test_static_scratch_matches_workspace_sort(lib, torch_cuda):
+    # two calls in a row on the same device array, the second one smaller: what the first left in
+    # the scratch (tile counters, descriptors, histograms, plan) must not reach the second
+    big = make_input(np.float32, (1 << 21,), seed=11)
+    small = make_input(np.float32, (300_001,), seed=12)
+    run_both(lib, torch_cuda, big, want_values=False, want_indices=True)
+    run_both(lib, torch_cuda, small, want_values=False, want_indices=True)
+    # values + indices, in place, other key widths, batched long rows, the per-row kernels
+    run_both(lib, torch_cuda, make_input(np.int64, (1 << 20,), seed=13), True, True)
+    run_both(lib, torch_cuda, make_input(np.int32, (70_000,), seed=14), True, False, in_place=True)
+    run_both(lib, torch_cuda, make_input(np.float64, (3, 40_000), seed=15), True, True, offset=5)
+    run_both(lib, torch_cuda, make_input(np.uint16, (12, 20_000), seed=16), False, True)
+    run_both(lib, torch_cuda, make_input(np.float16, (257, 1000), seed=17), True, False)
+    run_both(lib, torch_cuda, make_input(np.int8, (1000, 31), seed=18), True, True)
+    run_both(lib, torch_cuda, make_input(np.complex64, (100_000,), seed=19), True, True)
+    run_both(lib, torch_cuda, small, want_values=True, want_indices=False)
+
+
+def test_static_scratch_rejects_what_does_not_fit(lib, torch_cuda):
+    torch = torch_cuda
+    n = 1 << 25  # a float32 argsort of 2^25 keys needs about 400 MiB of workspace
+    code = _lib.DTYPE_CODES[np.dtype(np.float32)]
+    assert lib.cpn_local_sort_temp_bytes(code, n, n, 0, 1, 0) > _lib.STATIC_SCRATCH_BYTES
+    d_in = torch.zeros(n, dtype=torch.float32, device="cuda")
+    d_idx = torch.full((n,), -7, dtype=torch.int64, device="cuda")
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rc = lib.cpn_local_sort_static(code, d_in.data_ptr(), None, d_idx.data_ptr(), n, n, 0, 1, None, stream)
+    assert rc == _lib.CPN_ERR_SCRATCH
+    assert b"static scratch" in lib.cpn_status_string(rc)
+    torch.cuda.synchronize()
+    assert bool((d_idx == -7).all()), "a rejected request must not write"
+    # argument errors are reported like cpn_local_sort's
+    assert lib.cpn_local_sort_static(99, d_in.data_ptr(), None, d_idx.data_ptr(), 8, 8, 0, 1, None, stream) == _lib.CPN_ERR_DTYPE
+    assert lib.cpn_local_sort_static(code, d_in.data_ptr(), None, d_idx.data_ptr(), 10, 3, 0, 1, None, stream) == _lib.CPN_ERR_SHAPE
+    assert lib.cpn_local_sort_static(code, None, None, None, 0, 0, 0, 1, None, stream) == _lib.CPN_OK
+    # rows that fit the per-row kernels need 2 KiB of workspace whatever the volume
+    rows = make_input(np.float32, (4096, 2048), seed=20)
+    run_both(lib, torch, rows, want_values=True, want_indices=False)
