@@ -34,8 +34,18 @@
 
 namespace cpn {
 
+// Waves per SIMD the compiler has to leave room for.  1024 threads with 8 keys of up to 4 bytes each stay below 64
+// vector registers and 80 KiB of LDS so that two workgroups share a CU; that also takes at most
+// 100 scalar registers per wave, which the compiler exceeds unless it is told (it then keeps a
+// few uniform values in vector registers instead).
+__host__ __device__ constexpr int lds_row_waves_per_simd(int block, int items, int key_bytes)
+{
+  return (block == 1024 && items <= 8 && key_bytes <= 4) ? 8 : 1;
+}
+
 template <typename KeyT, int CODEC, bool HAS_IDX, int BLOCK, int ITEMS>
-__global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in,
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(lds_row_waves_per_simd(BLOCK, ITEMS, sizeof(KeyT)))))
+void lds_row_sort_kernel(const KeyT* keys_in,
                                                               KeyT* keys_out,
                                                               int64_t* idx_out,
                                                               uint32_t seg,
@@ -69,8 +79,17 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
   const int lane      = tid & (WAVE - 1);
   const int wave      = tid / WAVE;
   const uint64_t base = static_cast<uint64_t>(blockIdx.x) * seg;
-  const uint32_t woff = wave * WTILE + lane;
   const bool full     = (seg == TILE);
+  // A row shorter than the tile is dealt in equal contiguous shares of whole 64-key rounds, so that
+  // every wave works on `rounds` keys per lane and the cost follows the row length, not the tile.
+  // (Only the 1024-thread shapes, which take the longest rows and a wide range of lengths: in the
+  // smaller ones the extra uniform branches cost full rows 3-10 % and the shapes are a factor of two apart.)
+  constexpr bool BALANCE = (BLOCK == 1024);
+  const uint32_t rounds  = (!BALANCE || full) ? ITEMS : (seg + BLOCK - 1) / BLOCK;
+  const uint32_t woff    = wave * ((!BALANCE || full) ? WTILE : rounds * WAVE) + lane;
+  auto holds = [&](int i) -> bool {
+    return full || ((!BALANCE || i < static_cast<int>(rounds)) && woff + i * WAVE < seg);
+  };
 
   KeyT key[ITEMS];
   uint32_t idx[HAS_IDX ? ITEMS : 1];
@@ -84,7 +103,7 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t o = woff + i * WAVE;
-    if (full || o < seg) {
+    if (holds(i)) {
       key[i] = keys_in[base + o];
       uint64_t w[NW];
       KT::words(key[i], w);
@@ -199,7 +218,12 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
     uint32_t dpk[(ITEMS + 3) / 4];  // the digits, four per register
 #pragma unroll
     for (int i = 0; i < ITEMS; ++i) {
-      const bool valid = full || (woff + i * WAVE < seg);
+      if constexpr (BALANCE) {
+        if (!full && i >= static_cast<int>(rounds)) {
+          break;  // uniform: no wave holds a key in this round
+        }
+      }
+      const bool valid = holds(i);
       const uint32_t d = digit_of(key[i], pass);
       dpk[i / 4]       = (i % 4 == 0) ? d : (dpk[i / 4] | (d << (8 * (i % 4))));
       if (!HAS_IDX && free_first && first_running) {  // uniform
@@ -247,7 +271,7 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < ITEMS; ++i) {
-      if (full || (woff + i * WAVE < seg)) {
+      if (holds(i)) {
         const uint32_t d   = (dpk[i / 4] >> (8 * (i % 4))) & 0xFFu;
         const uint32_t pos = base[d] + rnk[i];
         s_keys[pos]        = key[i];
@@ -260,7 +284,7 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
 #pragma unroll
     for (int i = 0; i < ITEMS; ++i) {
       const uint32_t o = woff + i * WAVE;
-      if (full || o < seg) {
+      if (holds(i)) {
         key[i] = s_keys[o];
         if constexpr (HAS_IDX) {
           idx[i] = s_idx[o];
@@ -294,7 +318,7 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
 #pragma unroll
       for (int i = 0; i < ITEMS; ++i) {
         const uint32_t o = woff + i * WAVE;
-        if (o + 1 < seg) {
+        if (holds(i) && o + 1 < seg) {
           bad |= misordered(key[i], s_keys[o + 1]) ? 1 : 0;
         }
       }
@@ -323,7 +347,7 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
 #pragma unroll
       for (int i = 0; i < ITEMS; ++i) {
         const uint32_t o = woff + i * WAVE;
-        if (full || o < seg) {
+        if (holds(i)) {
           key[i] = s_keys[o];
           if constexpr (HAS_IDX) {
             idx[i] = s_idx[o];
@@ -349,7 +373,7 @@ __global__ __launch_bounds__(BLOCK) void lds_row_sort_kernel(const KeyT* keys_in
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t o = woff + i * WAVE;
-    if (full || o < seg) {
+    if (holds(i)) {
       if (keys_out != nullptr) {
         keys_out[base + o] = key[i];
       }

@@ -299,65 +299,83 @@ static __global__ void plan_kernel(const uint32_t* __restrict__ varying, SortPla
   }
 }
 
-// One block per (row, pass): exclusive scan of 256 counts in place.  A pass on whose digit
-// all keys of a row agree (one bin holds the whole row) would be the identity permutation for
-// that row; `varying[pass]` is raised by every row for which that is not so.
+// Exclusive scan of every 256-bin histogram in place, one wavefront per (row, pass) histogram
+// (four bins per lane), the wavefronts of the grid striding over the histograms: a request of
+// many short rows has as many histograms as rows x passes, and one workgroup each, with one
+// device-scope atomic each for the plan, took longer than the scatter passes.  A pass on whose
+// digit all keys of a row agree (one bin holds the whole row) would be the identity permutation
+// for that row; `varying[pass]` is raised by every row for which that is not so.
+constexpr int SCAN_BLOCK = 256;
 template <typename OffT>
-__global__ __launch_bounds__(RADIX) void histogram_scan_kernel(OffT* __restrict__ hist,
-                                                               uint32_t* __restrict__ varying,
-                                                               uint64_t seg,
-                                                               uint32_t passes,
-                                                               const VirtPlan* __restrict__ vplan,
-                                                               uint32_t second,
-                                                               uint32_t* __restrict__ blocks_done,
-                                                               SortPlan* __restrict__ plan,
-                                                               PlanRequest rq)
+__global__ __launch_bounds__(SCAN_BLOCK) void histogram_scan_kernel(OffT* __restrict__ hist,
+                                                                    uint32_t* __restrict__ varying,
+                                                                    uint64_t seg,
+                                                                    uint32_t passes,
+                                                                    uint64_t n_hist,
+                                                                    const VirtPlan* __restrict__ vplan,
+                                                                    uint32_t second,
+                                                                    uint32_t* __restrict__ blocks_done,
+                                                                    SortPlan* __restrict__ plan,
+                                                                    PlanRequest rq)
 {
   // first use (`second` == 0): nothing when the sort already runs on the ranks of the row's
   // different keys.  Second use, after vplan_kernel: scans the histograms of the grouped virtual
-  // digits (one row, block = group) and nothing when that plan is not in force.
+  // digits (one row, histogram = group) and nothing when that plan is not in force.
   if (vplan != nullptr) {
     const uint32_t mode = vplan->enabled;
-    if (second == 0 ? (mode == VIRT_DISTINCT) : (mode != VIRT_GROUPS || blockIdx.x >= vplan->n_groups)) {
+    if (second == 0 ? (mode == VIRT_DISTINCT) : (mode != VIRT_GROUPS)) {
       return;
     }
-  }
-  __shared__ OffT s_wsum[RADIX / WAVE];
-  const int tid  = threadIdx.x;
-  const int lane = tid & (WAVE - 1);
-  const int wave = tid / WAVE;
-  OffT* h        = hist + static_cast<uint64_t>(blockIdx.x) * RADIX;
-  const OffT c   = h[tid];
-  const int one_bin = __syncthreads_or(c == static_cast<OffT>(seg));
-  if (!one_bin && tid == 0) {
-    __hip_atomic_fetch_or(&varying[blockIdx.x % passes], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-  OffT incl      = c;
-#pragma unroll
-  for (int delta = 1; delta < WAVE; delta <<= 1) {
-    const OffT t = __shfl_up(incl, delta, WAVE);
-    if (lane >= delta) {
-      incl += t;
+    if (second != 0 && n_hist > vplan->n_groups) {
+      n_hist = vplan->n_groups;
     }
   }
-  if (lane == WAVE - 1) {
-    s_wsum[wave] = incl;
+  constexpr int PER_LANE = RADIX / WAVE;
+  const int tid          = threadIdx.x;
+  const int lane         = tid & (WAVE - 1);
+  const uint64_t wave    = static_cast<uint64_t>(blockIdx.x) * (SCAN_BLOCK / WAVE) + tid / WAVE;
+  const uint64_t nwaves  = static_cast<uint64_t>(gridDim.x) * (SCAN_BLOCK / WAVE);
+  uint32_t raised        = 0;  // passes this wavefront has flagged already
+  for (uint64_t h = wave; h < n_hist; h += nwaves) {
+    OffT* p = hist + h * RADIX + lane * PER_LANE;
+    OffT c[PER_LANE];
+    OffT sum     = 0;
+    bool one_bin = false;
+#pragma unroll
+    for (int j = 0; j < PER_LANE; ++j) {
+      c[j] = p[j];
+      one_bin |= (c[j] == static_cast<OffT>(seg));
+      sum += c[j];
+    }
+    const uint32_t pass = static_cast<uint32_t>(h % passes);
+    if (__builtin_amdgcn_ballot_w64(one_bin) == 0 && ((raised >> pass) & 1u) == 0) {
+      raised |= 1u << pass;
+      if (lane == 0) {
+        __hip_atomic_fetch_or(&varying[pass], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    OffT incl = sum;
+#pragma unroll
+    for (int delta = 1; delta < WAVE; delta <<= 1) {
+      const OffT t = __shfl_up(incl, delta, WAVE);
+      if (lane >= delta) {
+        incl += t;
+      }
+    }
+    OffT run = incl - sum;
+#pragma unroll
+    for (int j = 0; j < PER_LANE; ++j) {
+      p[j] = run;
+      run += c[j];
+    }
   }
-  __syncthreads();
-  OffT prefix = 0;
-  for (int w = 0; w < wave; ++w) {
-    prefix += s_wsum[w];
-  }
-  h[tid] = prefix + incl - c;
   // `blocks_done` given: the block that finishes last also makes the pass plan (saves a launch)
   if (blocks_done != nullptr) {
-    __shared__ uint32_t s_last;
-    __syncthreads();  // this block's flag (thread 0, above) is on its way
+    __syncthreads();  // the flags of this block's wavefronts are on their way
     if (tid == 0) {
       __threadfence();
       const uint32_t before = __hip_atomic_fetch_add(blocks_done, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-      s_last                = (before + 1 == gridDim.x) ? 1u : 0u;
-      if (s_last != 0) {
+      if (before + 1 == gridDim.x) {
         make_plan(varying, plan, rq);
       }
     }
@@ -427,6 +445,7 @@ struct SweepArgs {
   int pass;                // which 8-bit digit this pass sorts by
   int idx_final;           // idx_out is the caller's int64 array
   uint32_t spin_limit;     // polls of one descriptor before the tile gives up (LOOKBACK_SPIN_LIMIT)
+  uint32_t single_ticket;  // hand tiles out through `ticket` alone instead of the per-XCD counters
   const VirtPlan* vplan;   // virtual digits (virtual_digits.h), nullptr when the request cannot use them
   const DistinctTable* dtable;  // with vplan: the row's different keys when there are at most 256
   int free_rank;                // from the plan: this pass need not be stable
@@ -447,8 +466,9 @@ struct SweepArgs {
 // resident workgroups hold lower tiles only, which finish without it.  What the order does
 // assume is that every XCD keeps receiving workgroups of this launch: if other work kept one XCD
 // fully occupied for seconds, tiles elsewhere would wait for that XCD's share until the bounded
-// look-back gave up and the call reported CPN_ERR_DEVICE (a single counter for all XCDs has no
-// such dependence, at the price of the split lines).
+// look-back gave up and the call reported CPN_ERR_DEVICE.  A single counter for all XCDs has no
+// such dependence, at the price of the split lines: cpn_set_tile_order selects it at run time
+// (SweepArgs::single_ticket), and a caller that met CPN_ERR_DEVICE can repeat the sort that way.
 constexpr uint32_t XCD_COUNT = 8;
 #ifndef CPN_TILE_GROUP
 #define CPN_TILE_GROUP 8
@@ -876,7 +896,15 @@ void onesweep_kernel(const SweepArgs<BIG> a_in)
     // nothing more is sorted then.  (An ordinary load: what earlier launches wrote is visible
     // at the start of this one.  A failure inside this pass leaves its input consistent, every
     // offset stays inside the row, and waiting tiles notice the status word and drain.)
-    const uint32_t ticket = claim_tile(a.xcd_tickets, a.num_tiles);
+    uint32_t ticket;
+    if (a.single_ticket != 0) {  // tiles in launch-wide ascending order, whichever XCD asks
+      ticket = __hip_atomic_fetch_add(a.ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (ticket >= a.num_tiles) {
+        ticket = 0xFFFFFFFFu;
+      }
+    } else {
+      ticket = claim_tile(a.xcd_tickets, a.num_tiles);
+    }
     const uint32_t failed = *a.status;
     sh.tile               = (failed != 0) ? 0xFFFFFFFFu : ticket;
   }

@@ -48,6 +48,14 @@ uint64_t wide_row_threshold()
   return (t < 0 || static_cast<uint64_t>(t) > BIG_ROW_ELEMENTS) ? BIG_ROW_ELEMENTS : static_cast<uint64_t>(t);
 }
 
+// 0: tiles dealt per XCD, 1: one ticket counter for the launch
+static std::atomic<int> g_tile_order{[] {
+  const char* e = getenv("CPN_SORT_TILE_ORDER");
+  return (e != nullptr && (e[0] == 's' || e[0] == '1')) ? 1 : 0;
+}()};
+
+bool tile_order_single() { return g_tile_order.load(std::memory_order_relaxed) != 0; }
+
 static std::atomic<long long> g_spin_limit{static_cast<long long>(LOOKBACK_SPIN_LIMIT)};
 
 uint32_t lookback_spin_limit() { return static_cast<uint32_t>(g_spin_limit.load(std::memory_order_relaxed)); }
@@ -58,6 +66,13 @@ static std::atomic<long long> g_virt_threshold{[] {
 }()};
 
 uint64_t virtual_digit_threshold() { return static_cast<uint64_t>(g_virt_threshold.load(std::memory_order_relaxed)); }
+
+static const long long g_count16_min_row = [] {
+  const char* e = getenv("CPN_SORT_COUNT16_MIN_ROW");
+  return (e != nullptr && *e != 0) ? atoll(e) : static_cast<long long>(COUNT16_MIN_ROW);
+}();
+
+uint64_t count16_min_row() { return g_count16_min_row < 0 ? 0 : static_cast<uint64_t>(g_count16_min_row); }
 
 uint64_t wave_row_limit()
 {
@@ -155,6 +170,8 @@ int64_t cpn_set_lookback_spin_limit(int64_t polls)
   const long long v = (polls < 1 || polls > (1ll << 31)) ? static_cast<long long>(cpn::LOOKBACK_SPIN_LIMIT) : polls;
   return static_cast<int64_t>(cpn::g_spin_limit.exchange(v));
 }
+
+int cpn_set_tile_order(int single) { return cpn::g_tile_order.exchange(single != 0 ? 1 : 0); }
 
 int64_t cpn_set_wave_row_limit(int64_t limit)
 {

@@ -9,6 +9,7 @@
 #include <stdint.h>
 
 #include "../../include/cpn_sort.h"
+#include "count_row_sort.h"
 #include "lds_row_sort.h"
 #include "onesweep.h"
 #include "profile.h"
@@ -51,6 +52,9 @@ constexpr uint64_t BIG_ROW_ELEMENTS = 1ull << 30;
 constexpr uint64_t VIRT_MIN_ROW_ELEMENTS = 1ull << 26;
 // The threshold in force (cpn_set_virtual_digit_threshold; tests lower it).
 uint64_t virtual_digit_threshold();
+// How the scatter passes hand out their tiles: per XCD (default) or through one counter
+// (cpn_set_tile_order, CPN_SORT_TILE_ORDER=single).
+bool tile_order_single();
 // Rows of at least this many elements use 64-bit counts, descriptors and row positions:
 // BIG_ROW_ELEMENTS unless lowered by cpn_set_wide_row_threshold / CPN_SORT_WIDE_ROW_THRESHOLD
 // (for tests that exercise the 64-bit kernels without a 2^30-element row).
@@ -83,10 +87,11 @@ __host__ __device__ constexpr int global_tile(int key_bytes, bool big)
   return global_block(key_bytes) * global_items(key_bytes, big);
 }
 
-// Longest row the LDS kernel can take, per key width (keeps static LDS below 64 KiB).
+// Longest row the LDS kernel can take, per key width: 1024 threads with the row in 64 KiB of LDS
+// (plus staged row positions and the per-wave digit counters, 112 KiB at most of the CU's 160).
 __host__ __device__ constexpr uint64_t lds_row_capacity(int key_bytes)
 {
-  return key_bytes == 16 ? 2048 : (key_bytes == 8 ? 4096 : 8192);
+  return key_bytes == 16 ? 4096 : (key_bytes == 8 ? 8192 : 16384);
 }
 // Radix passes of a key: one per byte, plus the NaN-class pass of complex keys.
 __host__ __device__ constexpr int key_passes(int key_bytes, int codec)
@@ -97,6 +102,11 @@ __host__ __device__ constexpr int key_passes(int key_bytes, int codec)
 // Row length up to which one wavefront (instead of one workgroup) sorts a row; at most 1024.
 // Changed by cpn_set_wave_row_limit / CPN_SORT_WAVE_ROW_LIMIT for A/B runs.
 uint64_t wave_row_limit();
+
+// Shortest row of 2-byte keys that a values-only sort gives to the counting kernel
+// (count_row_sort.h): COUNT16_MIN_ROW unless CPN_SORT_COUNT16_MIN_ROW in the environment says
+// otherwise (A/B runs; a value above the LDS row capacity switches the kernel off).
+uint64_t count16_min_row();
 
 // Row length up to which the LDS kernel is used.  Equals lds_row_capacity unless the
 // environment variable CPN_SORT_LDS_ROW_LIMIT or cpn_set_lds_row_limit lowers it, e.g. to 0
@@ -259,6 +269,20 @@ inline int launch_lds_rows(const SortRequest& r)
   return CPN_OK;
 }
 
+template <int CODEC, int ITEMS>
+inline int launch_count16_rows(const SortRequest& r)
+{
+  const uint64_t rows = r.volume / r.seg;
+  {
+    ProfileScope prof("count16_row_sort", r.stream);
+    hipLaunchKernelGGL((count16_row_sort_kernel<CODEC, ITEMS>), dim3(static_cast<uint32_t>(rows)), dim3(COUNT16_BLOCK),
+                       0, r.stream, static_cast<const uint16_t*>(r.values_in), static_cast<uint16_t*>(r.values_out),
+                       static_cast<uint32_t>(r.seg), static_cast<uint32_t*>(r.temp));
+  }
+  CPN_HIP_TRY(hipGetLastError());
+  return CPN_OK;
+}
+
 template <typename KeyT, int CODEC, bool HAS_IDX, int ITEMS>
 inline int launch_wave_rows(const SortRequest& r)
 {
@@ -330,6 +354,12 @@ inline int sort_rows_in_lds(const SortRequest& r)
       return launch_wave_rows<KeyT, CODEC, HAS_IDX, 16>(r);
     }
   }
+  if constexpr (sizeof(KeyT) == 2 && !HAS_IDX && CODEC != CODEC_COMPLEX) {
+    // values only, 2-byte keys: long rows are counted instead of ranked
+    if (r.seg >= count16_min_row() && r.seg >= 64) {
+      return r.seg <= 8192 ? launch_count16_rows<CODEC, 8>(r) : launch_count16_rows<CODEC, 16>(r);
+    }
+  }
   if (r.seg <= 64) {
     return launch_lds_rows<KeyT, CODEC, HAS_IDX, 64, 1>(r);
   } else if (r.seg <= 256) {
@@ -340,7 +370,7 @@ inline int sort_rows_in_lds(const SortRequest& r)
     return launch_lds_rows<KeyT, CODEC, HAS_IDX, 256, 8>(r);
   }
   if constexpr (sizeof(KeyT) == 16) {
-    return CPN_ERR_UNSUPPORTED;  // not reached: lds_row_capacity(16) == 2048
+    return launch_lds_rows<KeyT, CODEC, HAS_IDX, 1024, 4>(r);  // lds_row_capacity(16) == 4096
   } else {
     if (r.seg <= 4096) {
       // eight keys per thread when a thread also carries positions or 8-byte keys (10-25 % faster
@@ -351,16 +381,19 @@ inline int sort_rows_in_lds(const SortRequest& r)
         return launch_lds_rows<KeyT, CODEC, HAS_IDX, 256, 16>(r);
       }
     }
-    if constexpr (sizeof(KeyT) < 8) {
-      // sixteen waves of eight keys hide the ranking latency better than eight waves of sixteen
-      // (4-12 % on 2- and 4-byte keys); one-pass sorts of single bytes prefer fewer barriers
-      if constexpr (sizeof(KeyT) == 1) {
-        return launch_lds_rows<KeyT, CODEC, HAS_IDX, 512, 16>(r);
-      } else {
-        return launch_lds_rows<KeyT, CODEC, HAS_IDX, 1024, 8>(r);
-      }
+    if constexpr (sizeof(KeyT) == 8) {
+      return launch_lds_rows<KeyT, CODEC, HAS_IDX, 1024, 8>(r);  // lds_row_capacity(8) == 8192
     } else {
-      return CPN_ERR_UNSUPPORTED;  // not reached: lds_row_capacity(8) == 4096
+      if (r.seg <= 8192) {
+        // sixteen waves of eight keys hide the ranking latency better than eight waves of sixteen
+        // (4-12 % on 2- and 4-byte keys); one-pass sorts of single bytes prefer fewer barriers
+        if constexpr (sizeof(KeyT) == 1) {
+          return launch_lds_rows<KeyT, CODEC, HAS_IDX, 512, 16>(r);
+        } else {
+          return launch_lds_rows<KeyT, CODEC, HAS_IDX, 1024, 8>(r);
+        }
+      }
+      return launch_lds_rows<KeyT, CODEC, HAS_IDX, 1024, 16>(r);  // up to 16 384 keys
     }
   }
 }
@@ -455,8 +488,13 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
     CPN_HIP_TRY(hipGetLastError());
     {
       ProfileScope prof("histogram_scan", r.stream);
-      hipLaunchKernelGGL((histogram_scan_kernel<OffT>), dim3(static_cast<uint32_t>(L.rows * PASSES)),
-                         dim3(RADIX), 0, r.stream, hist, varying, r.seg, static_cast<uint32_t>(PASSES),
+      const uint64_t n_hist = L.rows * PASSES;
+      uint64_t sgrid        = (n_hist + SCAN_BLOCK / WAVE - 1) / (SCAN_BLOCK / WAVE);
+      if (sgrid > 1024) {
+        sgrid = 1024;
+      }
+      hipLaunchKernelGGL((histogram_scan_kernel<OffT>), dim3(static_cast<uint32_t>(sgrid)), dim3(SCAN_BLOCK), 0,
+                         r.stream, hist, varying, r.seg, static_cast<uint32_t>(PASSES), n_hist,
                          static_cast<const VirtPlan*>(vplan), 0u,
                          L.virt ? nullptr : reinterpret_cast<uint32_t*>(ws + HEADER_SCAN_DONE), plan, rq);
     }
@@ -480,9 +518,9 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
         CPN_HIP_TRY(hipGetLastError());
         {
           ProfileScope prof("virtual_scan", r.stream);
-          hipLaunchKernelGGL((histogram_scan_kernel<OffT>), dim3(static_cast<uint32_t>(PASSES)), dim3(RADIX), 0,
-                             r.stream, hist, varying, r.seg, static_cast<uint32_t>(PASSES), vplan, 1u,
-                             static_cast<uint32_t*>(nullptr), plan, rq);
+          hipLaunchKernelGGL((histogram_scan_kernel<OffT>), dim3((PASSES + SCAN_BLOCK / WAVE - 1) / (SCAN_BLOCK / WAVE)),
+                             dim3(SCAN_BLOCK), 0, r.stream, hist, varying, r.seg, static_cast<uint32_t>(PASSES),
+                             static_cast<uint64_t>(PASSES), vplan, 1u, static_cast<uint32_t*>(nullptr), plan, rq);
         }
         CPN_HIP_TRY(hipGetLastError());
       }
@@ -527,6 +565,7 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
     a.num_tiles          = static_cast<uint32_t>(L.num_tiles);
     a.pass               = p;
     a.spin_limit         = lookback_spin_limit();
+    a.single_ticket      = tile_order_single() ? 1u : 0u;
     a.vplan              = vplan;
     a.dtable             = dtable;
     {

@@ -109,6 +109,18 @@ int64_t cpn_set_wide_row_threshold(int64_t elements);
 int64_t cpn_set_lookback_spin_limit(int64_t polls);
 
 /*
+ * Process-wide tunable: how the scatter passes of the global sort hand their tiles to workgroups.
+ * 0 (default): per XCD, so that neighbouring tiles share an L2 (faster; assumes that every XCD of
+ * the device keeps receiving workgroups of the launch: if foreign work held one XCD for seconds,
+ * the bounded look-back would give up with CPN_ERR_DEVICE).  Non-zero: one ticket counter for the
+ * whole launch, which has no such dependence; a caller that met CPN_ERR_DEVICE repeats the sort
+ * this way.  Results do not depend on it.  Returns the previous setting.  Also initialised from the
+ * environment variable CPN_SORT_TILE_ORDER ("single" selects the one counter).  The reference has no
+ * counterpart (cub's onesweep takes tiles from one counter, behind src/cupynumeric/sort/cub_sort.cuh:120-143).
+ */
+int cpn_set_tile_order(int single);
+
+/*
  * Process-wide tunable: a 1-D sort of real 8-byte keys with at least `elements` elements lets
  * the device replace its eight byte passes by one pass on the ranks of the keys when the row
  * holds at most 256 different keys, or by fewer passes on "virtual digits" when the

@@ -114,7 +114,7 @@ SORT_TYPES = ["quicksort", "mergesort", "heapsort", "stable"]
 def test_integration_sort_and_argsort(size):
     # tests/integration/test_sort.py:84-125, test_argsort.py (same structure); duplicates are
     # present, so every kind is held to the stable result
-    rng = np.random.default_rng(hash(str(size)) & 0xFFFF)
+    rng = np.random.default_rng(1000 + SIZES.index(size))
     arr_np = rng.integers(-100, 100, size)
     arr_num = num.array(arr_np)
     for kind in SORT_TYPES:
@@ -153,7 +153,8 @@ def test_random_module_and_flatten():
 
 
 # ---- per-row LDS path: every dtype, lengths around every workgroup-shape boundary -------------------
-LDS_LENGTHS = [1, 2, 3, 63, 64, 65, 255, 256, 257, 1000, 1023, 1024, 1025, 4095, 4096, 4097, 8191, 8192]
+LDS_LENGTHS = [1, 2, 3, 63, 64, 65, 255, 256, 257, 1000, 1023, 1024, 1025, 4095, 4096, 4097, 8191, 8192, 8193,
+               12000, 16383, 16384]
 
 
 @pytest.mark.parametrize("dtype", ALL_DTYPES)
@@ -170,7 +171,7 @@ def test_lds_many_short_rows(lib, torch_cuda):
 
 
 @pytest.mark.parametrize("dtype", [np.int64, np.uint64, np.float64, np.complex64, np.complex128])
-@pytest.mark.parametrize("seg", [600, 1024, 1500, 4096])
+@pytest.mark.parametrize("seg", [600, 1024, 1500, 4096, 6000, 8192])
 def test_lds_rows_leading_digit_shortcut(lib, torch_cuda, dtype, seg):
     """Wide keys in the row kernels: rows that the leading digits order completely, rows with ties on
     the leading digits whose low digits are out of order (the check must fail and every pass run),
@@ -766,6 +767,80 @@ def test_lookback_gives_up_cleanly(lib, torch_cuda):
     assert np.array_equal(out.cpu().numpy(), np.sort(x, kind="stable") if want is None else want)
     if not seen_failure:  # timing: every poll of every tile happened to be answered at once
         pytest.skip("no look-back had to wait in five runs, the failure path was not reached")
+
+
+def test_single_ticket_tile_order(lib, torch_cuda, global_path):
+    """cpn_set_tile_order(1): tiles handed out through one counter instead of per XCD; same results."""
+    prev = lib.cpn_set_tile_order(1)
+    try:
+        assert prev == 0
+        for dtype, shape in [(np.float32, (300_001,)), (np.int64, (70_000,)), (np.uint16, (5, 40_000)), (np.int32, (3, 16385))]:
+            check_rows(lib, torch_cuda, make_input(dtype, shape, seed=5), f"single ticket {np.dtype(dtype)} {shape}")
+    finally:
+        assert lib.cpn_set_tile_order(prev) == 1
+
+
+def test_python_layer_status_modes(lib, torch_cuda, monkeypatch):
+    """The Python layer's handling of the device status word: lazy (default: read when data next
+    reaches the host), eager with one repeat in single-ticket order, off.  The failure is forced from
+    the host: a spin limit of one poll (lazy), a status read that reports it (eager)."""
+    from cupynumeric_amd import _sort
+    from cupynumeric_amd.runtime import runtime
+
+    rng = np.random.default_rng(8)
+    x = rng.integers(0, 1 << 31, 1 << 22).astype(np.int32)
+    want = np.argsort(x, kind="stable")
+    a = num.array(x)
+    # lazy: consecutive sorts, one read-back at the first host access
+    monkeypatch.setattr(runtime, "check_mode", "lazy")
+    first, second = num.argsort(a), num.sort(a)
+    assert runtime._status_used == 2
+    assert np.array_equal(np.asarray(first), want) and runtime._status_used == 0
+    assert np.array_equal(np.asarray(second), x[want])
+    # row sorts leave no status word behind
+    rows = num.array(x.reshape(1 << 10, 1 << 12))
+    num.sort(rows)
+    assert runtime._status_used == 0
+    # lazy, with every look-back forced to give up at its first unanswered poll: the error comes
+    # with the host read, when a sort failed (timing decides whether one did), and the layer recovers
+    prev = lib.cpn_set_lookback_spin_limit(1)
+    try:
+        results = [num.argsort(a) for _ in range(4)]
+        torch_cuda.cuda.synchronize()
+    finally:
+        lib.cpn_set_lookback_spin_limit(prev)
+    failed = bool(runtime._status_slots[: runtime._status_used].cpu().any())
+    if failed:
+        with pytest.raises(RuntimeError, match="failed on the device"):
+            np.asarray(results[0])
+    assert np.array_equal(np.asarray(num.argsort(a)), want)
+    # eager: a reported failure is answered by one repeat with the single tile counter
+    monkeypatch.setattr(runtime, "check_mode", "eager")
+    real_check = lib.cpn_local_sort_check
+    calls = {"n": 0, "order_at_repeat": None}
+
+    def failing_once(temp, stream):
+        calls["n"] += 1
+        if calls["n"] == 1:
+            real_check(temp, stream)
+            return _lib.CPN_ERR_DEVICE
+        calls["order_at_repeat"] = lib.cpn_set_tile_order(1)  # returns the order in force
+        lib.cpn_set_tile_order(calls["order_at_repeat"])
+        return real_check(temp, stream)
+
+    monkeypatch.setattr(lib, "cpn_local_sort_check", failing_once)
+    got = num.argsort(a)
+    monkeypatch.setattr(lib, "cpn_local_sort_check", real_check)
+    assert calls == {"n": 2, "order_at_repeat": 1}
+    assert lib.cpn_set_tile_order(0) == 0, "the tile order was not restored"
+    assert np.array_equal(np.asarray(got), want)
+    # an in-place sort cannot be repeated (its input is gone): the failure is raised
+    calls["n"] = 0
+    monkeypatch.setattr(lib, "cpn_local_sort_check", failing_once)
+    b = num.array(x)
+    with pytest.raises(RuntimeError):
+        b.sort()
+    monkeypatch.setattr(lib, "cpn_local_sort_check", real_check)
 
 
 # ---- virtual digits: fewer passes for keys whose bytes take few distinct values ---------------------
