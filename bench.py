@@ -34,16 +34,18 @@ if str(ROOT) not in sys.path:
 
 HBM_PEAK_BYTES_PER_S = 8.0e12  # MI355X HBM3E
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# of this file scaled by a plain copy of known size (profiles/*_traffic.txt).  Keyed by
-# (config, keys); workloads without such a measurement report null.
-MEASURED_TRAFFIC_BYTES = {
-    ("c1", 1 << 24): 1.44e8,    # onesweep, profiles/onesweep_c1_traffic.txt
-    ("c2", 1 << 28): 4.303e9,   # onesweep, profiles/onesweep_c2_traffic.txt
-    ("c3", 1 << 26): 1.074e9,   # lds_row_sort, profiles/lds_row_sort_c3_traffic.txt
-    ("c4", 1 << 27): 2.211e9,   # onesweep (the one pass on the ranks of the 16 different keys), profiles/onesweep_c4_traffic.txt
-    ("c5", 1 << 26): 2.69e8,    # lds_row_sort, profiles/lds_row_sort_c5_traffic.txt
-}
+def measured_traffic_bytes(config: str, kernel: str) -> float | None:
+    """HBM bytes per launch of `kernel` on workload `config`, as measured with rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE and scaled by a plain copy of known size: read from the summary line
+    of profiles/<kernel>_<config>_traffic.txt ("<kernel>: X GB of HBM traffic per launch"), so the
+    figure changes with the committed profile and is null where none exists."""
+    import re
+
+    path = ROOT / "profiles" / f"{kernel}_{config}_traffic.txt"
+    if not path.exists():
+        return None
+    m = re.search(rf"^{re.escape(kernel)}: ([0-9.]+) GB of HBM traffic per launch", path.read_text(), flags=re.M)
+    return float(m.group(1)) * 1e9 if m else None
 
 
 # -------------------------------------------------------------------------------------------------
@@ -88,6 +90,19 @@ def make_config(name: str, log2n: int | None = None, rows: int | None = None) ->
         x = rng.standard_normal((r, r)).astype(np.float16)
         return dict(name=name, x=x, op="sort", axis=0,
                     workload=f"c5: np.sort float16 ({r},{r}) axis 0, normal, seed 4")
+    if name in ("flat", "skinny"):
+        # examples/microbenchmarks/sort_bench.py:54-68 at size s: ceil(s^1/4) x ceil(s^3/4) ("2D-flat") and
+        # its transpose ("2D-skinny"), float32 from rng.random (examples/_benchmark/random_array.py:43-49)
+        import math
+
+        s_total = 1 << (28 if log2n is None else log2n)
+        a, b = math.ceil(math.pow(s_total, 1 / 4)), math.ceil(math.pow(s_total, 3 / 4))
+        shape = (a, b) if name == "flat" else (b, a)
+        rng = np.random.default_rng(8 if name == "flat" else 9)
+        x = rng.random(size=shape, dtype=np.float32)
+        return dict(name=name, x=x, op="sort", axis=-1,
+                    workload=f"sort-2D-{name}: np.sort float32 {shape} last axis, uniform [0,1), seed "
+                             f"{8 if name == 'flat' else 9} (the reference's sort_bench.py shape at s=2^{int(math.log2(s_total))})")
     raise ValueError(f"unknown config {name}")
 
 
@@ -552,18 +567,172 @@ def run_consumer(args) -> dict:
 
 
 # -------------------------------------------------------------------------------------------------
+ROW_KERNELS = ("tiny_row_sort", "wave_row_sort", "lds_row_sort", "count16_row_sort")
+
+
+def verify_result(job: GpuJob, cfg: dict) -> str:
+    """End-of-run check of the device result, on the device (full parity lives in tests/): 1-D
+    argsorts through permutation, order and stability, which together fix the stable argsort; value
+    sorts against torch.sort of the same input, element for element (equal or both NaN)."""
+    torch = job.torch
+    if cfg["op"] == "argsort":
+        return verify_sample(job, cfg)
+    tdt = {np.dtype(np.int32): torch.int32, np.dtype(np.float32): torch.float32, np.dtype(np.float64): torch.float64,
+           np.dtype(np.float16): torch.float16, np.dtype(np.int64): torch.int64}.get(cfg["x"].dtype)
+    if tdt is None:
+        return "not checked here"
+    x = job.d_in.view(tdt).view(job.shape)
+    got = job.d_val.view(tdt).view(job.shape)
+    ref = torch.sort(x, dim=0 if job.transposed else -1).values
+    same = (got == ref) | ((got != got) & (ref != ref))
+    return "ok" if bool(same.all()) else f"FAILED: {int((~same).sum())} elements differ from torch.sort"
+
+
+def run_sort_workload(name: str, steps: int, warmup: int, log2n=None, rows=None, profile_steps: int = 5,
+                      calibrate_copy: bool = False) -> tuple[dict, dict, GpuJob]:
+    """One sort workload: `steps` timed steps between two device synchronisations with the library's
+    launch timing off (that is `ms_per_step`), the same steps timed one by one with events on the
+    stream (median and min), then a separate short loop with launch timing on for the per-kernel
+    durations.  Returns (result fields, config, job)."""
+    from cupynumeric_amd import _lib
+
+    cfg = make_config(name, log2n, rows)
+    job = GpuJob(cfg)
+    torch, lib = job.torch, job.lib
+    if calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0").normal_()
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)  # reads 1 GiB, writes 1 GiB (shows up as the runtime's copyBuffer kernel)
+        torch.cuda.synchronize()
+        del src, dst
+
+    lib.cpn_profile_enable(0)
+    for _ in range(warmup):
+        job.step()
+    torch.cuda.synchronize()
+    job.check_status()
+
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        job.step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    job.check_status()
+
+    # the same step, one at a time, between events on the stream the library launches on
+    per_step = []
+    for _ in range(steps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        job.step()
+        e1.record()
+        torch.cuda.synchronize()
+        per_step.append(e0.elapsed_time(e1))
+
+    # per-kernel launch durations: the library's own HIP events, in a loop of their own (recording
+    # them costs a few microseconds per launch, which the timed loop above does not pay)
+    lib.cpn_profile_enable(1)
+    _lib.profile_collect()  # drop anything recorded earlier
+    torch.cuda.synchronize()
+    for _ in range(profile_steps):
+        job.step()
+    torch.cuda.synchronize()
+    lib.cpn_profile_enable(0)
+    records = _lib.profile_collect()
+    job.check_status()
+
+    step_s = elapsed / steps
+    by_label: dict[str, list[float]] = {}
+    for label, ms in records:
+        by_label.setdefault(label, []).append(ms)
+    passes_run = None
+    if "onesweep" in by_label:  # launches of skipped passes exit at once: keep the ones that moved data
+        longest = max(by_label["onesweep"])
+        skipped = [t for t in by_label["onesweep"] if t < 0.1 * longest]
+        by_label["onesweep"] = [t for t in by_label["onesweep"] if t >= 0.1 * longest]
+        if skipped:
+            by_label["onesweep_skipped"] = skipped
+        passes_run = round(len(by_label["onesweep"]) / profile_steps)
+    # sweeps whose launch exits at once because the device-side plan has no use for them
+    for label in ("histogram", "virtual_histogram", "distinct_sweep"):
+        if label in by_label and cfg["x"].nbytes >= (1 << 26) and max(by_label[label]) < 0.02:
+            by_label[label + "_skipped"] = by_label.pop(label)
+    alg = algorithmic_bytes(cfg, job.uses_lds_rows, passes_run)
+    if job.uses_lds_rows:  # whichever of the per-row kernels the row length selects
+        dominant = next(k for k in ROW_KERNELS if k in by_label)
+        alg[dominant] = alg["lds_row_sort"]
+    else:
+        dominant = "onesweep"
+    avg_ms = float(np.mean(by_label[dominant]))
+    achieved = alg[dominant] / (avg_ms * 1e-3)
+    kernels = {
+        label: {"launches_per_step": len(v) / profile_steps, "avg_ms": float(np.mean(v)),
+                "algorithmic_GBps": (alg[label] / (float(np.mean(v)) * 1e-3) / 1e9) if label in alg else None}
+        for label, v in by_label.items()
+    }
+    roofline = {
+        "kernel": dominant,
+        "bound": "hbm",
+        "achieved": achieved / 1e9,
+        "peak": HBM_PEAK_BYTES_PER_S / 1e9,
+        "unit": "GB/s",
+        "frac": achieved / HBM_PEAK_BYTES_PER_S,
+        "traffic": measured_traffic_bytes(name, dominant) if (log2n is None and rows is None) else None,
+        "bytes_per_launch": alg[dominant],
+        "avg_launch_ms": avg_ms,
+        "launches_per_step": len(by_label[dominant]) / profile_steps,
+    }
+    if "onesweep_baseline_formula" in alg and dominant == "onesweep":
+        # for comparison only: the baseline's accounting moves an 8-byte payload in every pass, this
+        # build moves 4-byte row positions, so `achieved` above is the smaller, real figure
+        fb = alg["onesweep_baseline_formula"]
+        roofline["baseline_formula"] = {"bytes_per_launch": fb, "achieved": fb / (avg_ms * 1e-3) / 1e9,
+                                        "frac": fb / (avg_ms * 1e-3) / HBM_PEAK_BYTES_PER_S}
+    step_bytes = sum(alg.get(k, 0) * len(v) / profile_steps for k, v in by_label.items() if k in alg)
+    fields = {
+        "value": cfg["x"].size / step_s,
+        "ms_per_step": step_s * 1e3,
+        "ms_per_step_median": float(np.median(per_step)),
+        "ms_per_step_min": float(np.min(per_step)),
+        "dtype": {1: "u8", 2: "u16", 4: "u32", 8: "u64"}[cfg["x"].dtype.itemsize],
+        "config": {"workload": cfg["workload"], "keys": int(cfg["x"].size), "op": cfg["op"],
+                   "path": dominant if job.uses_lds_rows else f"onesweep, 8-bit digits, {passes_run} passes ran",
+                   "workspace_bytes": int(job.temp_bytes)},
+        "roofline": roofline,
+        "whole_step": {"algorithmic_bytes": step_bytes, "GBps": step_bytes / step_s / 1e9,
+                       "frac_of_hbm_peak": step_bytes / step_s / HBM_PEAK_BYTES_PER_S,
+                       **({"baseline_formula_bytes": alg["whole_baseline_formula"],
+                           "baseline_formula_frac": alg["whole_baseline_formula"] / step_s / HBM_PEAK_BYTES_PER_S}
+                          if "whole_baseline_formula" in alg else {})},
+        "kernels": kernels,
+        "verify": verify_result(job, cfg),
+    }
+    return fields, cfg, job
+
+
+# the other workloads reported beside the headline: the baseline's configs and the reference's own
+# 2-D microbenchmark shapes
+ALL_CONFIGS = ("c1", "c3", "c4", "c5", "flat", "skinny")
+
+
 def main() -> None:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="c2",
-                    choices=["c1", "c2", "c3", "c4", "c5", "lexsort", "searchsorted", "unique"],
-                    help="c1..c5: the sort workloads of the baseline; lexsort / searchsorted / unique: the "
-                         "callers and consumers of the sort path, on workloads of this file's own choosing")
+                    choices=["c1", "c2", "c3", "c4", "c5", "flat", "skinny", "lexsort", "searchsorted", "unique"],
+                    help="c1..c5: the sort workloads of the baseline; flat / skinny: the 2-D shapes of the "
+                         "reference's sort microbenchmark; lexsort / searchsorted / unique: the callers and "
+                         "consumers of the sort path, on workloads of this file's own choosing")
     ap.add_argument("--log2n", type=int, default=None, help="shrink a 1-D workload to 2^L keys")
     ap.add_argument("--rows", type=int, default=None, help="shrink a 2-D workload to this many rows")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-all-configs", action="store_true",
+                    help="the default run (c2 at full size) also times the other workloads, 10 steps each, and "
+                         "reports them under all_configs; this switch leaves them out")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy, the known-size kernel that "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -575,121 +744,58 @@ def main() -> None:
         print(json.dumps(run_consumer(args)))
         return
 
-    cfg = make_config(args.config, args.log2n, args.rows)
-    job = GpuJob(cfg)
+    fields, cfg, job = run_sort_workload(args.config, args.steps, args.warmup, args.log2n, args.rows,
+                                         calibrate_copy=args.calibrate_copy)
     torch = job.torch
-    lib = job.lib
-    from cupynumeric_amd import _lib
-
-    if args.calibrate_copy:
-        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0").normal_()
-        dst = torch.empty_like(src)
-        torch.cuda.synchronize()
-        dst.copy_(src)  # reads 1 GiB, writes 1 GiB (shows up as the runtime's copyBuffer kernel)
-        torch.cuda.synchronize()
-        del src, dst
-
-    for _ in range(args.warmup):
-        job.step()
-    torch.cuda.synchronize()
-    job.check_status()
-
-    lib.cpn_profile_enable(1)
-    _lib.profile_collect()  # drop anything recorded earlier
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        job.step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    lib.cpn_profile_enable(0)
-    records = _lib.profile_collect()
-    job.check_status()
-
-    ms_per_step = elapsed * 1e3 / args.steps
-    keys_per_s = cfg["x"].size / (elapsed / args.steps)
-
-    # per-kernel launch durations from the library's HIP events
-    by_label: dict[str, list[float]] = {}
-    for label, ms in records:
-        by_label.setdefault(label, []).append(ms)
-    passes_run = None
-    if "onesweep" in by_label:  # launches of skipped passes exit at once: keep the ones that moved data
-        longest = max(by_label["onesweep"])
-        skipped = [t for t in by_label["onesweep"] if t < 0.1 * longest]
-        by_label["onesweep"] = [t for t in by_label["onesweep"] if t >= 0.1 * longest]
-        if skipped:
-            by_label["onesweep_skipped"] = skipped
-        passes_run = round(len(by_label["onesweep"]) / args.steps)
-    # sweeps whose launch exits at once because the device-side plan has no use for them
-    for label in ("histogram", "virtual_histogram", "distinct_sweep"):
-        if label in by_label and cfg["x"].nbytes >= (1 << 26) and max(by_label[label]) < 0.02:
-            by_label[label + "_skipped"] = by_label.pop(label)
-    alg = algorithmic_bytes(cfg, job.uses_lds_rows, passes_run)
-    if job.uses_lds_rows:  # whichever of the per-row kernels the row length selects
-        dominant = next(k for k in ("tiny_row_sort", "wave_row_sort", "lds_row_sort") if k in by_label)
-        alg[dominant] = alg["lds_row_sort"]
-    else:
-        dominant = "onesweep"
-    avg_ms = float(np.mean(by_label[dominant]))
-    achieved = alg[dominant] / (avg_ms * 1e-3)
-    kernels = {
-        label: {"launches_per_step": len(v) / args.steps, "avg_ms": float(np.mean(v)),
-                "algorithmic_GBps": (alg[label] / (float(np.mean(v)) * 1e-3) / 1e9) if label in alg else None}
-        for label, v in by_label.items()
-    }
-    traffic = MEASURED_TRAFFIC_BYTES.get((args.config, cfg["x"].size))
     device_rates = measure_device_rates(torch)
-    roofline = {
-        "kernel": dominant,
-        "bound": "hbm",
-        "achieved": achieved / 1e9,
-        "peak": HBM_PEAK_BYTES_PER_S / 1e9,
-        "unit": "GB/s",
-        "frac": achieved / HBM_PEAK_BYTES_PER_S,
-        "traffic": traffic,
-        "bytes_per_launch": alg[dominant],
-        "avg_launch_ms": avg_ms,
-        "launches_per_step": len(by_label[dominant]) / args.steps,
-        # what this device sustains on plain streaming kernels, measured in this run: the published
-        # peak is not reached by a copy either
-        "device_rates": device_rates,
-        "frac_of_device_copy": achieved / 1e9 / device_rates["copy_GBps"],
-    }
-    if "onesweep_baseline_formula" in alg and dominant == "onesweep":
-        # for comparison only: the baseline's accounting moves an 8-byte payload in every pass, this
-        # build moves 4-byte row positions, so `achieved` above is the smaller, real figure
-        fb = alg["onesweep_baseline_formula"]
-        roofline["baseline_formula"] = {"bytes_per_launch": fb, "achieved": fb / (avg_ms * 1e-3) / 1e9,
-                                        "frac": fb / (avg_ms * 1e-3) / HBM_PEAK_BYTES_PER_S}
-    step_bytes = sum(alg.get(k, 0) * len(v) / args.steps for k, v in by_label.items() if k in alg)
-
+    # what this device sustains on plain streaming kernels, measured in this run: the published peak
+    # is not reached by a copy either
+    fields["roofline"]["device_rates"] = device_rates
+    fields["roofline"]["frac_of_device_copy"] = fields["roofline"]["achieved"] / device_rates["copy_GBps"]
+    headline = args.config == "c2" and args.log2n is None
     line = {
-        "metric": "sorted keys/sec, stable argsort fp32 N=2^28, 1 GPU" if args.config == "c2" and args.log2n is None
+        "metric": "sorted keys/sec, stable argsort fp32 N=2^28, 1 GPU" if headline
         else f"sorted keys/sec, config {args.config}, 1 GPU",
-        "value": keys_per_s,
+        "value": fields["value"],
         "unit": "keys/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
+        "ms_per_step": fields["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": {1: "u8", 2: "u16", 4: "u32", 8: "u64"}[cfg["x"].dtype.itemsize],
+        "dtype": fields["dtype"],
         "data": "synthetic",
-        "config": {"workload": cfg["workload"], "keys": int(cfg["x"].size), "op": cfg["op"],
-                   "path": dominant if job.uses_lds_rows else f"onesweep, 8-bit digits, {passes_run} passes ran",
-                   "workspace_bytes": int(job.temp_bytes)},
-        "roofline": roofline,
-        "whole_step": {"algorithmic_bytes": step_bytes, "GBps": step_bytes / (elapsed / args.steps) / 1e9,
-                       "frac_of_hbm_peak": step_bytes / (elapsed / args.steps) / HBM_PEAK_BYTES_PER_S,
-                       **({"baseline_formula_bytes": alg["whole_baseline_formula"],
-                           "baseline_formula_frac": alg["whole_baseline_formula"] / (elapsed / args.steps)
-                           / HBM_PEAK_BYTES_PER_S} if "whole_baseline_formula" in alg else {})},
-        "kernels": kernels,
-        "verify": verify_sample(job, cfg),
+        "config": fields["config"],
+        "roofline": fields["roofline"],
+        "ms_per_step_median": fields["ms_per_step_median"],
+        "ms_per_step_min": fields["ms_per_step_min"],
+        "whole_step": fields["whole_step"],
+        "kernels": fields["kernels"],
+        "verify": fields["verify"],
     }
+    del job
+    torch.cuda.empty_cache()
+    if headline and not args.no_all_configs:
+        others = {}
+        for name in ALL_CONFIGS:
+            f, _, j = run_sort_workload(name, steps=10, warmup=2)
+            r = f["roofline"]
+            others[name] = {
+                "workload": f["config"]["workload"], "keys": f["config"]["keys"], "path": f["config"]["path"],
+                "ms_per_step": f["ms_per_step"], "ms_per_step_median": f["ms_per_step_median"],
+                "ms_per_step_min": f["ms_per_step_min"], "keys_per_s": f["value"],
+                "dominant_kernel": r["kernel"], "kernel_avg_ms": r["avg_launch_ms"],
+                "kernel_launches_per_step": r["launches_per_step"], "algorithmic_bytes_per_launch": r["bytes_per_launch"],
+                "frac": r["frac"], "traffic": r["traffic"],
+                "whole_step_frac": f["whole_step"]["frac_of_hbm_peak"],
+                "kernels_ms": {k: round(v["avg_ms"] * v["launches_per_step"], 4) for k, v in f["kernels"].items()},
+                "verify": f["verify"],
+            }
+            del j
+            torch.cuda.empty_cache()
+        line["all_configs"] = others
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(cfg)
     print(json.dumps(line))

@@ -74,6 +74,26 @@ class ndarray:
         thunk = self._thunk.copy().reshape((self.size,))
         return ndarray(thunk.shape, thunk.dtype, thunk=thunk)
 
+    def reshape(self, *shape: Any, order: str = "C") -> "ndarray":
+        """View of the same dense storage under another shape (`cupynumeric/_array/array.py:3222-3283`;
+        C order only, one dimension may be -1)."""
+        if order not in ("C", "A"):
+            raise NotImplementedError("only C-order reshape is supported")
+        if len(shape) == 1 and not isinstance(shape[0], (int, np.integer)):
+            shape = tuple(shape[0])
+        dims = [int(d) for d in shape]
+        if dims.count(-1) > 1:
+            raise ValueError("can only specify one unknown dimension")
+        if -1 in dims:
+            known = int(np.prod([d for d in dims if d != -1], dtype=np.int64))
+            if known == 0 or self.size % known != 0:
+                raise ValueError(f"cannot reshape array of size {self.size} into shape {tuple(dims)}")
+            dims[dims.index(-1)] = self.size // known
+        if int(np.prod(dims, dtype=np.int64)) != self.size or any(d < 0 for d in dims):
+            raise ValueError(f"cannot reshape array of size {self.size} into shape {tuple(dims)}")
+        thunk = self._thunk.reshape(tuple(dims))
+        return ndarray(thunk.shape, thunk.dtype, thunk=thunk)
+
     def setflags(self, write: bool | None = None) -> None:
         if write is not None:
             self._writeable = bool(write)

@@ -80,24 +80,45 @@ def sort_task(output: "DeviceArray", input: "DeviceArray", argsort: bool, stable
             "cpn_local_sort",
         )
         raise NotImplementedError(f"cpn_local_sort: no workspace layout for dtype={input.dtype}, shape={input.shape}")
-    temp = runtime.empty_bytes(temp_bytes)
-    stream = runtime.stream_handle()
-    status = lib.cpn_local_sort(
-        code,
-        values_in,
-        values_out,
-        indices_out,
-        volume,
-        seg,
-        0,  # rect.lo[last] of a single-GPU launch (`src/cupynumeric/sort/sort.cu:1851`)
-        int(stable),
-        temp.data_ptr(),
-        temp_bytes,
-        ctypes.c_void_p(stream),
-    )
+    stream = ctypes.c_void_p(runtime.stream_handle())
+
+    def issue():
+        temp = runtime.empty_bytes(temp_bytes)
+        status = lib.cpn_local_sort(
+            code,
+            values_in,
+            values_out,
+            indices_out,
+            volume,
+            seg,
+            0,  # rect.lo[last] of a single-GPU launch (`src/cupynumeric/sort/sort.cu:1851`)
+            int(stable),
+            temp.data_ptr(),
+            temp_bytes,
+            stream,
+        )
+        _lib.check(status, "cpn_local_sort")
+        return temp
+
+    temp = issue()
+    # Rows sorted by the per-row kernels cannot fail on the device (the request then needs nothing but
+    # the workspace header).  The global sort can: a bounded wait between its tiles may run out.
+    if runtime.check_mode == "off" or temp_bytes == lib.cpn_local_sort_temp_bytes(code, 0, 0, 1, 0, 0):
+        return
+    if runtime.check_mode == "lazy":
+        runtime.defer_status(temp)
+        return
+    status = lib.cpn_local_sort_check(temp.data_ptr(), stream)
+    if status == _lib.CPN_ERR_DEVICE and not in_place:
+        # once more, from a fresh workspace, with the tiles handed out through one counter: that order
+        # does not depend on every XCD taking part (the input was not touched: it is not the output)
+        previous = lib.cpn_set_tile_order(1)
+        try:
+            temp = issue()
+            status = lib.cpn_local_sort_check(temp.data_ptr(), stream)
+        finally:
+            lib.cpn_set_tile_order(previous)
     _lib.check(status, "cpn_local_sort")
-    if runtime.check_status:
-        _lib.check(lib.cpn_local_sort_check(temp.data_ptr(), ctypes.c_void_p(stream)), "cpn_local_sort")
 
 
 def sort_deferred(

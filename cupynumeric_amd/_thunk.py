@@ -172,7 +172,7 @@ class DeviceArray:
             ctypes.c_void_p(runtime.stream_handle()),
         )
         _lib.check(status, "cpn_take_along_last_axis")
-        if runtime.check_status and int(flag.item()) != 0:
+        if runtime.check_mode != "off" and int(flag.item()) != 0:
             raise IndexError("index out of bounds in take_along_axis")
         return out
 
@@ -274,7 +274,9 @@ class DeviceArray:
             stream,
         )
         _lib.check(status, "cpn_searchsorted")
-        if temp is not None and runtime.check_status:
+        if temp is not None and runtime.check_mode == "lazy":
+            runtime.defer_status(temp)  # (the values were sorted first: that sort's status word)
+        elif temp is not None and runtime.check_mode == "eager":
             _lib.check(lib.cpn_local_sort_check(temp.data_ptr(), stream), "cpn_searchsorted")
 
     def unique(self) -> "DeviceArray":
@@ -296,7 +298,7 @@ class DeviceArray:
             code, self.base.ptr(), out.base.ptr(), self.size, count.data_ptr(), temp.data_ptr(), temp_bytes, stream
         )
         _lib.check(status, "cpn_unique")
-        if runtime.check_status:
+        if runtime.check_mode != "off":  # (reading the count below synchronises anyway)
             _lib.check(lib.cpn_local_sort_check(temp.data_ptr(), stream), "cpn_unique")
         n_unique = int(count.item())
         return DeviceArray((n_unique,), self.dtype, out.base)

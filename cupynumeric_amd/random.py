@@ -1,5 +1,6 @@
-"""Host-side random inputs wrapped as device arrays: the one `cupynumeric.random` call the
-reference's sort tests use (`tests/integration/test_sort.py`, `num.random.randint`)."""
+"""Host-side random inputs wrapped as device arrays: the `cupynumeric.random` calls that the
+reference's sort tests and its sort example make (`tests/integration/test_sort.py`:
+`num.random.randint`; `examples/sort.py:52-71`: `seed`, `randint`, `random`)."""
 from __future__ import annotations
 
 from typing import Any
@@ -15,3 +16,9 @@ def randint(low: int, high: int | None = None, size: Any = None, dtype: Any = in
     from . import array
 
     return array(np.random.randint(low, high, size=size, dtype=dtype))
+
+
+def random(size: Any = None):
+    from . import array
+
+    return array(np.random.random(size))

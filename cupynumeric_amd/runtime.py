@@ -19,10 +19,44 @@ if TYPE_CHECKING:
 class Runtime:
     """Process-wide state: device, settings."""
 
+    # status words of global sorts not yet read back (lazy mode): this many fit before a flush
+    STATUS_SLOTS = 256
+
     def __init__(self) -> None:
-        # read back the device status word after every sort (costs one stream sync)
-        self.check_status = os.environ.get("CUPYNUMERIC_AMD_CHECK_STATUS", "1") != "0"
+        # What happens to the device status word of a global sort (the per-row kernels cannot fail):
+        #   "lazy"  (default) it is copied to a small device array, asynchronously, and read back when
+        #           data next reaches the host; consecutive sorts do not synchronise
+        #   "eager" read back after every global sort (one stream sync each); a sort that failed is
+        #           repeated once with tiles handed out through one counter
+        #   "off"   never read
+        mode = os.environ.get("CUPYNUMERIC_AMD_CHECK_STATUS", "lazy").lower()
+        self.check_mode = {"0": "off", "off": "off", "1": "eager", "eager": "eager"}.get(mode, "lazy")
         self._torch = None
+        self._status_slots = None
+        self._status_used = 0
+
+    def defer_status(self, temp: "torch.Tensor") -> None:
+        """Lazy mode: keep the status word of the sort that just used `temp` (stream-ordered copy)."""
+        torch = self.torch
+        if self._status_slots is None:
+            self._status_slots = torch.zeros(self.STATUS_SLOTS, dtype=torch.int32, device=temp.device)
+        if self._status_used == self.STATUS_SLOTS:
+            self.flush_status()
+        self._status_slots[self._status_used : self._status_used + 1].copy_(temp[:4].view(torch.int32))
+        self._status_used += 1
+
+    def flush_status(self) -> None:
+        """Read back the deferred status words (synchronises); raises if a sort failed on the device."""
+        used, self._status_used = self._status_used, 0
+        if used == 0:
+            return
+        words = self._status_slots[:used].cpu()
+        if bool(words.any()):
+            raise RuntimeError(
+                "cpn_local_sort: a sort issued since the last host read failed on the device (a bounded wait "
+                "inside a kernel ran out, cpn_status -7); its result and everything computed from it are "
+                "invalid.  Repeat the work with CPN_SORT_TILE_ORDER=single or CUPYNUMERIC_AMD_CHECK_STATUS=eager"
+            )
 
     @property
     def torch(self):
@@ -69,6 +103,7 @@ class Runtime:
         return torch.from_numpy(flat).to(dev)
 
     def download(self, buf: "torch.Tensor", shape: tuple[int, ...], dtype: np.dtype) -> np.ndarray:
+        self.flush_status()
         nbytes = int(np.prod(shape, dtype=np.int64)) * dtype.itemsize
         if nbytes == 0:
             return np.empty(shape, dtype=dtype)

@@ -191,6 +191,18 @@ def argsort(a, axis=-1, kind="quicksort", order=None, threads: int = 1) -> np.nd
     return _thunk_sort(x, True, axis, kind, order, threads)
 
 
+def sort_complex(a, threads: int = 1) -> np.ndarray:
+    """`cupynumeric/_module/ssc_sorting.py:124-159`: sort along the last axis, then force a complex
+    result: complex input keeps its type, integers of at most 16 bits become complex64, everything
+    else complex128."""
+    result = sort(a, threads=threads)
+    if np.issubdtype(result.dtype, np.complexfloating):
+        return result
+    if np.issubdtype(result.dtype, np.integer) and result.dtype.itemsize <= 2:
+        return result.astype(np.complex64)
+    return result.astype(np.complex128)
+
+
 def lexsort(keys, axis=-1, threads: int = 1) -> np.ndarray:
     """`cupynumeric/_module/ssc_sorting.py:271-444`: validation, then a stable argsort of the first
     key and, for every further key, reorder / argsort / reorder.  Keys keep their own element

@@ -5,11 +5,13 @@ tests hold for sort and argsort.
 
 Only data is taken: the literal input arrays, the shapes/axes they are tried on and the literal
 expected outputs in
-    tests/cpp/integration/test_sort.cc     (int32 :26-60, double :62-96, inputs :541-555)
-    tests/cpp/integration/test_argsort.cc  (12-element :26-60, 4-D..7-D :62-204, inputs :282-377)
+    tests/cpp/integration/test_sort.cc          (int32 :26-60, double :62-96, inputs :541-555)
+    tests/cpp/integration/test_argsort.cc       (12-element :26-60, 4-D..7-D :62-204, inputs :282-377)
+    tests/cpp/integration/test_sort_complex.cc  (complex :27-126, from integers :141-152, 4-D..7-D
+                                                 :154-195, inputs and shapes :257-345)
 The reference is read as text, never imported, built or run.  Cases the reference generates by
-formula (10 000 reversed elements :379-410, empty :412-433, single item :435-455) are restated as
-formulas in tests/test_oracle.py instead of being stored.  Complex values are stored as
+formula (10 000 reversed elements :379-410, empty :412-433, single item :435-455; test_sort_complex.cc
+:347-390) are restated as formulas in tests/test_oracle.py instead of being stored.  Complex values are stored as
 [real, imag] pairs (test_sort.cc:98-134,557-571, test_argsort.cc:298-311,330-344).
 """
 from __future__ import annotations
@@ -43,7 +45,7 @@ def parse_expect_table(body: str) -> list[dict[str, list[float]]]:
     return [{str(axis): vals for axis, vals in per_shape} for per_shape in nested]
 
 
-COMPLEX = re.compile(r"legate::Complex<float>\(\s*([-0-9.eE]+)\s*,\s*([-0-9.eE]+)\s*\)")
+COMPLEX = re.compile(r"legate::Complex<\w+>\(\s*([-0-9.eE]+)\s*,\s*([-0-9.eE]+)\s*\)")
 
 
 def decomplex(text: str) -> str:
@@ -131,9 +133,51 @@ def main() -> None:
         table = parse_expect_table(function_body(argsort_cc, f"get_argsort_expect_result_{nd}d"))
         add("argsort", "int32", data16, shapes, table, False, f"test_argsort.cc get_argsort_expect_result_{nd}d")
 
+    # sort_complex: test_sort_complex.cc.  One expected array per shape (the sort is along the last axis).
+    cplx_cc = (tdir / "test_sort_complex.cc").read_text()
+    out["source"] += ", test_sort_complex.cc"
+    out["sort_complex_cases"] = []
+
+    def add_complex(in_dtype, out_dtype, data, shapes, table, where):
+        assert len(shapes) == len(table), (where, len(shapes), len(table))
+        for shape, expect in zip(shapes, table):
+            out["sort_complex_cases"].append({"in_dtype": in_dtype, "out_dtype": out_dtype, "input": data,
+                                              "shape": shape, "expect": expect, "where": where})
+
+    def int_table(fn_name):
+        body = function_body(cplx_cc, fn_name)
+        init = body[body.index("= {") + 2 : body.index("};") + 1]
+        return [[[float(v), 0.0] for v in row] for row in json.loads(init.replace("{", "[").replace("}", "]"))]
+
+    def complex_table(fn_name):
+        body = decomplex(function_body(cplx_cc, fn_name))
+        init = body[body.index("= {") + 2 : body.index("};") + 1]
+        return json.loads(init.replace("{", "[").replace("}", "]"))
+
+    body = cplx_cc[cplx_cc.index("void sort_complex_basic()") : cplx_cc.index("void sort_complex_basic_max_dim()")]
+    shapes_int = parse_shapes(body, "test_shapes_int")
+    from_int = int_table("get_sort_complex_expect_result_from_int")
+    ints = parse_array(body, "in_array1")
+    assert ints == parse_array(body, "in_array2") == parse_array(body, "int_array3")
+    add_complex("int8", "complex64", ints, shapes_int, from_int, "test_sort_complex.cc:141-152,257-274")
+    add_complex("int16", "complex64", ints, shapes_int, from_int, "test_sort_complex.cc:141-152,265-268")
+    add_complex("int32", "complex128", ints, shapes_int, from_int, "test_sort_complex.cc:141-152,271-274")
+    shapes_c = parse_shapes(body[body.index("// Test complex type") :], "test_shapes")
+    table_c = complex_table("get_sort_complex_expect_result")
+    in4 = parse_complex_array(body, "in_array4")
+    assert in4 == parse_complex_array(body, "in_array5")
+    add_complex("complex64", "complex64", in4, shapes_c, table_c, "test_sort_complex.cc:27-126,277-295")
+    add_complex("complex128", "complex128", in4, shapes_c, table_c, "test_sort_complex.cc:27-126,297-312")
+    body = cplx_cc[cplx_cc.index("void sort_complex_basic_max_dim()") : cplx_cc.index("void sort_complex_large_array()")]
+    data16c = parse_array(body, "in_array")
+    for nd in (4, 5, 6, 7):
+        add_complex("int16", "complex64", data16c, parse_shapes(body, f"test_shapes_{nd}d"),
+                    int_table(f"get_sort_complex_expect_result_{nd}d"),
+                    f"test_sort_complex.cc get_sort_complex_expect_result_{nd}d")
+
     dst = Path(__file__).resolve().parent / "reference_vectors.json"
     dst.write_text(json.dumps(out, separators=(",", ":")) + "\n")
-    print(f"{len(out['cases'])} cases -> {dst}")
+    print(f"{len(out['cases'])} sort/argsort cases, {len(out['sort_complex_cases'])} sort_complex cases -> {dst}")
 
 
 if __name__ == "__main__":

@@ -4,10 +4,11 @@ brute-force insertion sort on adversarial float alphabets.  CPU only."""
 from __future__ import annotations
 
 import itertools
+import json
 
 import numpy as np
 import pytest
-from conftest import ALL_REAL_DTYPES, COMPLEX_DTYPES, assert_same_bits, case_array, make_input
+from conftest import ALL_REAL_DTYPES, COMPLEX_DTYPES, ROOT, assert_same_bits, case_array, make_input
 
 from oracle import sort_oracle as oracle
 
@@ -27,6 +28,24 @@ def test_reference_golden_vectors(reference_vectors):
                 got = oracle.argsort(x, axis=case["axis"], kind=kind)
                 want = np.array(case["expect"], dtype=np.int64).reshape(case["shape"])
             assert_same_bits(got, want, f"{case['where']} shape={case['shape']} axis={case['axis']} kind={kind}")
+
+
+def test_reference_sort_complex_golden_vectors():
+    # tests/cpp/integration/test_sort_complex.cc:27-195,257-345 (43 cases) and the formula case :347-390
+    cases = json.loads((ROOT / "tests" / "golden" / "reference_vectors.json").read_text())["sort_complex_cases"]
+    assert len(cases) == 43
+    for c in cases:
+        x = case_array(c["input"], c["in_dtype"], c["shape"])
+        want = case_array(c["expect"], c["out_dtype"], c["shape"])
+        got = oracle.sort_complex(x)
+        assert got.dtype == want.dtype and got.shape == want.shape, c["where"]
+        assert np.array_equal(got, want), (c["where"], c["shape"])
+        assert np.array_equal(got, np.sort_complex(x).astype(want.dtype)), c["where"]
+    count = 10000
+    for dt, out in ((np.int16, np.complex64), (np.int32, np.complex128), (np.complex64, np.complex64)):
+        x = (count - np.arange(count)).astype(dt)
+        got = oracle.sort_complex(x)
+        assert got.dtype == out and np.array_equal(got, (np.arange(count) + 1).astype(out))
 
 
 def test_reference_large_reversed():

@@ -25,6 +25,31 @@ def test_sort_complex_matches_numpy(dtype):
         assert np.array_equal(np.asarray(got), want)
 
 
+def test_sort_complex_reference_golden_vectors():
+    # tests/cpp/integration/test_sort_complex.cc:27-195,257-345 through the public API; the
+    # 10 000-element reversed input of :347-390 by its formula
+    import json
+
+    from conftest import ROOT, case_array
+
+    from oracle import sort_oracle as oracle
+
+    cases = json.loads((ROOT / "tests" / "golden" / "reference_vectors.json").read_text())["sort_complex_cases"]
+    assert len(cases) == 43
+    for c in cases:
+        x = case_array(c["input"], c["in_dtype"], c["shape"])
+        want = case_array(c["expect"], c["out_dtype"], c["shape"])
+        got = num.sort_complex(num.array(x))
+        assert got.dtype == want.dtype and got.shape == want.shape, c["where"]
+        assert np.array_equal(np.asarray(got), want), (c["where"], c["shape"])
+        assert np.array_equal(np.asarray(got), oracle.sort_complex(x)), c["where"]
+    count = 10000
+    for dt, out in ((np.int16, np.complex64), (np.int32, np.complex128), (np.complex64, np.complex64)):
+        x = (count - np.arange(count)).astype(dt)
+        got = num.sort_complex(num.array(x))
+        assert got.dtype == out and np.array_equal(np.asarray(got), (np.arange(count) + 1).astype(out))
+
+
 def partition_property(part: np.ndarray, original: np.ndarray, kth: int, axis: int) -> None:
     """tests/integration/test_partition.py:23-47: everything left of kth is <=, right is >=; and
     the element at kth is the one a full sort puts there."""
