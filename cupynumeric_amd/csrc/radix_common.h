@@ -74,6 +74,33 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v, int lane)
   return v;
 }
 
+// Inclusive scans across a wave through DPP lane moves (no LDS traffic, a few cycles per step, where
+// a shuffle goes through the LDS crossbar): four shifts inside each row of 16 lanes, then the last
+// lane of row 0 is added to row 1 and that of row 2 to row 3, then lane 31 to rows 2 and 3.  Lanes
+// without a source read 0, the identity of both operations (values are unsigned).
+template <bool MAX>
+__device__ __forceinline__ uint32_t wave_inclusive_scan_dpp_impl(uint32_t v)
+{
+  auto combine = [](uint32_t a, uint32_t b) -> uint32_t { return MAX ? (a > b ? a : b) : a + b; };
+  const int x  = static_cast<int>(v);
+  // row_shr:1 = 0x111, row_shr:2 = 0x112, row_shr:4 = 0x114, row_shr:8 = 0x118, row_bcast:15 = 0x142, row_bcast:31 = 0x143
+  uint32_t t = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, x, 0x111, 0xF, 0xF, true));
+  v          = combine(v, t);
+  t          = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x112, 0xF, 0xF, true));
+  v          = combine(v, t);
+  t          = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x114, 0xF, 0xF, true));
+  v          = combine(v, t);
+  t          = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x118, 0xF, 0xF, true));
+  v          = combine(v, t);
+  t          = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x142, 0xA, 0xF, false));
+  v          = combine(v, t);
+  t          = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x143, 0xC, 0xF, false));
+  v          = combine(v, t);
+  return v;
+}
+__device__ __forceinline__ uint32_t wave_inclusive_sum_dpp(uint32_t v) { return wave_inclusive_scan_dpp_impl<false>(v); }
+__device__ __forceinline__ uint32_t wave_inclusive_max_dpp(uint32_t v) { return wave_inclusive_scan_dpp_impl<true>(v); }
+
 // How the 256 digits of a tile are spread over the threads that scan them.
 template <int BLOCK>
 struct DigitThreads {

@@ -269,15 +269,43 @@ inline int launch_lds_rows(const SortRequest& r)
   return CPN_OK;
 }
 
-template <int CODEC, int ITEMS>
+// Compute units of the current device (the persistent grid of the counting kernel), looked up once.
+inline int compute_units()
+{
+  static thread_local int cached_device = -1;
+  static thread_local int cached_count  = 0;
+  int dev                               = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    return 256;
+  }
+  if (dev != cached_device) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+      n = 256;
+    }
+    cached_device = dev;
+    cached_count  = n;
+  }
+  return cached_count;
+}
+
+template <int CODEC>
 inline int launch_count16_rows(const SortRequest& r)
 {
   const uint64_t rows = r.volume / r.seg;
   {
     ProfileScope prof("count16_row_sort", r.stream);
-    hipLaunchKernelGGL((count16_row_sort_kernel<CODEC, ITEMS>), dim3(static_cast<uint32_t>(rows)), dim3(COUNT16_BLOCK),
-                       0, r.stream, static_cast<const uint16_t*>(r.values_in), static_cast<uint16_t*>(r.values_out),
-                       static_cast<uint32_t>(r.seg), static_cast<uint32_t*>(r.temp));
+    if (r.seg <= 8192) {
+      const uint64_t cus  = static_cast<uint64_t>(compute_units());
+      const uint64_t grid = rows < cus ? rows : cus;  // one workgroup per CU, each loops over its rows
+      hipLaunchKernelGGL((count16_rows_kernel<CODEC>), dim3(static_cast<uint32_t>(grid)), dim3(COUNT16_BLOCK), 0, r.stream,
+                         static_cast<const uint16_t*>(r.values_in), static_cast<uint16_t*>(r.values_out),
+                         static_cast<uint32_t>(r.seg), static_cast<uint32_t>(rows), static_cast<uint32_t*>(r.temp));
+    } else {
+      hipLaunchKernelGGL((count16_long_rows_kernel<CODEC>), dim3(static_cast<uint32_t>(rows)), dim3(COUNT16_BLOCK), 0,
+                         r.stream, static_cast<const uint16_t*>(r.values_in), static_cast<uint16_t*>(r.values_out),
+                         static_cast<uint32_t>(r.seg), static_cast<uint32_t*>(r.temp));
+    }
   }
   CPN_HIP_TRY(hipGetLastError());
   return CPN_OK;
@@ -357,7 +385,7 @@ inline int sort_rows_in_lds(const SortRequest& r)
   if constexpr (sizeof(KeyT) == 2 && !HAS_IDX && CODEC != CODEC_COMPLEX) {
     // values only, 2-byte keys: long rows are counted instead of ranked
     if (r.seg >= count16_min_row() && r.seg >= 64) {
-      return r.seg <= 8192 ? launch_count16_rows<CODEC, 8>(r) : launch_count16_rows<CODEC, 16>(r);
+      return launch_count16_rows<CODEC>(r);
     }
   }
   if (r.seg <= 64) {

@@ -61,11 +61,14 @@ THRUST_LIB_PATH = HERE / "_build" / "libcpnthrust.so"
 _thrust = None
 
 
-def thrust_local_sort(x: np.ndarray, argsort: bool, stable: bool = True, use_omp: bool = False):
+def thrust_local_sort(x: np.ndarray, argsort: bool, stable: bool = True, use_omp: bool = False,
+                      transparent: bool = False):
     """Baseline only (bench.py): the reference's CPU / OpenMP variant over rocThrust's host backends
     (thrust_baseline.cpp).  Copy + index initialisation as in `SortImplBodyCpu`
-    (`src/cupynumeric/sort/sort_cpu.inl:974-1025`), then the per-row thrust calls.  Floats with NaN
-    or -0.0 do not come out in NumPy's order."""
+    (`src/cupynumeric/sort/sort_cpu.inl:974-1025`), then the per-row thrust calls, with the typed
+    comparator `thrust::less<VAL>` (rocThrust's host radix sort) or, `transparent`, with
+    `thrust::less<>` as the reference passes it (`sort_cpu.inl:62-83`; rocThrust's merge sort).
+    Floats with NaN or -0.0 do not come out in NumPy's order either way."""
     global _thrust
     if _thrust is None:
         if not THRUST_LIB_PATH.exists():
@@ -76,6 +79,7 @@ def thrust_local_sort(x: np.ndarray, argsort: bool, stable: bool = True, use_omp
         _thrust.cpn_thrust_local_sort.restype = ctypes.c_int
         _thrust.cpn_thrust_local_sort.argtypes = [
             ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_int, ctypes.c_int,
+            ctypes.c_int,
         ]
     x = np.ascontiguousarray(x)
     seg = x.shape[-1]
@@ -85,7 +89,7 @@ def thrust_local_sort(x: np.ndarray, argsort: bool, stable: bool = True, use_omp
         indices = np.ascontiguousarray(np.broadcast_to(np.arange(seg, dtype=np.int64), x.shape))
     rc = _thrust.cpn_thrust_local_sort(
         DTYPE_CODES[x.dtype], values.ctypes.data, indices.ctypes.data if argsort else None, x.size, seg,
-        int(stable), int(use_omp),
+        int(stable), int(use_omp), int(transparent),
     )
     if rc != 0:
         raise RuntimeError(f"cpn_thrust_local_sort failed: {rc}")

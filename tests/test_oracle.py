@@ -315,8 +315,10 @@ def test_thrust_baseline_matches_numpy_on_plain_data():
             info = np.iinfo(dtype)
             x = rng.integers(info.min, info.max, (7, 3001), dtype=dtype, endpoint=True)
         for use_omp in (False, True):
-            assert np.array_equal(oracle.thrust_local_sort(x, False, use_omp=use_omp), np.sort(x, axis=-1, kind="stable"))
-            assert np.array_equal(oracle.thrust_local_sort(x, True, use_omp=use_omp), np.argsort(x, axis=-1, kind="stable"))
+            for transparent in (False, True):  # thrust::less<VAL> (radix sort) and thrust::less<> (merge sort)
+                kw = dict(use_omp=use_omp, transparent=transparent)
+                assert np.array_equal(oracle.thrust_local_sort(x, False, **kw), np.sort(x, axis=-1, kind="stable"))
+                assert np.array_equal(oracle.thrust_local_sort(x, True, **kw), np.argsort(x, axis=-1, kind="stable"))
 
 
 def test_unique_reference_golden_vectors():
