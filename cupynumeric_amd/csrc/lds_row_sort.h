@@ -19,6 +19,14 @@
 // FIXUP_ROUNDS, all passes are run, from the state reached, which is still a stable sort of
 // the input.
 //
+// Values-only sorts of rows whose keys that tie are the same bits (integers; floats without NaN and
+// -0.0): no order among equal keys shows, so the row need not go through stable passes at all.  It is
+// first split into 8192 ranges of equal width between its smallest and its largest key, one LDS atomic
+// per key on a histogram of 8192 bins, which leaves a handful of keys per bin on evenly or normally
+// distributed data; every key then finds its place inside its bin by counting the smaller keys of the bin.  A row that crowds
+// more than BUCKET_LIMIT keys into one bin (few different keys, tight clusters) goes through the
+// radix passes instead.  Used by the 1024-thread shapes (rows of more than 4096 keys).
+//
 // Floating-point rows without NaN and without -0.0 (found during the same reduction): on such
 // a row the ordered image of a key is a bijection of its bits, so the keys are replaced by
 // their images once, the passes take plain bytes of them, and the images are mapped back
@@ -29,10 +37,35 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "radix_common.h"
 #include "wave_row_sort.h"  // wave_all_and / wave_all_or, FIXUP_ROUNDS
 
 namespace cpn {
+
+// Bins of the split above for a tile of `tile` keys: four per key, 4096 to 8192.
+__host__ __device__ constexpr int bucket_bins_log2(int tile) { return tile <= 1024 ? 12 : 13; }
+// Most keys a bin may hold for the split to be used (each key of a bin is compared with all others).
+constexpr uint32_t BUCKET_LIMIT = 24;
+// Bins are kept in 16-byte chunks whose index is XOR-swizzled, so that the scan, in which a thread
+// walks consecutive chunks of its own, spreads a wave over all LDS banks.
+__device__ __forceinline__ uint32_t bucket_word(uint32_t bin)
+{
+  const uint32_t chunk = bin >> 2;
+  return ((chunk ^ ((chunk >> 4) & 15u)) << 2) | (bin & 3u);
+}
+
+// The arithmetic type of a real key of 4 or 8 bytes.
+template <int CODEC, int BYTES>
+struct NativeKey {
+  using type = uint32_t;
+};
+template <> struct NativeKey<CODEC_UNSIGNED, 8> { using type = uint64_t; };
+template <> struct NativeKey<CODEC_SIGNED, 4> { using type = int32_t; };
+template <> struct NativeKey<CODEC_SIGNED, 8> { using type = int64_t; };
+template <> struct NativeKey<CODEC_FLOAT, 4> { using type = float; };
+template <> struct NativeKey<CODEC_FLOAT, 8> { using type = double; };
 
 // Waves per SIMD the compiler has to leave room for.  1024 threads with 8 keys of up to 4 bytes each stay below 64
 // vector registers and 80 KiB of LDS so that two workgroups share a CU; that also takes at most
@@ -69,9 +102,23 @@ void lds_row_sort_kernel(const KeyT* keys_in,
   // costs registers beyond the 64 that let two workgroups share a CU
   constexpr bool IMAGES_OK = (CODEC == CODEC_FLOAT) && sizeof(KeyT) >= 4 && BLOCK <= 512;
 
+  // the split on leading bits: real keys of 4 and 8 bytes, values only
+  // (only the 1024-thread shapes, rows of more than 4096 keys: in the smaller shapes the bins cost
+  // the LDS that lets many workgroups share a CU, and rows of 1024 float64 keys went from 0.41 to 0.60 ms)
+  constexpr bool BUCKETS_OK = !HAS_IDX && NW == 1 && sizeof(KeyT) >= 4 && sizeof(KeyT) <= 8 && BLOCK == 1024 &&
+                              (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT);
+  constexpr int BINS_LOG2   = bucket_bins_log2(TILE);
+  constexpr int BINS        = 1 << BINS_LOG2;
+  constexpr int BINS_PER_THREAD = BINS / BLOCK;
+  static_assert(!BUCKETS_OK || (BINS_PER_THREAD >= 4 && BINS_PER_THREAD % 4 == 0), "a thread scans whole 16-byte chunks");
+
   __shared__ __align__(16) KeyT s_keys[TILE];
   __shared__ IdxS s_idx[HAS_IDX ? TILE : 1];
-  __shared__ uint32_t s_ctr[WAVES * RADIX];
+  // the per-wave digit counters of the radix passes and the bins of the split share their memory
+  // (the split is over, or given up, before the first radix pass clears its counters)
+  constexpr int CTR_WORDS = (BUCKETS_OK && BINS > WAVES * RADIX) ? BINS : WAVES * RADIX;
+  __shared__ __align__(16) uint32_t s_ctr[CTR_WORDS];
+  uint32_t* const s_bins = s_ctr;
   __shared__ uint32_t s_wsum[DT::WAVES];
   __shared__ SW s_red[2 * WAVES * NW];
 
@@ -202,6 +249,192 @@ void lds_row_sort_kernel(const KeyT* keys_in,
 #pragma unroll
       for (int i = 0; i < ITEMS; ++i) {
         key[i] = sign_flip(key[i]);
+      }
+    }
+  }
+  if constexpr (BUCKETS_OK) {
+    static_assert(!BUCKETS_OK || !IMAGES_OK, "the split works on the keys' own bits");
+    if (free_first && __builtin_popcount(active) >= 2) {  // uniform
+      using NT = typename NativeKey<CODEC, sizeof(KeyT)>::type;  // float, double or the integer type
+      auto native = [](KeyT k) -> NT {
+        NT v;
+        __builtin_memcpy(&v, &k, sizeof(NT));
+        return v;
+      };
+      // smallest and largest key of the row (the row holds no NaN and no -0.0: the keys' own order
+      // is the sort order), through the staging area, which is free until the keys are placed
+      NT lo = native(keys_in[base]), hi = lo;  // (a key of the row, whatever this lane holds)
+#pragma unroll
+      for (int i = 0; i < ITEMS; ++i) {
+        if (holds(i)) {
+          const NT v = native(key[i]);
+          lo         = v < lo ? v : lo;
+          hi         = v > hi ? v : hi;
+        }
+      }
+#pragma unroll
+      for (int d = 1; d < WAVE; d <<= 1) {
+        const NT a = __shfl_xor(lo, d, WAVE), b = __shfl_xor(hi, d, WAVE);
+        lo         = a < lo ? a : lo;
+        hi         = b > hi ? b : hi;
+      }
+      NT* s_ext = reinterpret_cast<NT*>(s_keys);
+      if (lane == 0) {
+        s_ext[wave]         = lo;
+        s_ext[WAVES + wave] = hi;
+      }
+      for (int j = tid; j < BINS / 4; j += BLOCK) {
+        reinterpret_cast<uint4*>(s_bins)[j] = make_uint4(0u, 0u, 0u, 0u);
+      }
+      __syncthreads();
+      for (int w = 0; w < WAVES; ++w) {
+        const NT a = s_ext[w], b = s_ext[WAVES + w];
+        lo         = a < lo ? a : lo;
+        hi         = b > hi ? b : hi;
+      }
+      // The bin of a key: its place between the smallest and the largest key, in equal steps of the
+      // value.  Float keys: subtraction of a constant, scaling and truncation never decrease with the
+      // key, rounding included, so a key in a lower bin is a smaller key, which is all the split
+      // needs.  (An infinite extreme or span makes the scale 0 or the product NaN, which converts to
+      // bin 0: the row then crowds one bin and takes the radix passes.)  Integer keys: the distance
+      // from the smallest key, shifted down until the largest distance fits the bins.
+      using FT = typename std::conditional<sizeof(KeyT) == 4, float, double>::type;
+      FT origin = 0, scale = 0;
+      KeyT img_lo = 0;
+      int shift   = 0;
+      if constexpr (CODEC == CODEC_FLOAT) {
+        origin = lo;
+        scale  = static_cast<FT>(BINS) / (hi - lo);
+      } else {
+        img_lo          = ordered_bits<CODEC, KeyT>(static_cast<KeyT>(lo));
+        const KeyT span = static_cast<KeyT>(ordered_bits<CODEC, KeyT>(static_cast<KeyT>(hi)) - img_lo);
+        const int bits  = 64 - __builtin_clzll(static_cast<unsigned long long>(span) | 1ull);
+        shift           = bits > BINS_LOG2 ? bits - BINS_LOG2 : 0;
+      }
+      auto bin_of = [&](KeyT k) -> uint32_t {
+        if constexpr (CODEC == CODEC_FLOAT) {
+          const uint32_t b = static_cast<uint32_t>((native(k) - origin) * scale);
+          return b < static_cast<uint32_t>(BINS) ? b : static_cast<uint32_t>(BINS - 1);
+        } else {
+          return static_cast<uint32_t>(static_cast<KeyT>(ordered_bits<CODEC, KeyT>(k) - img_lo) >> shift);
+        }
+      };
+#pragma unroll
+      for (int i = 0; i < ITEMS; ++i) {
+        if (holds(i)) {
+          atomicAdd(&s_bins[bucket_word(bin_of(key[i]))], 1u);
+        }
+      }
+      __syncthreads();
+      // exclusive scan of the bins: thread t owns bins [t*BINS_PER_THREAD, (t+1)*BINS_PER_THREAD)
+      uint32_t cnt[BINS_PER_THREAD];
+      uint32_t total = 0, largest = 0;
+#pragma unroll
+      for (int c = 0; c < BINS_PER_THREAD / 4; ++c) {
+        const uint4 q4 = *reinterpret_cast<const uint4*>(&s_bins[bucket_word((tid * BINS_PER_THREAD) + 4 * c)]);
+        cnt[4 * c] = q4.x, cnt[4 * c + 1] = q4.y, cnt[4 * c + 2] = q4.z, cnt[4 * c + 3] = q4.w;
+      }
+#pragma unroll
+      for (int j = 0; j < BINS_PER_THREAD; ++j) {
+        total += cnt[j];
+        largest = cnt[j] > largest ? cnt[j] : largest;
+      }
+      const uint32_t incl = wave_inclusive_sum_dpp(total);
+      if (lane == WAVE - 1) {
+        s_wsum[wave] = incl;
+      }
+      const int crowded = __syncthreads_or(largest > BUCKET_LIMIT ? 1 : 0);
+      if (crowded == 0) {
+        uint32_t run = incl - total;
+        for (int w = 0; w < wave; ++w) {
+          run += s_wsum[w];
+        }
+#pragma unroll
+        for (int c = 0; c < BINS_PER_THREAD / 4; ++c) {
+          uint32_t e[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            e[j] = run;
+            run += cnt[4 * c + j];
+          }
+          *reinterpret_cast<uint4*>(&s_bins[bucket_word((tid * BINS_PER_THREAD) + 4 * c)]) = make_uint4(e[0], e[1], e[2], e[3]);
+        }
+        __syncthreads();
+        // every key into its bin, in whatever order the atomics hand out
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+          if (holds(i)) {
+            const uint32_t pos = atomicAdd(&s_bins[bucket_word(bin_of(key[i]))], 1u);
+            s_keys[pos]        = key[i];
+          }
+        }
+        __syncthreads();
+        // Each bin now ends where its counter stands and starts where the bin before it ends.  The
+        // key at position p of the row goes to the start of its bin plus the number of keys of the
+        // bin that come before it: smaller ones, and equal ones at lower positions (equal keys are
+        // the same bits here, the rule only keeps the places distinct).
+        // (All keys of a thread walk their bins in step, so that every round has ITEMS independent
+        // LDS reads in flight instead of one.)
+        uint32_t place[ITEMS], len[ITEMS];
+        uint32_t longest = 0;
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+          place[i] = 0, len[i] = 0;
+          if (holds(i)) {
+            key[i] = s_keys[woff + i * WAVE];
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+          if (holds(i)) {
+            const uint32_t b   = bin_of(key[i]);
+            const uint32_t end = s_bins[bucket_word(b)];
+            place[i]           = (b == 0) ? 0u : s_bins[bucket_word(b - 1)];  // start of the bin
+            len[i]             = end - place[i];
+            longest            = len[i] > longest ? len[i] : longest;
+          }
+        }
+        uint32_t before[ITEMS];
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+          before[i] = 0;
+        }
+        for (uint32_t j = 0; j < longest; ++j) {
+          // (reads past the end of a bin are clamped to its start and not counted: no branch, so the
+          // reads of a round are issued together)
+          KeyT other[ITEMS];
+#pragma unroll
+          for (int i = 0; i < ITEMS; ++i) {
+            other[i] = s_keys[place[i] + (j < len[i] ? j : 0u)];
+          }
+#pragma unroll
+          for (int i = 0; i < ITEMS; ++i) {
+            const uint32_t at = place[i] + j;
+            const NT a = native(other[i]), b = native(key[i]);
+            const bool first = a < b || (a == b && at < woff + i * WAVE);
+            before[i] += (j < len[i] && first) ? 1u : 0u;
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+          place[i] += before[i];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+          if (holds(i)) {
+            s_keys[place[i]] = key[i];
+          }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+          if (holds(i)) {
+            key[i] = s_keys[woff + i * WAVE];
+          }
+        }
+        todo     = 0;      // sorted: no radix pass is left
+        shortcut = false;
       }
     }
   }

@@ -165,6 +165,50 @@ def test_lds_rows_all_dtypes(lib, torch_cuda, dtype):
             check_rows(lib, torch_cuda, x, f"{np.dtype(dtype)} rows={rows} seg={seg}")
 
 
+@pytest.mark.parametrize("dtype", [np.int32, np.uint32, np.float32, np.int64, np.uint64, np.float64])
+def test_lds_rows_split_on_leading_bits(lib, torch_cuda, dtype):
+    """Values-only sorts of rows whose ties are the same bits take the split on the leading bits and
+    the counting inside each bin: rows of distinct keys, rows with pairs and small groups of equal
+    keys, keys that differ in few bits or only in low bits, clusters that fill a bin up to and past
+    the limit (the radix passes take over), all lengths of the row kernels that have the path."""
+    rng = np.random.default_rng(np.dtype(dtype).itemsize * 31 + np.dtype(dtype).num)
+    dt = np.dtype(dtype)
+    for seg in (1024, 1500, 2048, 4095, 4096, 6000, 8192, 8193, 12000, 16384):
+        if dt.itemsize == 8 and seg > 8192:
+            continue
+        rows = 7
+        if dt.kind == "f":
+            x = rng.standard_normal((rows, seg)).astype(dtype)
+            x[1] = rng.random(seg).astype(dtype)                    # [0, 1): most exponent bits idle
+            x[2] = (1.0 + rng.random(seg) * 1e-3).astype(dtype)      # keys differ in low bits only
+            x[3, : seg // 2] = x[3, seg // 2 : 2 * (seg // 2)]      # every key twice
+            x[4] = np.round(x[4] * 64) / 64                          # a few hundred different keys: crowded bins
+            x[5, ::3] = dtype(0.5)                                   # one third of the row in one bin
+            x[x == 0] = dtype(1.0)                                   # (no zeros: -0.0 would leave the path)
+        else:
+            info = np.iinfo(dtype)
+            x = rng.integers(info.min, info.max, (rows, seg), dtype=dtype, endpoint=True)
+            x[1] = rng.integers(0, 1 << 20, seg).astype(dtype)       # 20 varying bits
+            x[2] = (rng.integers(0, 200, seg) + 1000).astype(dtype)  # 8 varying bits: bins of equal keys
+            x[3, : seg // 2] = x[3, seg // 2 : 2 * (seg // 2)]
+            x[4] = (x[4] >> dtype(dt.itemsize * 8 - 9))              # 512 different keys
+            x[5, ::3] = x[5, 0]
+        x[6] = np.sort(x[6])[::-1]
+        want = np.sort(x, axis=-1, kind="stable")
+        got, _ = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=False)
+        assert_same_bits(got, want, f"{dt} seg={seg}")
+        got, _ = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=False, in_place=True)
+        assert_same_bits(got, want, f"{dt} seg={seg} in place")
+    # groups of equal keys of every size around the limit of a bin
+    for group in (2, 23, 24, 25, 40):
+        seg = 4096
+        base = rng.permutation(seg // group + 1).astype(dtype)
+        x = np.repeat(base, group)[:seg].reshape(1, seg).copy()
+        rng.shuffle(x[0])
+        got, _ = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=False)
+        assert_same_bits(got, np.sort(x, axis=-1, kind="stable"), f"{dt} groups of {group}")
+
+
 def test_lds_many_short_rows(lib, torch_cuda):
     for dtype, shape in [(np.float64, (3000, 37)), (np.int8, (5000, 5)), (np.float16, (700, 401)), (np.uint32, (129, 1024))]:
         check_rows(lib, torch_cuda, make_input(dtype, shape, seed=11), f"{np.dtype(dtype)} {shape}")
