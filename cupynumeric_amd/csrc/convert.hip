@@ -37,6 +37,31 @@ struct Elem {
     static_cast<T*>(p)[i] = static_cast<T>(re);
   }
 };
+// float16 from a wider value with ONE rounding to nearest even, as NumPy's casts do.  float32 goes
+// through the hardware conversion.  float64 is first brought to float32 by truncation with the lost
+// bits ORed into the last place ("round to odd"): float32 keeps 13 bits more than float16, so the
+// second, proper rounding sees exactly what a direct one would.  64-bit integers go through float64
+// (exact below 2^53, and everything from 65520 up is infinity in float16 either way).
+__device__ __forceinline__ __half half_from(float v) { return __float2half(v); }
+__device__ __forceinline__ __half half_from(double v)
+{
+  float f = __double2float_rz(v);
+  if (v == v && static_cast<double>(f) != v) {  // inexact (not NaN): make the result odd
+    uint32_t bits;
+    __builtin_memcpy(&bits, &f, 4);
+    bits |= 1u;
+    __builtin_memcpy(&f, &bits, 4);
+  }
+  return __float2half(f);
+}
+__device__ __forceinline__ __half half_from(int64_t v) { return half_from(static_cast<double>(v)); }
+__device__ __forceinline__ __half half_from(uint64_t v) { return half_from(static_cast<double>(v)); }
+template <typename C>
+__device__ __forceinline__ __half half_from(C v)  // narrower integers and bool bytes: exact in float32 below 65520
+{
+  return __float2half(static_cast<float>(v));
+}
+
 template <>
 struct Elem<__half> {
   using carrier = float;
@@ -49,7 +74,7 @@ struct Elem<__half> {
   template <typename C>
   static __device__ __forceinline__ void store(void* p, uint64_t i, C re, C)
   {
-    static_cast<__half*>(p)[i] = __float2half(static_cast<float>(re));
+    static_cast<__half*>(p)[i] = half_from(re);
   }
 };
 template <>

@@ -191,6 +191,9 @@ extern "C" int cpn_take_along_last_axis(int elem_bytes, const void* src, const i
                                         uint64_t rows, uint64_t src_seg, uint64_t idx_seg, uint32_t* oob_flag,
                                         void* stream)
 {
+  if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8 && elem_bytes != 16) {
+    return CPN_ERR_DTYPE;  // (before anything divides by it)
+  }
   if (rows == 0 || idx_seg == 0) {
     return CPN_OK;
   }

@@ -661,8 +661,23 @@ int sort_typed(const SortRequest& r)
     return CPN_ERR_TEMP;
   }
   if (r.seg <= lds_row_limit(KB)) {
-    // one launch: the row kernels clear the status word of the workspace themselves
-    return has_idx ? sort_rows_in_lds<KeyT, CODEC, true>(r) : sort_rows_in_lds<KeyT, CODEC, false>(r);
+    // one launch: the row kernels clear the status word of the workspace themselves.  (More rows than a
+    // grid can have blocks, e.g. a (2^31, 1) array: one launch per 2^30 rows.)
+    constexpr uint64_t ROWS_PER_LAUNCH = 1ull << 30;
+    const uint64_t rows                = r.volume / r.seg;
+    for (uint64_t first = 0; first < rows; first += ROWS_PER_LAUNCH) {
+      const uint64_t count = rows - first < ROWS_PER_LAUNCH ? rows - first : ROWS_PER_LAUNCH;
+      SortRequest c        = r;
+      c.volume             = count * r.seg;
+      c.values_in          = static_cast<const KeyT*>(r.values_in) + first * r.seg;
+      c.values_out         = r.values_out != nullptr ? static_cast<KeyT*>(r.values_out) + first * r.seg : nullptr;
+      c.indices_out        = r.indices_out != nullptr ? r.indices_out + first * r.seg : nullptr;
+      const int rc         = has_idx ? sort_rows_in_lds<KeyT, CODEC, true>(c) : sort_rows_in_lds<KeyT, CODEC, false>(c);
+      if (rc != CPN_OK) {
+        return rc;
+      }
+    }
+    return CPN_OK;
   }
   const GlobalLayout L = global_layout(KB, PASSES, r.volume, r.seg, r.values_out != nullptr, has_idx, in_place);
   if (L.big) {

@@ -208,3 +208,35 @@ def test_more_than_2_to_31_elements():
     assert rc == 0, _lib.status_string(rc)
     assert lib.cpn_local_sort_check(temp.data_ptr(), stream) == 0
     assert bool(((out.to(torch.int32) & 0xFFFF) == k).all()), "sorted values differ from keys[argsort]"
+
+
+def test_more_rows_than_a_grid_has_blocks():
+    """(2^31 + 7, 1) int8: rows of one element, more of them than one launch can take; the row kernels
+    are launched in chunks.  Sorting rows of one element is the identity, their argsort is the offset."""
+    import ctypes
+
+    import torch
+
+    from cupynumeric_amd import _lib
+
+    free, _total = torch.cuda.mem_get_info()
+    if free < 30 * (1 << 30):
+        pytest.skip("needs about 22 GiB of free device memory")
+    lib = _lib.load()
+    dev = torch.device("cuda")
+    n = (1 << 31) + 7
+    g = torch.Generator(device=dev)
+    g.manual_seed(32)
+    keys = torch.randint(-128, 128, (n,), dtype=torch.int8, device=dev, generator=g)
+    code = _lib.DTYPE_CODES[np.dtype(np.int8)]
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    tb = lib.cpn_local_sort_temp_bytes(code, n, 1, 1, 1, 0)
+    assert tb > 0
+    temp = torch.empty(tb, dtype=torch.uint8, device=dev)
+    out = torch.zeros_like(keys)
+    idx = torch.full((n,), -7, dtype=torch.int64, device=dev)
+    rc = lib.cpn_local_sort(code, keys.data_ptr(), out.data_ptr(), idx.data_ptr(), n, 1, 3, 1, temp.data_ptr(), tb, stream)
+    assert rc == 0, _lib.status_string(rc)
+    assert lib.cpn_local_sort_check(temp.data_ptr(), stream) == 0
+    assert bool((out == keys).all())
+    assert bool((idx == 3).all())

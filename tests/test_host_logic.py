@@ -77,6 +77,11 @@ def test_argument_validation_without_a_device(lib):
     assert swap(4, 18, 64, shape, 2, 0, 1, None) == _lib.CPN_ERR_ALIGN
     empty = (ctypes.c_int64 * 2)(0, 4)
     assert swap(4, None, None, empty, 2, 0, 1, None) == _lib.CPN_OK
+    # an element size the gather does not know is refused before anything is computed from it
+    take = lib.cpn_take_along_last_axis
+    assert take(0, 16, 64, 128, 1, 4, 4, None, None) == _lib.CPN_ERR_DTYPE
+    assert take(3, 16, 64, 128, 1, 4, 4, None, None) == _lib.CPN_ERR_DTYPE
+    assert take(4, 18, 64, 128, 1, 4, 4, None, None) == _lib.CPN_ERR_ALIGN
 
 
 def test_temp_bytes_layout(lib):

@@ -199,3 +199,29 @@ def test_take_along_axis_public():
         num.take_along_axis(x, np.full((4, 5), 5), 1)
     with pytest.raises(np.exceptions.AxisError):
         num.take_along_axis(x, np.zeros((4, 5), dtype=int), 2)
+
+
+def test_astype_float16_rounds_once():
+    """Casts to float16 from wider types must round to nearest even once, as NumPy does: values on and
+    around the midpoints between neighbouring float16 numbers, where rounding to float32 first and to
+    float16 afterwards lands on the other neighbour."""
+    halves = np.array([1.0, 1.5, 1023.0, 2048.0, 6.1e-5, 5.96e-8, 3.0e-6, 65472.0, 0.333], dtype=np.float16)
+    nxt = np.nextafter(halves, np.float16(np.inf))
+    mid = (halves.astype(np.float64) + nxt.astype(np.float64)) / 2  # exact midpoints (representable in float64)
+    eps = np.abs(mid) * 2.0**-40
+    x = np.concatenate([mid, mid + eps, mid - eps, -mid, -(mid + eps), -(mid - eps),
+                        [65519.99, 65520.0, 65520.01, 1e300, -1e300, 2.0**-25, 2.0**-25 * (1 + 2.0**-30), np.nan, np.inf]])
+    got = np.asarray(num.array(x).astype(np.float16))
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16)
+    assert np.array_equal(got.view(np.uint16)[~np.isnan(want)], want.view(np.uint16)[~np.isnan(want)])
+    assert np.isnan(got[np.isnan(want)]).all()
+    for dt in (np.int64, np.uint64, np.int32):
+        v = np.array([0, 1, 2047, 2049, 4097, 4099, 65503, 65519, 65520, 70000, 2**30 + 1], dtype=dt)
+        if np.dtype(dt).itemsize == 8:
+            v = np.concatenate([v, np.array([2**40 + 1, 2**62 + 12345], dtype=dt)])
+        if np.dtype(dt).kind == "i":
+            v = np.concatenate([v, -v])
+        with np.errstate(over="ignore"):
+            want = v.astype(np.float16)
+        assert np.array_equal(np.asarray(num.array(v).astype(np.float16)).view(np.uint16), want.view(np.uint16)), dt
