@@ -20,6 +20,7 @@ from ._thunk import SUPPORTED_DTYPES, DeviceArray, check_dtype
 
 __all__ = [
     "ndarray", "array", "asarray", "sort", "argsort", "sort_complex", "partition", "argpartition", "lexsort", "searchsorted", "unique", "take_along_axis",
+    "quantile", "percentile", "median",
     "random",
     "SUPPORTED_DTYPES",
 ]
@@ -233,3 +234,6 @@ def _split_first_axis(a: ndarray) -> list[ndarray]:
     for i in range(a.shape[0]):
         out.append(ndarray(inner, a.dtype, thunk=host_or_dev.slice_first_axis(i, n_inner, inner)))
     return out
+
+
+from ._stats import median, percentile, quantile  # noqa: E402  (they call `sort` of this module)

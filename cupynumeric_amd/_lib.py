@@ -78,6 +78,10 @@ PROTOTYPES: dict[str, tuple] = {
     ),
     "cpn_unique_temp_bytes": (c_uint64, [c_int, c_uint64]),
     "cpn_unique": (c_int, [c_int, c_void_p, c_void_p, c_uint64, c_void_p, c_void_p, c_uint64, c_void_p]),
+    "cpn_quantile_sorted": (
+        c_int,
+        [c_int, c_void_p, c_uint64, c_uint64, c_uint64, c_uint64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p],
+    ),
     "cpn_take_along_last_axis": (
         c_int, [c_int, c_void_p, c_void_p, c_void_p, c_uint64, c_uint64, c_uint64, c_void_p, c_void_p]
     ),

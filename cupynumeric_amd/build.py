@@ -28,6 +28,7 @@ SOURCES = [
     "gather.hip",
     "searchsorted.hip",
     "unique.hip",
+    "quantile.hip",
     "sort_keys8.hip",
     "sort_keys16.hip",
     "sort_keys32.hip",

@@ -281,6 +281,24 @@ int cpn_unique(int dtype, const void* values_in, void* values_out, uint64_t volu
                uint64_t* count_out, void* temp, uint64_t temp_bytes, void* stream);
 
 /*
+ * Quantiles along the middle axis of `sorted`, a dense [outer][n][inner] array that is already
+ * sorted along that axis, for num_q quantiles whose positions the caller has worked out:
+ *   interpolate == 0   out[q][o][i] = sorted[o][left[q]][i]                       (element type `dtype`)
+ *   interpolate != 0   out[q][o][i] = (1 - gamma[q]) * sorted[o][left[q]][i]
+ *                                     + gamma[q] * sorted[o][right[q]][i]          (float64)
+ * with the two products and the sum rounded separately in the arithmetic the reference's
+ * expression has (the element type for float16 / float32 / float64, float64 for integers and bool).
+ * left, right (int64, in [0, n)) and gamma (float64) are device arrays of num_q entries; right and
+ * gamma may be NULL when interpolate == 0.  Complex types return CPN_ERR_DTYPE.  Replaces the
+ * per-quantile take / multiply / add tasks at the end of _quantile_impl
+ * (cupynumeric/_module/stats_order.py:249-337), which quantile, percentile and median run after
+ * their sort (stats_order.py:476-482, cupynumeric/_module/stats_avgs_vars.py:373-443).
+ */
+int cpn_quantile_sorted(int dtype, const void* sorted, uint64_t outer, uint64_t n, uint64_t inner,
+                        uint64_t num_q, const int64_t* left, const int64_t* right, const double* gamma,
+                        int interpolate, void* out, void* stream);
+
+/*
  * out[r][j] = src[r][indices[r][j]] for `rows` dense rows: src rows hold src_seg elements of
  * elem_bytes (1, 2, 4, 8 or 16) bytes, indices and out rows hold idx_seg elements.  Indices are
  * int64, negative ones count from the end of the row.  An index outside [-src_seg, src_seg)

@@ -324,3 +324,117 @@ def unique(ar, threads: int = 1) -> np.ndarray:
         differ &= ~(nan[1:] & nan[:-1])
     keep = np.concatenate(([True], differ))
     return s[keep]
+
+
+# ---- order statistics on top of the sort (`cupynumeric/_module/stats_order.py`) -------------------------
+_DESIRED_MOD_2 = int(np.lib.NumpyVersion(np.__version__) < "2.0.1")  # `stats_order.py:126`
+
+
+def _quantile_position(method: str, q: float, n: int):
+    """`stats_order.py:106-232`: (gamma, 0-based left position) of the thirteen estimators; gamma None
+    means the method picks a sample."""
+    import math
+
+    if method == "inverted_cdf":
+        pos = q * n
+        left = int(pos)
+        return (1.0 if pos - left > 0 else 0.0, left - 1)
+    if method == "averaged_inverted_cdf":
+        pos = q * n
+        left = int(pos)
+        return (1.0 if pos - left > 0 else 0.5, left - 1)
+    if method == "closest_observation":
+        pos = q * n - 0.5
+        left = int(pos)
+        gamma = 1 if (left != pos or left % 2 != _DESIRED_MOD_2) else 0
+        return (None, left - 1 + gamma)
+    one_based = {
+        "interpolated_inverted_cdf": lambda: q * n,
+        "hazen": lambda: q * n + 0.5,
+        "weibull": lambda: q * (n + 1),
+        "linear": lambda: q * (n - 1) + 1,
+        "median_unbiased": lambda: q * (n + 1.0 / 3.0) + 1.0 / 3.0,
+        "normal_unbiased": lambda: q * (n + 0.25) + 3.0 / 8.0,
+    }
+    if method in one_based:
+        pos = one_based[method]()
+        left = int(pos)
+        return (pos - left, left - 1)
+    pos = q * (n - 1)
+    if method == "lower":
+        return (None, int(pos))
+    if method == "higher":
+        return (None, int(math.ceil(pos)))
+    if method == "midpoint":
+        left = int(pos)
+        return (0.5 if pos != left else 0.0, left)
+    if method == "nearest":
+        return (None, int(np.round(pos)))
+    raise KeyError(method)
+
+
+def quantile(a, q, axis=None, method: str = "linear", keepdims: bool = False, threads: int = 1) -> np.ndarray:
+    """`stats_order.py:358-536` with `_quantile_impl` (`:249-337`) and `_reshuffle_reshape` (`:51-85`):
+    sort along the (merged) axis with the oracle's sort, then per quantile the sample at `left`, or
+    `(1.0 - gamma) * left_samples + gamma * right_samples` in NumPy's own arithmetic (a Python float
+    times an array keeps a float array's type and makes integers float64), assigned into an array of the
+    result type.  `out` and `overwrite_input` change no value and are left out."""
+    x = np.asarray(a)
+    original_shape = x.shape
+    axes_set = ()
+    if axis is not None and not np.isscalar(axis):
+        axes_set = tuple(int(ax) % x.ndim for ax in axis)
+        if len(axes_set) == 1:
+            real_axis, x_rr = axes_set[0], x
+        else:
+            wanted = sorted(axes_set)
+            first = wanted[0]
+            moved = np.moveaxis(x, wanted, range(first, first + len(wanted)))
+            merged = int(np.prod(moved.shape[first : first + len(wanted)], dtype=np.int64))
+            x_rr = np.ascontiguousarray(moved).reshape(moved.shape[:first] + (merged,) + moved.shape[first + len(wanted) :])
+            real_axis = first
+    else:
+        real_axis, x_rr = axis, x
+        if real_axis is not None:
+            axes_set = (int(real_axis) % x.ndim,)
+            real_axis = axes_set[0]
+    q_arr = np.asarray(q)
+    arr = sort(x_rr, axis=real_axis, threads=threads)
+    if arr.dtype.kind == "c":
+        raise TypeError("input array cannot be of complex type")
+    to_dtype = arr.dtype if method in ("inverted_cdf", "closest_observation", "lower", "higher", "nearest") else np.dtype(np.float64)
+    if real_axis is None:
+        n = arr.size
+        remaining = (1,) * len(original_shape) if keepdims else ()
+    else:
+        n = arr.shape[real_axis]
+        if keepdims:
+            remaining = tuple(1 if k in axes_set else original_shape[k] for k in range(len(original_shape)))
+        else:
+            remaining = tuple(arr.shape[k] for k in range(arr.ndim) if k != real_axis)
+    res = np.zeros((*q_arr.shape, *remaining), dtype=to_dtype)
+    for index, qv in np.ndenumerate(q_arr):
+        gamma, left = _quantile_position(method, float(qv), n)
+        right = left + 1
+        if left >= n - 1:
+            left = right = n - 1
+        elif left < 0:
+            left = right = 0
+        if gamma is None:
+            res[index] = arr.take(left, real_axis).reshape(remaining)
+        else:
+            lvals = arr.take(left, real_axis).reshape(remaining)
+            rvals = arr.take(right, real_axis).reshape(remaining)
+            with np.errstate(invalid="ignore", over="ignore"):
+                res[index] = ((1.0 - gamma) * lvals + gamma * rvals).astype(to_dtype)
+    return res
+
+
+def percentile(a, q, axis=None, method: str = "linear", keepdims: bool = False, threads: int = 1) -> np.ndarray:
+    """`stats_order.py:540-650`."""
+    return quantile(a, np.asarray(q) / 100.0, axis, method=method, keepdims=keepdims, threads=threads)
+
+
+def median(a, axis=None, keepdims: bool = False, threads: int = 1) -> np.ndarray:
+    """`cupynumeric/_module/stats_avgs_vars.py:373-443`."""
+    return quantile(a, 0.5, axis=axis, method="midpoint", keepdims=keepdims, threads=threads)

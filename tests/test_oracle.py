@@ -327,3 +327,54 @@ def test_unique_reference_golden_vectors():
     for values, shape, expected, dtype in UNIQUE_GOLDEN:
         got = oracle.unique(np.array(values, dtype=dtype).reshape(shape))
         assert got.dtype == np.dtype(dtype) and got.tolist() == expected
+
+
+# ---- order statistics -------------------------------------------------------------------------------
+QUANTILE_METHODS = ("inverted_cdf", "averaged_inverted_cdf", "closest_observation", "interpolated_inverted_cdf", "hazen",
+                    "weibull", "linear", "median_unbiased", "normal_unbiased", "lower", "higher", "midpoint", "nearest")
+# tests/integration/test_quantiles.py:44-73: the reference's own input
+QUANTILE_REF_INPUT = np.array([1, 2, 2, 40, 1, 1, 2, 1, 0, 10, 3, 3, 40, 15, 3, 7, 5, 4, 7, 3, 5, 1, 0, 9], dtype=int).reshape(2, 3, 4)
+QUANTILE_REF_QS = (0.5, [0.001, 0.37, 0.42, 0.67, 0.83, 0.99, 0.39, 0.49, 0.5])
+
+
+@pytest.mark.parametrize("method", QUANTILE_METHODS)
+def test_quantile_matches_numpy_on_the_reference_cases(method):
+    """The oracle's quantile / percentile / median against numpy's on the inputs, axes, quantiles and
+    keepdims of tests/integration/test_quantiles.py:36-111 and test_percentiles.py, to the reference's
+    own tolerance (atol 1e-8: its interpolation formula is not NumPy's), exactly for methods that pick
+    samples; plus float inputs, axis=None and 1-D."""
+    eps = 1.0e-8
+    rng = np.random.default_rng(44)
+    inputs = [QUANTILE_REF_INPUT, QUANTILE_REF_INPUT.astype(np.float64) / 3, rng.standard_normal((2, 3, 4)).astype(np.float32),
+              rng.integers(0, 100, (5, 7)).astype(np.uint8)]
+    for arr in inputs:
+        for axes in (None, 0, 1, (0,), (0, 1), (0, 2) if arr.ndim == 3 else (1,)):
+            for qs in QUANTILE_REF_QS:
+                for keepdims in (False, True):
+                    want = np.quantile(arr, qs, axis=axes, method=method, keepdims=keepdims)
+                    got = oracle.quantile(arr, qs, axis=axes, method=method, keepdims=keepdims)
+                    assert got.shape == want.shape
+                    if arr.dtype != np.float32:
+                        assert got.dtype == want.dtype, (method, axes, got.dtype, want.dtype)
+                    else:  # the reference gives float64 for every float narrower than that (stats_order.py:501-510), NumPy float32
+                        assert got.dtype == (np.float32 if method in ("inverted_cdf", "closest_observation", "lower", "higher", "nearest") else np.float64)
+                    if method in ("inverted_cdf", "closest_observation", "lower", "higher", "nearest"):
+                        assert np.array_equal(got, want), (method, axes, qs)
+                    else:
+                        assert np.allclose(got, want, atol=eps if arr.dtype != np.float32 else 1e-6), (method, axes, qs)
+                    p = oracle.percentile(arr, np.asarray(qs) * 100.0, axis=axes, method=method, keepdims=keepdims)
+                    assert np.allclose(p, np.percentile(arr, np.asarray(qs) * 100.0, axis=axes, method=method, keepdims=keepdims),
+                                       atol=1e-6)
+    for arr in inputs:
+        for axes in (None, 0, -1):
+            assert np.allclose(oracle.median(arr, axis=axes), np.median(arr, axis=axes), atol=1e-6)
+            assert oracle.median(arr, axis=axes, keepdims=True).shape == np.median(arr, axis=axes, keepdims=True).shape
+
+
+def test_quantile_closed_forms():
+    x = np.arange(101, dtype=np.float64)[::-1].copy()
+    assert np.array_equal(oracle.quantile(x, [0.0, 0.25, 0.5, 1.0]), [0.0, 25.0, 50.0, 100.0])
+    assert oracle.median(np.array([3, 1, 2, 10])) == 2.5
+    assert oracle.quantile(np.array([7]), 0.3, method="weibull") == 7.0
+    with pytest.raises(TypeError):
+        oracle.quantile(np.array([1 + 2j, 3j]), 0.5)
