@@ -314,7 +314,7 @@ inline int launch_count16_rows(const SortRequest& r)
 template <typename KeyT, int CODEC, bool HAS_IDX, int ITEMS>
 inline int launch_wave_rows(const SortRequest& r)
 {
-  constexpr int LDS_PER_ROW    = wave_row_lds_bytes<CODEC, KeyT, ITEMS>();
+  constexpr int LDS_PER_ROW    = wave_row_lds_bytes<CODEC, KeyT, ITEMS, HAS_IDX>();
   constexpr int ROWS_PER_BLOCK = LDS_PER_ROW <= 12 * 1024 ? 4 : (LDS_PER_ROW <= 24 * 1024 ? 2 : 1);
   const uint64_t rows          = r.volume / r.seg;
   const uint64_t blocks        = (rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;

@@ -209,6 +209,47 @@ def test_lds_rows_split_on_leading_bits(lib, torch_cuda, dtype):
         assert_same_bits(got, np.sort(x, axis=-1, kind="stable"), f"{dt} groups of {group}")
 
 
+@pytest.mark.parametrize("dtype", [np.int32, np.uint32, np.float32])
+def test_wave_rows_split_into_ranges(lib, torch_cuda, dtype):
+    """One-wave-per-row sorts of 4-byte keys, values only, on rows whose ties are the same bits: the
+    split into value ranges with counting inside each range, rows that crowd a range (the radix passes
+    take over), keys in a narrow range, pairs of equal keys, every length class of the kernel."""
+    rng = np.random.default_rng(np.dtype(dtype).num + 7)
+    dt = np.dtype(dtype)
+    for seg in (33, 64, 65, 100, 128, 129, 200, 256, 300, 512, 777, 1024):
+        rows = 9
+        if dt.kind == "f":
+            x = rng.standard_normal((rows, seg)).astype(dtype)
+            x[1] = rng.random(seg).astype(dtype)
+            x[2] = (1.0 + rng.random(seg) * 1e-3).astype(dtype)
+            x[3, : seg // 2] = x[3, seg // 2 : 2 * (seg // 2)]
+            x[4] = np.round(x[4] * 4) / 4                      # few different keys: crowded ranges
+            x[5, ::3] = dtype(0.5)
+            x[7, 0] = np.inf                                   # an infinite span: one crowded range
+            x[8] = x[8] * dtype(1e30)
+            x[x == 0] = dtype(1.0)                             # (no zeros: -0.0 would leave the path)
+        else:
+            info = np.iinfo(dtype)
+            x = rng.integers(info.min, info.max, (rows, seg), dtype=dtype, endpoint=True)
+            x[1] = rng.integers(0, 1 << 20, seg).astype(dtype)
+            x[2] = (rng.integers(0, 100000, seg) + 5000).astype(dtype)
+            x[3, : seg // 2] = x[3, seg // 2 : 2 * (seg // 2)]
+            x[4] = (x[4] >> dtype(28)) if dt.kind == "u" else (x[4] // dtype(1 << 28))   # 16 different keys
+            x[5, ::3] = x[5, 0]
+            x[7, 0], x[7, 1] = info.min, info.max
+            x[8] = rng.integers(0, 3, seg).astype(dtype) * dtype(1 << 24) + rng.integers(0, 7, seg).astype(dtype)
+        x[6] = np.sort(x[6])[::-1]
+        want = np.sort(x, axis=-1, kind="stable")
+        got, _ = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=False)
+        assert_same_bits(got, want, f"{dt} seg={seg}")
+        got, _ = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=False, in_place=True)
+        assert_same_bits(got, want, f"{dt} seg={seg} in place")
+    big = rng.standard_normal((20000, 128)).astype(np.float32).view(np.uint32).view(dtype) if dt.kind != "f" else \
+        rng.standard_normal((20000, 128)).astype(dtype)
+    got, _ = abi_sort(lib, torch_cuda, big, want_values=True, want_indices=False)
+    assert_same_bits(got, np.sort(big, axis=-1, kind="stable"), f"{dt} many rows of 128")
+
+
 def test_lds_many_short_rows(lib, torch_cuda):
     for dtype, shape in [(np.float64, (3000, 37)), (np.int8, (5000, 5)), (np.float16, (700, 401)), (np.uint32, (129, 1024))]:
         check_rows(lib, torch_cuda, make_input(dtype, shape, seed=11), f"{np.dtype(dtype)} {shape}")
