@@ -18,36 +18,32 @@ if TYPE_CHECKING:
 
 
 def sort_flattened(output: "DeviceArray", input: "DeviceArray", argsort: bool, stable: bool) -> None:
-    """`cupynumeric/_thunk/_sort.py:37-47`."""
+    """`axis=None` on an array of several dimensions (`cupynumeric/_thunk/_sort.py:37-47`): the
+    C-order flattening is a view of the same dense storage, its 1-D sort is the result."""
     from ._thunk import DeviceArray
 
-    flattened = input.reshape((input.size,), order="C")
-
-    # run sort flattened -- return 1D solution
-    sort_result = DeviceArray(flattened.shape, dtype=output.dtype)
-    sort_deferred(sort_result, flattened, argsort, stable=stable)
-    output.base = sort_result.base
+    flat = input.reshape((input.size,), order="C")
+    result = DeviceArray(flat.shape, dtype=output.dtype)
+    sort_deferred(result, flat, argsort, stable=stable)
+    output.base = result.base
 
 
 def sort_swapped(output: "DeviceArray", input: "DeviceArray", argsort: bool, sort_axis: int, stable: bool) -> None:
-    """`cupynumeric/_thunk/_sort.py:50-76`.  The reference hands back a transposed view of the
-    sorted copy; here the result is copied back so that every array stays dense row-major."""
+    """A sort along an axis that is not the last (`cupynumeric/_thunk/_sort.py:50-76`): transposed
+    dense copy, last-axis sort of the copy, transposed back.  The reference hands back a transposed
+    view of the sorted copy; here the result is copied back so that every array stays dense row-major."""
     from ._thunk import DeviceArray
 
     sort_axis = normalize_axis_index(sort_axis, input.ndim)
     last = input.ndim - 1
-
-    # swap axes (dense copy)
-    swapped_copy = input.swapaxes_copy(sort_axis, last)
-
-    # run sort on last axis
-    if argsort is True:
-        sort_result = DeviceArray(swapped_copy.shape, dtype=output.dtype)
-        sort_deferred(sort_result, swapped_copy, argsort, stable=stable)
-        output.base = sort_result.swapaxes_copy(last, sort_axis).base
+    moved = input.swapaxes_copy(sort_axis, last)
+    if argsort:
+        positions = DeviceArray(moved.shape, dtype=output.dtype)
+        sort_deferred(positions, moved, argsort, stable=stable)
+        output.base = positions.swapaxes_copy(last, sort_axis).base
     else:
-        sort_deferred(swapped_copy, swapped_copy, argsort, stable=stable)
-        output.base = swapped_copy.swapaxes_copy(last, sort_axis).base
+        sort_deferred(moved, moved, argsort, stable=stable)  # the copy is ours: sorted in place
+        output.base = moved.swapaxes_copy(last, sort_axis).base
 
 
 def sort_task(output: "DeviceArray", input: "DeviceArray", argsort: bool, stable: bool) -> None:
@@ -128,36 +124,30 @@ def sort_deferred(
     axis: int | None = -1,
     stable: bool = False,
 ) -> None:
-    """`cupynumeric/_thunk/_sort.py:110-136`."""
-    # Handle 0-D arrays (scalars)
+    """Axis dispatch of sort and argsort (`cupynumeric/_thunk/_sort.py:110-136`): 0-D input, `axis=None`
+    (flatten, or axis 0 of a 1-D array), the last axis (the kernel call), any other axis (transposes)."""
     if input.ndim == 0:
         if axis is not None:
-            # NumPy raises AxisError for any other axis value
-            raise AxisError(axis, input.ndim)
-        # For 0-D arrays, axis=None just returns the scalar
+            raise AxisError(axis, input.ndim)  # NumPy's answer to any axis of a scalar
         if argsort:
-            # the reference aliases the input store here even for argsort; a value buffer is
-            # not an index buffer, so hand back the only possible index instead
+            # (the reference aliases the input store here even for argsort; a value buffer is not an
+            # index buffer, so the only possible index is handed back instead)
             import numpy as np
 
             from ._thunk import Storage
 
             output.base = Storage(8, host=np.zeros(1, dtype=np.int64))
         else:
-            output.base = input.base
+            output.base = input.base  # a scalar is sorted
+        return
+    if axis is None and input.ndim > 1:
+        sort_flattened(output, input, argsort, stable)
+        return
+    sort_axis = 0 if axis is None else normalize_axis_index(axis, input.ndim)
+    if sort_axis == input.ndim - 1:
+        sort_task(output, input, argsort, stable)
     else:
-        if axis is None and input.ndim > 1:
-            sort_flattened(output, input, argsort, stable)
-        else:
-            if axis is None:
-                computed_axis = 0
-            else:
-                computed_axis = normalize_axis_index(axis, input.ndim)
-
-            if computed_axis == input.ndim - 1:
-                sort_task(output, input, argsort, stable)
-            else:
-                sort_swapped(output, input, argsort, computed_axis, stable)
+        sort_swapped(output, input, argsort, sort_axis, stable)
 
 
 def _pack_keys(group: "list[DeviceArray]", indices: "DeviceArray | None") -> "DeviceArray":

@@ -189,20 +189,17 @@ class DeviceArray:
         result of sorting `rhs`."""
         from ._sort import sort_deferred
 
-        if kind == "stable":
-            stable = True
-        else:
-            stable = False
-
+        # (messages and exception types are the reference's: callers and its tests match on them)
         if order is not None:
             raise NotImplementedError(
                 "cuPyNumeric does not support sorting with 'order' as "
                 "ndarray only supports numeric values"
             )
-        if axis is not None and (axis >= rhs.ndim or axis < -rhs.ndim):
+        if axis is not None and not -rhs.ndim <= axis < rhs.ndim:
             raise ValueError("invalid axis")
-
-        sort_deferred(self, rhs, argsort, axis, stable)
+        # only "stable" sets the flag (any other kind, "mergesort" included, does not); every kernel
+        # here is stable whatever the flag says
+        sort_deferred(self, rhs, argsort, axis, stable=(kind == "stable"))
 
     def partition(
         self,
@@ -222,11 +219,9 @@ class DeviceArray:
                 "cuPyNumeric does not support partitioning with 'order' as "
                 "ndarray only supports numeric values"
             )
-        if axis is not None and (axis >= rhs.ndim or axis < -rhs.ndim):
+        if axis is not None and not -rhs.ndim <= axis < rhs.ndim:
             raise ValueError("invalid axis")
-
-        # fallback to sort for now
-        sort_deferred(self, rhs, argpartition, axis, False)
+        sort_deferred(self, rhs, argpartition, axis, False)  # a sorted row is partitioned at every kth
 
     def astype(self, dtype: Any) -> "DeviceArray":
         """Dense copy converted to `dtype` (`DeferredArray.convert`, `cupynumeric/_thunk/deferred.py:1899-1937`,
