@@ -37,6 +37,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <limits>
 #include <type_traits>
 
 #include "radix_common.h"
@@ -48,13 +49,8 @@ namespace cpn {
 __host__ __device__ constexpr int bucket_bins_log2(int tile) { return tile <= 1024 ? 12 : 13; }
 // Most keys a bin may hold for the split to be used (each key of a bin is compared with all others).
 constexpr uint32_t BUCKET_LIMIT = 24;
-// Bins are kept in 16-byte chunks whose index is XOR-swizzled, so that the scan, in which a thread
-// walks consecutive chunks of its own, spreads a wave over all LDS banks.
-__device__ __forceinline__ uint32_t bucket_word(uint32_t bin)
-{
-  const uint32_t chunk = bin >> 2;
-  return ((chunk ^ ((chunk >> 4) & 15u)) << 2) | (bin & 3u);
-}
+// Keys past the end of a bin that the walk over the bins may read (and not count).
+constexpr int BUCKET_PAD = 32;
 
 // The arithmetic type of a real key of 4 or 8 bytes.
 template <int CODEC, int BYTES>
@@ -112,7 +108,8 @@ void lds_row_sort_kernel(const KeyT* keys_in,
   constexpr int BINS_PER_THREAD = BINS / BLOCK;
   static_assert(!BUCKETS_OK || (BINS_PER_THREAD >= 4 && BINS_PER_THREAD % 4 == 0), "a thread scans whole 16-byte chunks");
 
-  __shared__ __align__(16) KeyT s_keys[TILE];
+  // (padded where the split is compiled in: its walk over a bin reads up to BUCKET_LIMIT keys past the bin's end)
+  __shared__ __align__(16) KeyT s_keys[TILE + (BUCKETS_OK ? BUCKET_PAD : 0)];
   __shared__ IdxS s_idx[HAS_IDX ? TILE : 1];
   // the per-wave digit counters of the radix passes and the bins of the split share their memory
   // (the split is over, or given up, before the first radix pass clears its counters)
@@ -147,11 +144,20 @@ void lds_row_sort_kernel(const KeyT* keys_in,
     all_and[n] = ~static_cast<SW>(0);
     all_or[n]  = 0;
   }
+  // (all loads first, from addresses that are inside the row whatever the lane holds, so that none
+  // of them sits behind a branch and waits for the one before it)
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t o = woff + i * WAVE;
+    key[i]           = KeyT{};
+    if (!BALANCE || full || i < static_cast<int>(rounds)) {  // uniform
+      key[i] = keys_in[base + (o < seg ? o : seg - 1)];
+    }
+  }
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t o = woff + i * WAVE;
     if (holds(i)) {
-      key[i] = keys_in[base + o];
       uint64_t w[NW];
       KT::words(key[i], w);
 #pragma unroll
@@ -261,22 +267,40 @@ void lds_row_sort_kernel(const KeyT* keys_in,
         __builtin_memcpy(&v, &k, sizeof(NT));
         return v;
       };
+      // (no NaN among the keys: the float minimum and maximum instructions order them like `<`)
+      auto lower = [](NT a, NT b) -> NT {
+        if constexpr (std::is_same<NT, float>::value) {
+          return __builtin_fminf(a, b);
+        } else if constexpr (std::is_same<NT, double>::value) {
+          return __builtin_fmin(a, b);
+        } else {
+          return a < b ? a : b;
+        }
+      };
+      auto upper = [](NT a, NT b) -> NT {
+        if constexpr (std::is_same<NT, float>::value) {
+          return __builtin_fmaxf(a, b);
+        } else if constexpr (std::is_same<NT, double>::value) {
+          return __builtin_fmax(a, b);
+        } else {
+          return a > b ? a : b;
+        }
+      };
       // smallest and largest key of the row (the row holds no NaN and no -0.0: the keys' own order
       // is the sort order), through the staging area, which is free until the keys are placed
-      NT lo = native(keys_in[base]), hi = lo;  // (a key of the row, whatever this lane holds)
+      NT lo = std::numeric_limits<NT>::max(), hi = std::numeric_limits<NT>::lowest();  // (lanes that hold no key)
 #pragma unroll
       for (int i = 0; i < ITEMS; ++i) {
         if (holds(i)) {
           const NT v = native(key[i]);
-          lo         = v < lo ? v : lo;
-          hi         = v > hi ? v : hi;
+          lo         = lower(v, lo);
+          hi         = upper(v, hi);
         }
       }
 #pragma unroll
       for (int d = 1; d < WAVE; d <<= 1) {
-        const NT a = __shfl_xor(lo, d, WAVE), b = __shfl_xor(hi, d, WAVE);
-        lo         = a < lo ? a : lo;
-        hi         = b > hi ? b : hi;
+        lo = lower(__shfl_xor(lo, d, WAVE), lo);
+        hi = upper(__shfl_xor(hi, d, WAVE), hi);
       }
       NT* s_ext = reinterpret_cast<NT*>(s_keys);
       if (lane == 0) {
@@ -288,9 +312,8 @@ void lds_row_sort_kernel(const KeyT* keys_in,
       }
       __syncthreads();
       for (int w = 0; w < WAVES; ++w) {
-        const NT a = s_ext[w], b = s_ext[WAVES + w];
-        lo         = a < lo ? a : lo;
-        hi         = b > hi ? b : hi;
+        lo = lower(s_ext[w], lo);
+        hi = upper(s_ext[w + WAVES], hi);
       }
       // The bin of a key: its place between the smallest and the largest key, in equal steps of the
       // value.  Float keys: subtraction of a constant, scaling and truncation never decrease with the
@@ -319,10 +342,17 @@ void lds_row_sort_kernel(const KeyT* keys_in,
           return static_cast<uint32_t>(static_cast<KeyT>(ordered_bits<CODEC, KeyT>(k) - img_lo) >> shift);
         }
       };
+      // (a partly filled tile: rounds in which no wave holds a key are skipped as a whole)
+      auto round_runs = [&](int i) -> bool { return !BALANCE || full || i < static_cast<int>(rounds); };
+      uint32_t bin[ITEMS];
 #pragma unroll
       for (int i = 0; i < ITEMS; ++i) {
-        if (holds(i)) {
-          atomicAdd(&s_bins[bucket_word(bin_of(key[i]))], 1u);
+        bin[i] = 0;
+        if (round_runs(i)) {  // uniform
+          bin[i] = bin_of(key[i]);
+          if (holds(i)) {
+            atomicAdd(&s_bins[bin[i]], 1u);
+          }
         }
       }
       __syncthreads();
@@ -331,7 +361,7 @@ void lds_row_sort_kernel(const KeyT* keys_in,
       uint32_t total = 0, largest = 0;
 #pragma unroll
       for (int c = 0; c < BINS_PER_THREAD / 4; ++c) {
-        const uint4 q4 = *reinterpret_cast<const uint4*>(&s_bins[bucket_word((tid * BINS_PER_THREAD) + 4 * c)]);
+        const uint4 q4 = *reinterpret_cast<const uint4*>(&s_bins[tid * BINS_PER_THREAD + 4 * c]);
         cnt[4 * c] = q4.x, cnt[4 * c + 1] = q4.y, cnt[4 * c + 2] = q4.z, cnt[4 * c + 3] = q4.w;
       }
 #pragma unroll
@@ -357,73 +387,87 @@ void lds_row_sort_kernel(const KeyT* keys_in,
             e[j] = run;
             run += cnt[4 * c + j];
           }
-          *reinterpret_cast<uint4*>(&s_bins[bucket_word((tid * BINS_PER_THREAD) + 4 * c)]) = make_uint4(e[0], e[1], e[2], e[3]);
+          *reinterpret_cast<uint4*>(&s_bins[tid * BINS_PER_THREAD + 4 * c]) = make_uint4(e[0], e[1], e[2], e[3]);
         }
         __syncthreads();
         // every key into its bin, in whatever order the atomics hand out
+        uint32_t self[ITEMS];  // where this thread's key i went
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {
-          if (holds(i)) {
-            const uint32_t pos = atomicAdd(&s_bins[bucket_word(bin_of(key[i]))], 1u);
-            s_keys[pos]        = key[i];
+          self[i] = 0;
+          if (round_runs(i) && holds(i)) {
+            self[i]         = atomicAdd(&s_bins[bin[i]], 1u);
+            s_keys[self[i]] = key[i];
           }
         }
         __syncthreads();
-        // Each bin now ends where its counter stands and starts where the bin before it ends.  The
-        // key at position p of the row goes to the start of its bin plus the number of keys of the
-        // bin that come before it: smaller ones, and equal ones at lower positions (equal keys are
-        // the same bits here, the rule only keeps the places distinct).
-        // (All keys of a thread walk their bins in step, so that every round has ITEMS independent
-        // LDS reads in flight instead of one.)
-        uint32_t place[ITEMS], len[ITEMS];
-        uint32_t longest = 0;
+        // Each bin now ends where its counter stands and starts where the bin before it ends.  A key
+        // goes to the start of its bin plus the number of keys of the bin that come before it: smaller
+        // ones, and equal ones that the atomics placed earlier (equal keys are the same bits here, the
+        // rule only keeps the places distinct).
+        // (Eight keys of a thread walk their bins in step, so that every round has eight independent
+        // LDS reads in flight instead of one; a read past the end of a bin fetches a key of a later
+        // bin, or of the padding, and is not counted.  Eight at a time, not all: the walk's state for
+        // 16 keys does not fit the registers of a 1024-thread workgroup.)
+        constexpr int GROUP = ITEMS < 8 ? ITEMS : 8;
+        static_assert(ITEMS % GROUP == 0, "whole groups");
 #pragma unroll
-        for (int i = 0; i < ITEMS; ++i) {
-          place[i] = 0, len[i] = 0;
-          if (holds(i)) {
-            key[i] = s_keys[woff + i * WAVE];
+        for (int g = 0; g < ITEMS; g += GROUP) {
+          if (!round_runs(g)) {
+            continue;  // uniform: no wave holds a key of this group
           }
-        }
+          uint32_t from[GROUP], len[GROUP], before[GROUP];
+          uint32_t longest = 0;
 #pragma unroll
-        for (int i = 0; i < ITEMS; ++i) {
-          if (holds(i)) {
-            const uint32_t b   = bin_of(key[i]);
-            const uint32_t end = s_bins[bucket_word(b)];
-            place[i]           = (b == 0) ? 0u : s_bins[bucket_word(b - 1)];  // start of the bin
-            len[i]             = end - place[i];
-            longest            = len[i] > longest ? len[i] : longest;
+          for (int k = 0; k < GROUP; ++k) {
+            const int i = g + k;
+            from[k] = 0, len[k] = 0, before[k] = 0;
+            if (round_runs(i) && holds(i)) {
+              const uint32_t end = s_bins[bin[i]];
+              from[k]            = (bin[i] == 0) ? 0u : s_bins[bin[i] - 1];  // start of the bin
+              len[k]             = end - from[k];
+              self[i] -= from[k];
+              longest = len[k] > longest ? len[k] : longest;
+            }
           }
-        }
-        uint32_t before[ITEMS];
+          // (two copies of the loop: a group whose every round runs pays no per-round checks)
+          auto walk = [&](auto every_round) {
+            for (uint32_t j = 0; j < longest; ++j) {
+              KeyT other[GROUP];
 #pragma unroll
-        for (int i = 0; i < ITEMS; ++i) {
-          before[i] = 0;
-        }
-        for (uint32_t j = 0; j < longest; ++j) {
-          // (reads past the end of a bin are clamped to its start and not counted: no branch, so the
-          // reads of a round are issued together)
-          KeyT other[ITEMS];
+              for (int k = 0; k < GROUP; ++k) {
+                if (!decltype(every_round)::value && !round_runs(g + k)) {
+                  break;
+                }
+                other[k] = s_keys[from[k] + j];
+              }
 #pragma unroll
-          for (int i = 0; i < ITEMS; ++i) {
-            other[i] = s_keys[place[i] + (j < len[i] ? j : 0u)];
+              for (int k = 0; k < GROUP; ++k) {
+                if (!decltype(every_round)::value && !round_runs(g + k)) {
+                  break;
+                }
+                const NT a = native(other[k]), b = native(key[g + k]);
+                // (bitwise, not short-circuit: no branch between the reads of a round)
+                const bool first = (a < b) | ((a == b) & (j < self[g + k]));
+                before[k] += (first & (j < len[k])) ? 1u : 0u;
+              }
+            }
+          };
+          if (round_runs(g + GROUP - 1)) {
+            walk(std::true_type{});
+          } else {
+            walk(std::false_type{});
           }
 #pragma unroll
-          for (int i = 0; i < ITEMS; ++i) {
-            const uint32_t at = place[i] + j;
-            const NT a = native(other[i]), b = native(key[i]);
-            const bool first = a < b || (a == b && at < woff + i * WAVE);
-            before[i] += (j < len[i] && first) ? 1u : 0u;
+          for (int k = 0; k < GROUP; ++k) {
+            self[g + k] = from[k] + before[k];  // where the key belongs
           }
-        }
-#pragma unroll
-        for (int i = 0; i < ITEMS; ++i) {
-          place[i] += before[i];
         }
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {
-          if (holds(i)) {
-            s_keys[place[i]] = key[i];
+          if (round_runs(i) && holds(i)) {
+            s_keys[self[i]] = key[i];
           }
         }
         __syncthreads();

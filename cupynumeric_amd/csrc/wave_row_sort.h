@@ -167,11 +167,19 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
     vary_and[n] = 0xFFFFFFFFu;
     vary_or[n]  = 0;
   }
+  // (all loads first, from addresses that are inside the row whatever the lane holds, so that none
+  // of them sits behind a branch and waits for the one before it)
+  KeyT loaded[ITEMS];
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t o = i * WAVE + lane;
+    loaded[i]        = keys_in[base + (o < seg ? o : seg - 1)];
+  }
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t o = i * WAVE + lane;
     if (full || o < seg) {
-      const KeyT raw = keys_in[base + o];
+      const KeyT raw = loaded[i];
       OW::encode(raw, w[i]);
 #pragma unroll
       for (int n = 0; n < NW; ++n) {
@@ -286,10 +294,12 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
         reinterpret_cast<uint4*>(ctr)[j * WAVE + lane] = make_uint4(0u, 0u, 0u, 0u);
       }
       __builtin_amdgcn_wave_barrier();
+      uint32_t bin[ITEMS];
 #pragma unroll
       for (int i = 0; i < ITEMS; ++i) {
+        bin[i] = bin_of(w[i][0]);
         if (full || (i * WAVE + lane < seg)) {
-          atomicAdd(&ctr[bin_of(w[i][0])], 1u);
+          atomicAdd(&ctr[bin[i]], 1u);
         }
       }
       __builtin_amdgcn_wave_barrier();
@@ -311,49 +321,52 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
         }
         __builtin_amdgcn_wave_barrier();
         // every key into its range, in whatever order the atomics hand out
+        uint32_t self[ITEMS];  // where this lane's key i went
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {
+          self[i] = 0;
           if (full || (i * WAVE + lane < seg)) {
-            const uint32_t p    = atomicAdd(&ctr[bin_of(w[i][0])], 1u);
-            s_words[wave][0][p] = w[i][0];
+            self[i]                   = atomicAdd(&ctr[bin[i]], 1u);
+            s_words[wave][0][self[i]] = w[i][0];
           }
         }
         __builtin_amdgcn_wave_barrier();
-        // A range now ends where its counter stands and starts where the range before it ends.  The
-        // key at position p goes to the start of its range plus the number of keys of the range that
-        // come before it: smaller ones, and equal ones at lower positions (equal keys are the same
-        // bits here; the rule only keeps the places distinct).  All keys of a lane walk in step.
-        uint32_t place[ITEMS], len[ITEMS], before[ITEMS];
+        // A range now ends where its counter stands and starts where the range before it ends.  A
+        // key goes to the start of its range plus the number of keys of the range that come before
+        // it: smaller ones, and equal ones that the atomics placed earlier (equal keys are the same
+        // bits here; the rule only keeps the places distinct).  All keys of a lane walk in step; a
+        // read past the end of a range fetches a key of a later range and is not counted.
+        uint32_t from[ITEMS], len[ITEMS], before[ITEMS];
         uint32_t longest = 0;
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {
-          place[i] = 0, len[i] = 0, before[i] = 0;
+          from[i] = 0, len[i] = 0, before[i] = 0;
           if (full || (i * WAVE + lane < seg)) {
-            w[i][0]          = s_words[wave][0][i * WAVE + lane];
-            const uint32_t b = bin_of(w[i][0]);
-            place[i]         = (b == 0) ? 0u : ctr[b - 1];
-            len[i]           = ctr[b] - place[i];
-            longest          = len[i] > longest ? len[i] : longest;
+            from[i] = (bin[i] == 0) ? 0u : ctr[bin[i] - 1];
+            len[i]  = ctr[bin[i]] - from[i];
+            self[i] -= from[i];
+            longest = len[i] > longest ? len[i] : longest;
           }
         }
         for (uint32_t j = 0; j < longest; ++j) {
           uint32_t other[ITEMS];
 #pragma unroll
           for (int i = 0; i < ITEMS; ++i) {
-            other[i] = s_words[wave][0][place[i] + (j < len[i] ? j : 0u)];
+            const uint32_t at = from[i] + j;
+            other[i]          = s_words[wave][0][at < static_cast<uint32_t>(TILE) ? at : static_cast<uint32_t>(TILE - 1)];
           }
 #pragma unroll
           for (int i = 0; i < ITEMS; ++i) {
-            const uint32_t at = place[i] + j;
-            const bool first  = other[i] < w[i][0] || (other[i] == w[i][0] && at < static_cast<uint32_t>(i * WAVE + lane));
-            before[i] += (j < len[i] && first) ? 1u : 0u;
+            // (bitwise, not short-circuit: no branch between the reads of a round)
+            const bool first = (other[i] < w[i][0]) | ((other[i] == w[i][0]) & (j < self[i]));
+            before[i] += (first & (j < len[i])) ? 1u : 0u;
           }
         }
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {
           if (full || (i * WAVE + lane < seg)) {
-            s_words[wave][0][place[i] + before[i]] = w[i][0];
+            s_words[wave][0][from[i] + before[i]] = w[i][0];
           }
         }
         __builtin_amdgcn_wave_barrier();
