@@ -86,6 +86,26 @@ __host__ __device__ __forceinline__ U sign_unflip(U image)
   return (image & sign) ? static_cast<U>(image ^ sign) : static_cast<U>(~image);
 }
 
+// Is the float with these bits a NaN or -0.0: the two kinds of key whose image is shared with keys
+// of other bits.  One class-test instruction for 4- and 8-byte floats.
+template <typename U>
+__device__ __forceinline__ bool is_nan_or_negative_zero(U raw)
+{
+  constexpr int CLASS_SNAN = 1, CLASS_QNAN = 2, CLASS_NEG_ZERO = 32;  // bits of the class mask
+  if constexpr (sizeof(U) == 4) {
+    float v;
+    __builtin_memcpy(&v, &raw, 4);
+    return __builtin_amdgcn_classf(v, CLASS_SNAN | CLASS_QNAN | CLASS_NEG_ZERO);
+  } else if constexpr (sizeof(U) == 8) {
+    double v;
+    __builtin_memcpy(&v, &raw, 8);
+    return __builtin_amdgcn_class(v, CLASS_SNAN | CLASS_QNAN | CLASS_NEG_ZERO);
+  } else {
+    constexpr U sign = FloatLayout<U>::sign;
+    return static_cast<U>(raw & static_cast<U>(~sign)) > FloatLayout<U>::inf || raw == sign;
+  }
+}
+
 template <int CODEC, typename U>
 __host__ __device__ __forceinline__ uint32_t radix_digit(U raw, int shift)
 {

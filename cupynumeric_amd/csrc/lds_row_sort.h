@@ -102,6 +102,7 @@ void lds_row_sort_kernel(const KeyT* keys_in,
   // (only the 1024-thread shapes, rows of more than 4096 keys: in the smaller shapes the bins cost
   // the LDS that lets many workgroups share a CU, and rows of 1024 float64 keys went from 0.41 to 0.60 ms)
   constexpr bool BUCKETS_OK = !HAS_IDX && NW == 1 && sizeof(KeyT) >= 4 && sizeof(KeyT) <= 8 && BLOCK == 1024 &&
+                              BLOCK * ITEMS * sizeof(KeyT) <= 64 * 1024 &&  // (the bins take 32 KiB beside the keys)
                               (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT);
   constexpr int BINS_LOG2   = bucket_bins_log2(TILE);
   constexpr int BINS        = 1 << BINS_LOG2;
@@ -137,13 +138,6 @@ void lds_row_sort_kernel(const KeyT* keys_in,
 
   KeyT key[ITEMS];
   uint32_t idx[HAS_IDX ? ITEMS : 1];
-  SW all_and[NW], all_or[NW];
-  int special = 0;  // float keys: the row holds a NaN or a -0.0
-#pragma unroll
-  for (int n = 0; n < NW; ++n) {
-    all_and[n] = ~static_cast<SW>(0);
-    all_or[n]  = 0;
-  }
   // (all loads first, from addresses that are inside the row whatever the lane holds, so that none
   // of them sits behind a branch and waits for the one before it)
 #pragma unroll
@@ -153,33 +147,64 @@ void lds_row_sort_kernel(const KeyT* keys_in,
     if (!BALANCE || full || i < static_cast<int>(rounds)) {  // uniform
       key[i] = keys_in[base + (o < seg ? o : seg - 1)];
     }
-  }
-#pragma unroll
-  for (int i = 0; i < ITEMS; ++i) {
-    const uint32_t o = woff + i * WAVE;
-    if (holds(i)) {
-      uint64_t w[NW];
-      KT::words(key[i], w);
-#pragma unroll
-      for (int n = 0; n < NW; ++n) {
-        all_and[n] &= w[n];
-        all_or[n] |= w[n];
-      }
-      if constexpr (CODEC == CODEC_FLOAT) {
-        special |= (static_cast<KeyT>(w[0]) != sign_flip(key[i])) ? 1 : 0;
-      }
-    } else {
-      key[i] = KeyT{};
-    }
     if constexpr (HAS_IDX) {
       idx[i] = o;
     }
   }
-  // bits on which the keys of the row differ
+  // ---- bits on which the keys of the row differ (passes on the other digits are skipped), and for
+  //      float keys whether the row holds a NaN or a -0.0 ----
+  // Real keys: taken from the keys' own bits.  The ordered image of a signed integer, and of a float
+  // row whose keys share one sign and hold no NaN and no -0.0, is the key XOR a constant, so it varies
+  // in the same bits; any other float row is taken to vary in every bit (it nearly always does: the
+  // images of its negative keys are complemented).  Complex keys: from the words of the image.
+  constexpr bool RAW_BITS = (NW == 1) && (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT);
+  SW all_and[NW], all_or[NW];
+  int special = 0;  // float keys: the row holds a NaN or a -0.0
 #pragma unroll
   for (int n = 0; n < NW; ++n) {
-    all_and[n] = wave_all_and(all_and[n]);
-    all_or[n]  = wave_all_or(all_or[n]);
+    all_and[n] = ~static_cast<SW>(0);
+    all_or[n]  = 0;
+  }
+  if constexpr (RAW_BITS) {
+    KeyT bits_and = static_cast<KeyT>(~static_cast<KeyT>(0)), bits_or = 0;
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      if (holds(i)) {
+        bits_and &= key[i];
+        bits_or |= key[i];
+        if constexpr (CODEC == CODEC_FLOAT) {
+          special |= is_nan_or_negative_zero(key[i]) ? 1 : 0;
+        }
+      } else {
+        key[i] = KeyT{};
+      }
+    }
+    all_and[0] = static_cast<SW>(bits_and);
+    all_or[0]  = static_cast<SW>(bits_or);
+  } else {
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      if (holds(i)) {
+        uint64_t w[NW];
+        KT::words(key[i], w);
+#pragma unroll
+        for (int n = 0; n < NW; ++n) {
+          all_and[n] &= w[n];
+          all_or[n] |= w[n];
+        }
+        if constexpr (CODEC == CODEC_FLOAT) {
+          special |= (static_cast<KeyT>(w[0]) != sign_flip(key[i])) ? 1 : 0;
+        }
+      } else {
+        key[i] = KeyT{};
+      }
+    }
+  }
+  using RedT = typename std::conditional<(sizeof(KeyT) <= 4 && NW == 1), uint32_t, SW>::type;  // the half that can be set
+#pragma unroll
+  for (int n = 0; n < NW; ++n) {
+    all_and[n] = wave_reduce_and_dpp(static_cast<RedT>(all_and[n]));
+    all_or[n]  = wave_reduce_or_dpp(static_cast<RedT>(all_or[n]));
     if (lane == 0) {
       s_red[(2 * wave) * NW + n]     = all_and[n];
       s_red[(2 * wave + 1) * NW + n] = all_or[n];
@@ -198,13 +223,26 @@ void lds_row_sort_kernel(const KeyT* keys_in,
   SW varying[NW];
 #pragma unroll
   for (int n = 0; n < NW; ++n) {
-    SW a = s_red[n], o = s_red[NW + n];
+    SW a, o;
+    if constexpr (WAVES >= 8) {
+      // every lane takes the words of one wave; AND and OR do not mind seeing a wave several times
+      a = wave_reduce_and_dpp(static_cast<RedT>(s_red[(2 * (lane % WAVES)) * NW + n]));
+      o = wave_reduce_or_dpp(static_cast<RedT>(s_red[(2 * (lane % WAVES) + 1) * NW + n]));
+    } else {
+      a = s_red[n], o = s_red[NW + n];
 #pragma unroll
-    for (int w = 1; w < WAVES; ++w) {
-      a &= s_red[(2 * w) * NW + n];
-      o |= s_red[(2 * w + 1) * NW + n];
+      for (int w = 1; w < WAVES; ++w) {
+        a &= s_red[(2 * w) * NW + n];
+        o |= s_red[(2 * w + 1) * NW + n];
+      }
     }
     varying[n] = a ^ o;
+  }
+  if constexpr (RAW_BITS && CODEC == CODEC_FLOAT) {
+    constexpr SW SIGN = static_cast<SW>(1) << (8 * sizeof(KeyT) - 1);
+    if (any_special != 0 || (varying[0] & SIGN) != 0) {
+      varying[0] = ~static_cast<SW>(0);
+    }
   }
   uint32_t active = 0;  // bit p: the keys of the row differ in digit p
 #pragma unroll
@@ -311,9 +349,15 @@ void lds_row_sort_kernel(const KeyT* keys_in,
         reinterpret_cast<uint4*>(s_bins)[j] = make_uint4(0u, 0u, 0u, 0u);
       }
       __syncthreads();
-      for (int w = 0; w < WAVES; ++w) {
-        lo = lower(s_ext[w], lo);
-        hi = upper(s_ext[w + WAVES], hi);
+      // (every lane takes the extremes of one wave, four exchanges inside each group of 16 lanes
+      // merge them; minimum and maximum do not mind seeing a wave several times)
+      static_assert(WAVES == 16, "one wave per lane of a 16-lane group");
+      lo = s_ext[lane % WAVES];
+      hi = s_ext[WAVES + lane % WAVES];
+#pragma unroll
+      for (int d = 1; d < WAVES; d <<= 1) {
+        lo = lower(__shfl_xor(lo, d, WAVE), lo);
+        hi = upper(__shfl_xor(hi, d, WAVE), hi);
       }
       // The bin of a key: its place between the smallest and the largest key, in equal steps of the
       // value.  Float keys: subtraction of a constant, scaling and truncation never decrease with the

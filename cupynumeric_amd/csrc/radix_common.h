@@ -101,6 +101,51 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan_dpp_impl(uint32_t v)
 __device__ __forceinline__ uint32_t wave_inclusive_sum_dpp(uint32_t v) { return wave_inclusive_scan_dpp_impl<false>(v); }
 __device__ __forceinline__ uint32_t wave_inclusive_max_dpp(uint32_t v) { return wave_inclusive_scan_dpp_impl<true>(v); }
 
+// AND / OR of one 32-bit value per lane over the whole wave, through the same DPP steps (lanes
+// without a source keep the identity); the result is read from the last lane and is uniform.
+template <bool IS_AND>
+__device__ __forceinline__ uint32_t wave_reduce_bits_dpp(uint32_t v)
+{
+  constexpr int ID = IS_AND ? -1 : 0;
+  auto combine     = [](uint32_t a, uint32_t b) -> uint32_t { return IS_AND ? (a & b) : (a | b); };
+  uint32_t t       = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(ID, static_cast<int>(v), 0x111, 0xF, 0xF, false));
+  v                = combine(v, t);
+  t                = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(ID, static_cast<int>(v), 0x112, 0xF, 0xF, false));
+  v                = combine(v, t);
+  t                = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(ID, static_cast<int>(v), 0x114, 0xF, 0xF, false));
+  v                = combine(v, t);
+  t                = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(ID, static_cast<int>(v), 0x118, 0xF, 0xF, false));
+  v                = combine(v, t);
+  t                = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(ID, static_cast<int>(v), 0x142, 0xA, 0xF, false));
+  v                = combine(v, t);
+  t                = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(ID, static_cast<int>(v), 0x143, 0xC, 0xF, false));
+  v                = combine(v, t);
+  return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), WAVE - 1));
+}
+// (any unsigned type of 4 or 8 bytes; the halves of a 64-bit value are reduced on their own)
+template <bool IS_AND, typename T>
+__device__ __forceinline__ T wave_reduce_bits(T v)
+{
+  static_assert(sizeof(T) == 4 || sizeof(T) == 8, "32- or 64-bit values");
+  if constexpr (sizeof(T) == 4) {
+    return static_cast<T>(wave_reduce_bits_dpp<IS_AND>(static_cast<uint32_t>(v)));
+  } else {
+    const uint32_t hi = wave_reduce_bits_dpp<IS_AND>(static_cast<uint32_t>(static_cast<uint64_t>(v) >> 32));
+    const uint32_t lo = wave_reduce_bits_dpp<IS_AND>(static_cast<uint32_t>(v));
+    return static_cast<T>((static_cast<uint64_t>(hi) << 32) | lo);
+  }
+}
+template <typename T>
+__device__ __forceinline__ T wave_reduce_and_dpp(T v)
+{
+  return wave_reduce_bits<true, T>(v);
+}
+template <typename T>
+__device__ __forceinline__ T wave_reduce_or_dpp(T v)
+{
+  return wave_reduce_bits<false, T>(v);
+}
+
 // How the 256 digits of a tile are spread over the threads that scan them.
 template <int BLOCK>
 struct DigitThreads {

@@ -80,10 +80,10 @@ uint64_t wave_row_limit()
   return limit < 0 ? 0 : (limit > 1024 ? 1024 : static_cast<uint64_t>(limit));
 }
 
-uint64_t lds_row_limit(int key_bytes)
+uint64_t lds_row_limit(int key_bytes, bool with_positions)
 {
   const long long limit = g_lds_row_limit.load(std::memory_order_relaxed);
-  const uint64_t cap    = lds_row_capacity(key_bytes);
+  const uint64_t cap    = lds_row_capacity(key_bytes, with_positions);
   if (limit >= 0 && static_cast<uint64_t>(limit) < cap) {
     return static_cast<uint64_t>(limit);
   }

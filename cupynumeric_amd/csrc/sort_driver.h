@@ -89,8 +89,11 @@ __host__ __device__ constexpr int global_tile(int key_bytes, bool big)
 
 // Longest row the LDS kernel can take, per key width: 1024 threads with the row in 64 KiB of LDS
 // (plus staged row positions and the per-wave digit counters, 112 KiB at most of the CU's 160).
-__host__ __device__ constexpr uint64_t lds_row_capacity(int key_bytes)
+// (8-byte keys: 12 and 16 per thread would fit the LDS without positions, but not the 128 vector
+// registers a thread of a 1024-thread workgroup can have: the compiler spills 0.7 to 1.5 KiB per thread.)
+__host__ __device__ constexpr uint64_t lds_row_capacity(int key_bytes, bool with_positions)
 {
+  (void)with_positions;
   return key_bytes == 16 ? 4096 : (key_bytes == 8 ? 8192 : 16384);
 }
 // Radix passes of a key: one per byte, plus the NaN-class pass of complex keys.
@@ -111,7 +114,7 @@ uint64_t count16_min_row();
 // Row length up to which the LDS kernel is used.  Equals lds_row_capacity unless the
 // environment variable CPN_SORT_LDS_ROW_LIMIT or cpn_set_lds_row_limit lowers it, e.g. to 0
 // to send every request down the global path for an A/B run.
-uint64_t lds_row_limit(int key_bytes);
+uint64_t lds_row_limit(int key_bytes, bool with_positions);
 
 // Element type code (enum cpn_dtype) -> key width and codec.
 struct KeyKind {
@@ -227,7 +230,7 @@ inline GlobalLayout global_layout(int key_bytes, int passes, uint64_t volume, ui
 inline uint64_t workspace_bytes(int key_bytes, int passes, uint64_t volume, uint64_t seg, bool want_values,
                                 bool want_indices, bool in_place)
 {
-  if (volume == 0 || seg <= lds_row_limit(key_bytes)) {
+  if (volume == 0 || seg <= lds_row_limit(key_bytes, want_indices)) {
     return HEADER_BYTES;
   }
   const GlobalLayout L = global_layout(key_bytes, passes, volume, seg, want_values, want_indices, in_place);
@@ -410,7 +413,7 @@ inline int sort_rows_in_lds(const SortRequest& r)
       }
     }
     if constexpr (sizeof(KeyT) == 8) {
-      return launch_lds_rows<KeyT, CODEC, HAS_IDX, 1024, 8>(r);  // lds_row_capacity(8) == 8192
+      return launch_lds_rows<KeyT, CODEC, HAS_IDX, 1024, 8>(r);  // lds_row_capacity(8, ...) == 8192
     } else {
       if (r.seg <= 8192) {
         // sixteen waves of eight keys hide the ranking latency better than eight waves of sixteen
@@ -660,7 +663,7 @@ int sort_typed(const SortRequest& r)
   if (r.temp == nullptr || r.temp_bytes < need || (reinterpret_cast<uintptr_t>(r.temp) % WORKSPACE_ALIGN) != 0) {
     return CPN_ERR_TEMP;
   }
-  if (r.seg <= lds_row_limit(KB)) {
+  if (r.seg <= lds_row_limit(KB, has_idx)) {
     // one launch: the row kernels clear the status word of the workspace themselves.  (More rows than a
     // grid can have blocks, e.g. a (2^31, 1) array: one launch per 2^30 rows.)
     constexpr uint64_t ROWS_PER_LAUNCH = 1ull << 30;

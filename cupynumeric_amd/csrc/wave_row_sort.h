@@ -187,7 +187,7 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
         vary_or[n] |= w[i][n];
       }
       if constexpr (CODEC == CODEC_FLOAT && !HAS_IDX) {
-        special = special || (ordered_bits<CODEC_FLOAT, KeyT>(raw) != sign_flip(raw));
+        special = special | is_nan_or_negative_zero(raw);
       }
     } else {
 #pragma unroll
