@@ -138,15 +138,14 @@ void lds_row_sort_kernel(const KeyT* keys_in,
 
   KeyT key[ITEMS];
   uint32_t idx[HAS_IDX ? ITEMS : 1];
-  // (all loads first, from addresses that are inside the row whatever the lane holds, so that none
-  // of them sits behind a branch and waits for the one before it)
+  // (all loads first, from offsets that are inside the row whatever the lane holds, so that none of
+  // them sits behind a branch and waits for the one before it; one uniform row pointer and 32-bit
+  // offsets, so that the addresses of 16 loads in flight do not take 32 registers)
+  const KeyT* const row_in = keys_in + base;
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t o = woff + i * WAVE;
-    key[i]           = KeyT{};
-    if (!BALANCE || full || i < static_cast<int>(rounds)) {  // uniform
-      key[i] = keys_in[base + (o < seg ? o : seg - 1)];
-    }
+    key[i]           = row_in[o < seg ? o : seg - 1];
     if constexpr (HAS_IDX) {
       idx[i] = o;
     }
