@@ -9,6 +9,7 @@ from __future__ import annotations
 
 import argparse
 import concurrent.futures as cf
+import json
 import os
 import shutil
 import subprocess
@@ -46,7 +47,16 @@ HIPCC_FLAGS = [
     "-Wno-unused-function",
     # packed fp32 instructions are kept out of every kernel of this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # per-kernel registers, scratch and LDS as compiler remarks: collected into
+    # csrc/_obj/<unit>.resources.json and checked below
+    "-Rpass-analysis=kernel-resource-usage",
 ]
+
+# Scratch memory (bytes per lane) a kernel may use.  The per-row kernels keep a whole row in
+# registers; one that spills runs several times slower without failing any test (a 16-keys-per-
+# thread shape once spilled 516 bytes per lane and took 3.3 ms instead of 0.8), so the build
+# refuses it.  The scatter pass of the global sort is allowed the few words it is known to park.
+SCRATCH_LIMITS = (("row_sort_kernel", 0), ("count16_", 0), ("onesweep_kernel", 32))
 
 
 def hipcc_path() -> str:
@@ -74,12 +84,61 @@ def _compile(src: str, force: bool, extra: list[str]) -> str:
     cmd = [hipcc_path(), *HIPCC_FLAGS, *extra, "-c", str(src_path), "-o", str(obj)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     # the host pass warns that it does not know the packed-fp32 feature; that is harmless
-    err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
+    lines = [l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l]
+    resources, lines = _split_resource_remarks(lines)
+    err = "\n".join(lines)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{err}")
     if err.strip():
         sys.stderr.write(err + "\n")
+    (OBJ_DIR / (Path(src).stem + ".resources.json")).write_text(json.dumps(resources, indent=1))
+    for kernel, use in resources.items():
+        for pattern, limit in SCRATCH_LIMITS:
+            if pattern in kernel and use.get("scratch_bytes_per_lane", 0) > limit:
+                obj.unlink(missing_ok=True)
+                raise RuntimeError(
+                    f"{src}: kernel {kernel} spills {use['scratch_bytes_per_lane']} bytes per lane "
+                    f"(limit {limit}); see SCRATCH_LIMITS in {Path(__file__).name}"
+                )
     return str(obj)
+
+
+_REMARK = "[-Rpass-analysis=kernel-resource-usage]"
+_FIELDS = {
+    "TotalSGPRs": "sgprs",
+    "VGPRs": "vgprs",
+    "ScratchSize [bytes/lane]": "scratch_bytes_per_lane",
+    "Occupancy [waves/SIMD]": "waves_per_simd",
+    "VGPRs Spill": "vgpr_spills",
+    "LDS Size [bytes/block]": "lds_bytes",
+}
+
+
+def _split_resource_remarks(lines: list[str]) -> tuple[dict[str, dict[str, int]], list[str]]:
+    """Take the compiler's per-kernel resource remarks (and the source excerpts printed under
+    them) out of `lines`; returns ({mangled kernel name: figures}, the other lines)."""
+    resources: dict[str, dict[str, int]] = {}
+    rest: list[str] = []
+    current: dict[str, int] | None = None
+    skip = 0
+    for line in lines:
+        if _REMARK in line:
+            text = line.split("remark:", 1)[1].replace(_REMARK, "").strip()
+            key, _, value = text.partition(":")
+            key, value = key.strip(), value.strip()
+            if key == "Function Name":
+                current = resources.setdefault(value, {})
+            elif current is not None and key in _FIELDS and value.lstrip("-").isdigit():
+                current[_FIELDS[key]] = int(value)
+            skip = 2  # the quoted source line and its caret
+        elif skip and (line.lstrip().startswith("|") or line.lstrip()[:1].isdigit()):
+            skip -= 1
+        elif line.startswith("In file included from") or "remarks generated" in line or "remark generated" in line:
+            continue
+        else:
+            skip = 0
+            rest.append(line)
+    return resources, rest
 
 
 def build(force: bool = True, jobs: int | None = None, extra_flags: list[str] | None = None) -> Path:

@@ -211,3 +211,49 @@ def test_missing_library_is_an_error(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "libcpnsort.so")
     with pytest.raises(_lib.NativeLibraryError, match="no CPU fallback"):
         _lib.load()
+
+
+def test_resource_remarks_are_parsed():
+    from cupynumeric_amd import build as B
+
+    tag = "[-Rpass-analysis=kernel-resource-usage]"
+    lines = [
+        "In file included from a.hip:1:",
+        f"./k.h:83:1: remark: Function Name: _Zkernel_a {tag}",
+        "   83 | {",
+        "      | ^",
+        f"./k.h:83:1: remark:     VGPRs: 59 {tag}",
+        "   83 | {",
+        "      | ^",
+        f"./k.h:83:1: remark:     ScratchSize [bytes/lane]: 516 {tag}",
+        "   83 | {",
+        "      | ^",
+        f"./k.h:83:1: remark:     LDS Size [bytes/block]: 10536 {tag}",
+        "   83 | {",
+        "      | ^",
+        "a.hip:7:3: warning: something else",
+        "11 remarks generated when compiling for gfx950.",
+    ]
+    resources, rest = B._split_resource_remarks(lines)
+    assert resources == {"_Zkernel_a": {"vgprs": 59, "scratch_bytes_per_lane": 516, "lds_bytes": 10536}}
+    assert rest == ["a.hip:7:3: warning: something else"]
+
+
+def test_built_row_kernels_do_not_spill():
+    """A row kernel that spills still sorts correctly, several times slower: the build refuses
+    it, and this test reads the reports of the build that produced the library under test."""
+    import json
+
+    from cupynumeric_amd import build as B
+
+    reports = sorted(B.OBJ_DIR.glob("*.resources.json"))
+    if not reports:
+        pytest.skip("no resource reports beside the objects (library built elsewhere)")
+    seen_row_kernels = 0
+    for report in reports:
+        for kernel, use in json.loads(report.read_text()).items():
+            for pattern, limit in B.SCRATCH_LIMITS:
+                if pattern in kernel:
+                    seen_row_kernels += pattern != "onesweep_kernel"
+                    assert use.get("scratch_bytes_per_lane", 0) <= limit, (report.name, kernel, use)
+    assert seen_row_kernels > 100  # the row kernels of five key widths were all looked at
