@@ -103,7 +103,60 @@ def make_config(name: str, log2n: int | None = None, rows: int | None = None) ->
         return dict(name=name, x=x, op="sort", axis=-1,
                     workload=f"sort-2D-{name}: np.sort float32 {shape} last axis, uniform [0,1), seed "
                              f"{8 if name == 'flat' else 9} (the reference's sort_bench.py shape at s=2^{int(math.log2(s_total))})")
+    if name.startswith("rows:"):
+        # rows:<dtype>:<rows>:<row length>:<sort|argsort> -- batched rows of any length, e.g. on either
+        # side of the row length at which the library changes kernels
+        _, dt, r, seg, op = name.split(":")
+        r, seg, dtype = int(r), int(seg), np.dtype(dt)
+        rng = np.random.default_rng(10)
+        if dtype == np.float64:
+            x = rng.random((r, seg))
+        elif dtype.kind == "f":
+            x = rng.standard_normal((r, seg), dtype=np.float32).astype(dtype)
+        else:
+            info = np.iinfo(dtype)
+            x = rng.integers(info.min, info.max, size=(r, seg), dtype=dtype, endpoint=True)
+        if op not in ("sort", "argsort"):
+            raise ValueError(f"rows config: op must be sort or argsort, not {op}")
+        return dict(name=name, x=x, op=op, axis=-1,
+                    workload=f"np.{op} {dtype.name} ({r},{seg}) last axis, "
+                             f"{'uniform [0,1)' if dtype == np.float64 else 'normal' if dtype.kind == 'f' else 'uniform'}, seed 10")
     raise ValueError(f"unknown config {name}")
+
+
+# Row lengths on either side of every length at which the library changes kernels (--edges): key type,
+# operation, lengths whose successor is timed too; 2^26 keys per run.
+EDGE_LENGTHS = (
+    ("float32", "sort", (32, 1024, 2048, 4096, 8192, 16384)),
+    ("float64", "sort", (512, 2048, 4096, 8192)),
+    ("float16", "sort", (4096, 8192, 16384)),
+    ("float32", "argsort", (4096, 8192, 16384)),
+    ("float64", "argsort", (4096, 8192)),
+)
+
+
+def run_edges() -> dict:
+    """Times batched rows of length n and n + 1 for every n of EDGE_LENGTHS (fastest and median of 7
+    single steps through the C ABI, launch timing off) and says which kernel path each took."""
+    import torch
+
+    table = []
+    for dt, op, lengths in EDGE_LENGTHS:
+        for n in lengths:
+            rows = (1 << 26) // n
+            pair = []
+            for seg in (n, n + 1):
+                f, _, job = run_sort_workload(f"rows:{dt}:{rows}:{seg}:{op}", steps=7, warmup=2, profile_steps=1)
+                pair.append({"row_length": seg, "ms_min": round(f["ms_per_step_min"], 4),
+                             "ms_median": round(f["ms_per_step_median"], 4),
+                             "ps_per_key": round(f["ms_per_step_min"] * 1e9 / (rows * seg), 2),
+                             "path": f["config"]["path"], "verify": f["verify"]})
+                del job
+                torch.cuda.empty_cache()
+            table.append({"dtype": dt, "op": op, "rows": rows, "below": pair[0], "above": pair[1],
+                          "step": round(pair[1]["ms_min"] / pair[0]["ms_min"], 2)})
+    return {"metric": "row-length edges of the per-row kernels, ms per sort of rows x row_length keys",
+            "unit": "ms", "n_gpus": 1, "data": "synthetic", "edges": table}
 
 
 def algorithmic_bytes(cfg: dict, lds_limit_rows: bool, passes_run: int | None = None) -> dict:
@@ -284,6 +337,14 @@ def verify_sample(job: GpuJob, cfg: dict) -> str:
         seen[idx] = True
         perm = bool(seen.all())
         return "ok" if (ordered and stable and perm) else f"FAILED ordered={ordered} stable={stable} permutation={perm}"
+    tdt = {np.dtype(np.float32): torch.float32, np.dtype(np.float64): torch.float64, np.dtype(np.int32): torch.int32,
+           np.dtype(np.int64): torch.int64}.get(cfg["x"].dtype)
+    if cfg["op"] == "argsort" and cfg["x"].ndim == 2 and tdt is not None and not np.isnan(cfg["x"][:1]).any():
+        # batched rows without NaN: the stable argsort is unique, torch's stable sort must give the same indices
+        x = job.d_in.view(tdt).view(job.shape)
+        ref = torch.sort(x, dim=-1, stable=True).indices
+        same = job.d_idx.view(job.shape) == ref
+        return "ok" if bool(same.all()) else f"FAILED: {int((~same).sum())} indices differ from torch.sort(stable=True)"
     return "not checked here"
 
 
@@ -748,11 +809,21 @@ def main() -> None:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--config", default="c2",
-                    choices=["c1", "c2", "c3", "c4", "c5", "flat", "skinny", "lexsort", "searchsorted", "unique"],
+    known = ["c1", "c2", "c3", "c4", "c5", "flat", "skinny", "lexsort", "searchsorted", "unique"]
+
+    def config_name(text: str) -> str:
+        if text in known or text.startswith("rows:"):
+            return text
+        raise argparse.ArgumentTypeError(f"one of {', '.join(known)} or rows:<dtype>:<rows>:<row length>:<sort|argsort>")
+
+    ap.add_argument("--config", default="c2", type=config_name,
                     help="c1..c5: the sort workloads of the baseline; flat / skinny: the 2-D shapes of the "
                          "reference's sort microbenchmark; lexsort / searchsorted / unique: the callers and "
-                         "consumers of the sort path, on workloads of this file's own choosing")
+                         "consumers of the sort path, on workloads of this file's own choosing; "
+                         "rows:<dtype>:<rows>:<row length>:<sort|argsort>: batched rows of any length")
+    ap.add_argument("--edges", action="store_true",
+                    help="instead of a workload: time rows of length n and n + 1 for every n at which the "
+                         "library changes kernels (EDGE_LENGTHS), one JSON line")
     ap.add_argument("--log2n", type=int, default=None, help="shrink a 1-D workload to 2^L keys")
     ap.add_argument("--rows", type=int, default=None, help="shrink a 2-D workload to this many rows")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -766,6 +837,9 @@ def main() -> None:
     if args.gpus != 1:
         sys.exit("bench.py: this build sorts on one GPU; --gpus must be 1 (no multi-GPU sample sort is built)")
 
+    if args.edges:
+        print(json.dumps(run_edges()))
+        return
     if args.config in CONSUMERS:
         print(json.dumps(run_consumer(args)))
         return
