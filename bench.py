@@ -128,10 +128,10 @@ def make_config(name: str, log2n: int | None = None, rows: int | None = None) ->
 # operation, lengths whose successor is timed too; 2^26 keys per run.
 EDGE_LENGTHS = (
     ("float32", "sort", (32, 1024, 2048, 4096, 8192, 16384)),
-    ("float64", "sort", (512, 2048, 4096, 8192)),
+    ("float64", "sort", (512, 2048, 4096, 8192, 16384)),
     ("float16", "sort", (4096, 8192, 16384)),
     ("float32", "argsort", (4096, 8192, 16384)),
-    ("float64", "argsort", (4096, 8192)),
+    ("float64", "argsort", (4096, 8192, 14336)),
 )
 
 

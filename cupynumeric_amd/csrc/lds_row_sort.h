@@ -46,11 +46,20 @@
 namespace cpn {
 
 // Bins of the split above for a tile of `tile` keys: four per key, 4096 to 8192.
-__host__ __device__ constexpr int bucket_bins_log2(int tile) { return tile <= 1024 ? 12 : 13; }
+// (a tile of more than 64 KiB leaves room for 4096 only: they then share the 16 KiB of the digit counters)
+__host__ __device__ constexpr int bucket_bins_log2(int tile, int key_bytes)
+{
+  return (tile <= 1024 || tile * key_bytes > 64 * 1024) ? 12 : 13;
+}
 // Most keys a bin may hold for the split to be used (each key of a bin is compared with all others).
 constexpr uint32_t BUCKET_LIMIT = 24;
+// (four keys per bin on average instead of one or two, in the shape with 4096 bins for up to 16 384 keys)
+#ifndef CPN_BUCKET_LIMIT_WIDE
+#define CPN_BUCKET_LIMIT_WIDE 48
+#endif
+constexpr uint32_t BUCKET_LIMIT_WIDE = CPN_BUCKET_LIMIT_WIDE;
 // Keys past the end of a bin that the walk over the bins may read (and not count).
-constexpr int BUCKET_PAD = 32;
+constexpr int BUCKET_PAD = 64;
 
 // The arithmetic type of a real key of 4 or 8 bytes.
 template <int CODEC, int BYTES>
@@ -102,9 +111,8 @@ void lds_row_sort_kernel(const KeyT* keys_in,
   // (only the 1024-thread shapes, rows of more than 4096 keys: in the smaller shapes the bins cost
   // the LDS that lets many workgroups share a CU, and rows of 1024 float64 keys went from 0.41 to 0.60 ms)
   constexpr bool BUCKETS_OK = !HAS_IDX && NW == 1 && sizeof(KeyT) >= 4 && sizeof(KeyT) <= 8 && BLOCK == 1024 &&
-                              BLOCK * ITEMS * sizeof(KeyT) <= 64 * 1024 &&  // (the bins take 32 KiB beside the keys)
                               (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT);
-  constexpr int BINS_LOG2   = bucket_bins_log2(TILE);
+  constexpr int BINS_LOG2   = bucket_bins_log2(TILE, sizeof(KeyT));
   constexpr int BINS        = 1 << BINS_LOG2;
   constexpr int BINS_PER_THREAD = BINS / BLOCK;
   static_assert(!BUCKETS_OK || (BINS_PER_THREAD >= 4 && BINS_PER_THREAD % 4 == 0), "a thread scans whole 16-byte chunks");
@@ -416,7 +424,9 @@ void lds_row_sort_kernel(const KeyT* keys_in,
       if (lane == WAVE - 1) {
         s_wsum[wave] = incl;
       }
-      const int crowded = __syncthreads_or(largest > BUCKET_LIMIT ? 1 : 0);
+      constexpr uint32_t LIMIT = (TILE > 2 * BINS) ? BUCKET_LIMIT_WIDE : BUCKET_LIMIT;
+      static_assert(LIMIT <= static_cast<uint32_t>(BUCKET_PAD), "the walk reads up to LIMIT keys past a bin's end");
+      const int crowded = __syncthreads_or(largest > LIMIT ? 1 : 0);
       if (crowded == 0) {
         uint32_t run = incl - total;
         for (int w = 0; w < wave; ++w) {

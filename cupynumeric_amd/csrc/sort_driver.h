@@ -87,14 +87,13 @@ __host__ __device__ constexpr int global_tile(int key_bytes, bool big)
   return global_block(key_bytes) * global_items(key_bytes, big);
 }
 
-// Longest row the LDS kernel can take, per key width: 1024 threads with the row in 64 KiB of LDS
-// (plus staged row positions and the per-wave digit counters, 112 KiB at most of the CU's 160).
-// (8-byte keys: 12 and 16 per thread would fit the LDS without positions, but not the 128 vector
-// registers a thread of a 1024-thread workgroup can have: the compiler spills 0.7 to 1.5 KiB per thread.)
+// Longest row the LDS kernel can take, per key width: 1024 threads with the row, the staged row
+// positions of an argsort (2 bytes each) and 16 KiB of per-wave digit counters in the CU's 160 KiB
+// of LDS.  Keys of up to 4 bytes: 16 per thread (64 + 32 + 16 KiB).  8-byte keys: 16 per thread for
+// values only (128 + 16 KiB), 14 with positions (112 + 28 + 16 KiB).  16-byte keys: 4 per thread.
 __host__ __device__ constexpr uint64_t lds_row_capacity(int key_bytes, bool with_positions)
 {
-  (void)with_positions;
-  return key_bytes == 16 ? 4096 : (key_bytes == 8 ? 8192 : 16384);
+  return key_bytes == 16 ? 4096 : (key_bytes == 8 ? (with_positions ? 14336 : 16384) : 16384);
 }
 // Radix passes of a key: one per byte, plus the NaN-class pass of complex keys.
 __host__ __device__ constexpr int key_passes(int key_bytes, int codec)
@@ -413,7 +412,11 @@ inline int sort_rows_in_lds(const SortRequest& r)
       }
     }
     if constexpr (sizeof(KeyT) == 8) {
-      return launch_lds_rows<KeyT, CODEC, HAS_IDX, 1024, 8>(r);  // lds_row_capacity(8, ...) == 8192
+      if (r.seg <= 8192) {
+        return launch_lds_rows<KeyT, CODEC, HAS_IDX, 1024, 8>(r);
+      }
+      // the longest rows that fit the LDS of a CU: lds_row_capacity(8, HAS_IDX)
+      return launch_lds_rows<KeyT, CODEC, HAS_IDX, 1024, (HAS_IDX ? 14 : 16)>(r);
     } else {
       if (r.seg <= 8192) {
         // sixteen waves of eight keys hide the ranking latency better than eight waves of sixteen

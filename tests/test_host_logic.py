@@ -95,6 +95,14 @@ def test_temp_bytes_layout(lib):
     header = tb(f32, 0, 0, 1, 0, 0)
     assert header == 2048
     assert tb(f32, 1 << 20, 1024, 1, 1, 0) == header  # rows that fit LDS need only the header
+    # longest rows of the per-row kernels: 16 384 keys of up to 4 bytes; 8-byte keys 16 384 for values
+    # only, 14 336 when positions are staged beside them; 16-byte keys 4096
+    f64, c128_ = 11, 13
+    assert tb(f32, 4 * 16384, 16384, 1, 1, 0) == header and tb(f32, 4 * 16385, 16385, 1, 0, 0) > header
+    assert tb(f64, 4 * 16384, 16384, 1, 0, 0) == header and tb(f64, 4 * 16385, 16385, 1, 0, 0) > header
+    assert tb(f64, 4 * 14336, 14336, 0, 1, 0) == header and tb(f64, 4 * 14337, 14337, 0, 1, 0) > header
+    assert tb(f64, 4 * 14337, 14337, 1, 0, 0) == header
+    assert tb(c128_, 4 * 4096, 4096, 1, 1, 0) == header and tb(c128_, 4 * 4097, 4097, 1, 0, 0) > header
     n = 1 << 24
     tiles = n // 16384  # 512 threads x 32 keys per tile for keys of up to 4 bytes
 

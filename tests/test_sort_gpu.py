@@ -154,7 +154,7 @@ def test_random_module_and_flatten():
 
 # ---- per-row LDS path: every dtype, lengths around every workgroup-shape boundary -------------------
 LDS_LENGTHS = [1, 2, 3, 63, 64, 65, 255, 256, 257, 1000, 1023, 1024, 1025, 4095, 4096, 4097, 8191, 8192, 8193,
-               12000, 16383, 16384]
+               12000, 14335, 14336, 14337, 16383, 16384, 16385]
 
 
 @pytest.mark.parametrize("dtype", ALL_DTYPES)
@@ -174,8 +174,6 @@ def test_lds_rows_split_on_leading_bits(lib, torch_cuda, dtype):
     rng = np.random.default_rng(np.dtype(dtype).itemsize * 31 + np.dtype(dtype).num)
     dt = np.dtype(dtype)
     for seg in (1024, 1500, 2048, 4095, 4096, 6000, 8192, 8193, 12000, 16384):
-        if dt.itemsize == 8 and seg > 8192:
-            continue
         rows = 7
         if dt.kind == "f":
             x = rng.standard_normal((rows, seg)).astype(dtype)
