@@ -40,6 +40,30 @@ __global__ __launch_bounds__(256) void transpose_last_kernel(const T* __restrict
 
   const int tx = threadIdx.x % TS;
   const int ty = threadIdx.x / TS;
+  // A tile that lies inside the array takes the path without bounds checks, in which every load of
+  // a thread is issued before the first one is used (under a per-element check the compiler waits
+  // for each load before it issues the next).
+  const bool inside = (static_cast<uint64_t>(ta) + 1) * TS <= A && (static_cast<uint64_t>(tb) + 1) * TS <= B;
+  if (inside) {
+    constexpr int STEPS = TS / ROWS_PER_STEP;
+    const T* src        = in + in_base + (static_cast<uint64_t>(ta) * TS + ty) * in_row + static_cast<uint64_t>(tb) * TS + tx;
+    T v[STEPS];
+#pragma unroll
+    for (int k = 0; k < STEPS; ++k) {
+      v[k] = src[static_cast<uint64_t>(k) * ROWS_PER_STEP * in_row];
+    }
+#pragma unroll
+    for (int k = 0; k < STEPS; ++k) {
+      tile[ty + k * ROWS_PER_STEP][tx] = v[k];
+    }
+    __syncthreads();
+    T* dst = out + out_base + (static_cast<uint64_t>(tb) * TS + ty) * out_row + static_cast<uint64_t>(ta) * TS + tx;
+#pragma unroll
+    for (int k = 0; k < STEPS; ++k) {
+      dst[static_cast<uint64_t>(k) * ROWS_PER_STEP * out_row] = tile[tx][ty + k * ROWS_PER_STEP];
+    }
+    return;
+  }
   {
     const uint64_t ib = static_cast<uint64_t>(tb) * TS + tx;
 #pragma unroll 4
@@ -97,6 +121,34 @@ __global__ __launch_bounds__(256) void transpose_pairs_kernel(const uint32_t* __
 
   const int x = threadIdx.x % HP;  // word inside a row (load: column pair, store: row pair)
   const int y = threadIdx.x / HP;  // 0..3
+  // (tiles inside the array: no bounds checks, every load of a thread issued before the first use)
+  if (a0 + PAIR_TS <= A && b0 + PAIR_TS <= B) {
+    constexpr int YS    = 256 / HP;      // row pairs in flight per step
+    constexpr int STEPS = HP / YS;       // 16
+    const uint32_t* src = in + (in_base + (a0 + 2 * y) * in_row + b0 + 2 * x) / 2;
+    const uint64_t pair_stride = (2 * YS * in_row) / 2;  // words between the row pairs of two steps
+    const uint64_t row_words   = in_row / 2;
+    uint32_t w0[STEPS], w1[STEPS];
+#pragma unroll
+    for (int k = 0; k < STEPS; ++k) {
+      w0[k] = src[k * pair_stride];
+      w1[k] = src[k * pair_stride + row_words];
+    }
+#pragma unroll
+    for (int k = 0; k < STEPS; ++k) {
+      const int rp        = y + k * YS;
+      tile[2 * x][rp]     = __builtin_amdgcn_perm(w1[k], w0[k], 0x05040100u);
+      tile[2 * x + 1][rp] = __builtin_amdgcn_perm(w1[k], w0[k], 0x07060302u);
+    }
+    __syncthreads();
+    uint32_t* dst = out + (out_base + (b0 + y) * out_row + a0 + 2 * x) / 2;
+    const uint64_t out_step = (YS * out_row) / 2;
+#pragma unroll
+    for (int k = 0; k < PAIR_TS / YS; ++k) {
+      dst[k * out_step] = tile[y + k * YS][x];
+    }
+    return;
+  }
   {
     const uint64_t ib = b0 + 2 * x;
 #pragma unroll 4
