@@ -20,7 +20,7 @@ from ._thunk import SUPPORTED_DTYPES, DeviceArray, check_dtype
 
 __all__ = [
     "ndarray", "array", "asarray", "sort", "argsort", "sort_complex", "partition", "argpartition", "lexsort", "searchsorted", "unique", "take_along_axis",
-    "quantile", "percentile", "median",
+    "quantile", "percentile", "median", "nanquantile", "nanpercentile", "nanmedian",
     "random",
     "SUPPORTED_DTYPES",
 ]
@@ -236,4 +236,4 @@ def _split_first_axis(a: ndarray) -> list[ndarray]:
     return out
 
 
-from ._stats import median, percentile, quantile  # noqa: E402  (they call `sort` of this module)
+from ._stats import median, nanmedian, nanpercentile, nanquantile, percentile, quantile  # noqa: E402  (they call `sort` of this module)

@@ -82,6 +82,12 @@ PROTOTYPES: dict[str, tuple] = {
         c_int,
         [c_int, c_void_p, c_uint64, c_uint64, c_uint64, c_uint64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p],
     ),
+    "cpn_count_not_nan_sorted": (c_int, [c_int, c_void_p, c_uint64, c_uint64, c_uint64, c_void_p, c_void_p]),
+    "cpn_nanquantile_sorted": (
+        c_int,
+        [c_int, c_void_p, c_uint64, c_uint64, c_uint64, c_uint64, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+         c_void_p, c_void_p],
+    ),
     "cpn_take_along_last_axis": (
         c_int, [c_int, c_void_p, c_void_p, c_void_p, c_uint64, c_uint64, c_uint64, c_void_p, c_void_p]
     ),

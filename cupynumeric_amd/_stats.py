@@ -1,4 +1,5 @@
-"""Order statistics that sit on top of the sort: `quantile`, `percentile`, `median`.
+"""Order statistics that sit on top of the sort: `quantile`, `percentile`, `median` and the
+variants that ignore NaNs, `nanquantile`, `nanpercentile`, `nanmedian`.
 
 The reference sorts along the requested axis and then, for every quantile, takes the elements
 at one or two positions of that axis and combines them (`cupynumeric/_module/stats_order.py:358-650`,
@@ -250,3 +251,148 @@ def median(a: Any, axis: Any = None, out: ndarray | None = None, overwrite_input
     if a is None:
         raise TypeError("'None' is not suported input to 'median'")
     return quantile(a, 0.5, axis=axis, out=out, overwrite_input=overwrite_input, keepdims=keepdims, method="midpoint")
+
+
+def nanquantile(
+    a: Any,
+    q: Any,
+    axis: Any = None,
+    out: ndarray | None = None,
+    overwrite_input: bool = False,
+    method: str = "linear",
+    keepdims: bool = False,
+) -> ndarray:
+    """q-th quantile(s) along the given axis or axes, ignoring NaNs (`stats_order.py:653-951`).
+
+    A slice without any element that is not NaN gives NaN.  As in the reference, the position of a
+    quantile follows from the number of elements of its slice that are not NaN, the weights are
+    rounded to the array's type and so is every step of the weighted sum; the input has to be of a
+    floating-point type (`numpy.finfo` of the input's type is taken); complex input raises
+    TypeError.  The reference replaces NaNs by the largest finite value before it sorts, so a slice
+    that holds NaNs and +inf reads that value where `numpy.nanquantile` reads +inf: kept.
+    With `axis=None` the array is flattened first, as NumPy does.
+    """
+    a = convert_to_ndarray(a)
+    original_shape = a.shape
+    axes_set: tuple[int, ...] = ()
+    if axis is not None and isinstance(axis, Iterable):
+        axes_set = _normalize_axes(axis, a.ndim)
+        if len(axes_set) == 1:
+            real_axis, a_rr = axes_set[0], a
+        else:
+            real_axis, a_rr = _collapse_axes(a, axes_set)
+            overwrite_input = False
+    else:
+        real_axis, a_rr = axis, a
+        if real_axis is not None:
+            axes_set = _normalize_axes(real_axis, a.ndim)
+            real_axis = axes_set[0]
+    if method not in METHODS:
+        raise KeyError(method)
+    q_arr = np.asarray(q)
+    if a_rr.dtype.kind == "c":
+        raise TypeError("input array cannot be of complex type")
+    np.finfo(a_rr.dtype)  # (integer and bool input: the reference fails here, with this error)
+
+    from . import sort
+
+    if overwrite_input:
+        a_rr.sort(axis=real_axis)
+        arr = a_rr
+    else:
+        arr = sort(a_rr, axis=real_axis)  # NaNs last in every slice
+    to_dtype = arr.dtype if method in _KEEP_DTYPE else np.dtype(np.float64)
+
+    if real_axis is None:
+        n, outer, inner = arr.size, 1, 1
+        remaining = (1,) * len(original_shape) if keepdims else ()
+    else:
+        n = arr.shape[real_axis]
+        outer = int(np.prod(arr.shape[:real_axis], dtype=np.int64))
+        inner = int(np.prod(arr.shape[real_axis + 1 :], dtype=np.int64))
+        if keepdims:
+            remaining = tuple(1 if k in axes_set else original_shape[k] for k in range(len(original_shape)))
+        else:
+            remaining = tuple(arr.shape[k] for k in range(arr.ndim) if k != real_axis)
+    result_shape = (*q_arr.shape, *remaining)
+    if out is not None and out.shape != result_shape:
+        raise ValueError("wrong shape on output array")
+
+    slices = outer * inner
+    result = DeviceArray(result_shape, to_dtype)
+    if result.size:
+        lib = _lib.load()
+        torch = runtime.torch
+        dev = runtime.require_device()
+        stream = ctypes.c_void_p(runtime.stream_handle())
+        code = _lib.DTYPE_CODES[arr.dtype]
+        src = arr._thunk.base.ptr() if arr.size else None
+        d_counts = torch.empty(slices, dtype=torch.int64, device=dev)
+        _lib.check(lib.cpn_count_not_nan_sorted(code, src, outer, n, inner, d_counts.data_ptr(), stream),
+                   "cpn_count_not_nan_sorted")
+        counts = d_counts.cpu().numpy()  # (synchronises: the positions below depend on the counts)
+        # positions and weights per quantile and slice, worked out once per different count
+        # (`stats_order.py:713-746`)
+        distinct, which = np.unique(counts, return_inverse=True)
+        left = np.zeros((q_arr.size, slices), dtype=np.int64)
+        right = np.zeros((q_arr.size, slices), dtype=np.int64)
+        gamma = np.zeros((q_arr.size, slices), dtype=np.float64)
+        interpolate = True
+        for k, qv in enumerate(q_arr.reshape(-1)):
+            l_of = np.zeros(distinct.size, dtype=np.int64)
+            r_of = np.zeros(distinct.size, dtype=np.int64)
+            g_of = np.zeros(distinct.size, dtype=np.float64)
+            for j, cnt in enumerate(distinct):
+                cnt = int(cnt)
+                if cnt == 0:
+                    continue
+                g, lpos = _position(method, float(qv), cnt)
+                rpos = lpos + 1
+                if lpos >= cnt - 1:
+                    lpos = rpos = cnt - 1
+                elif lpos < 0:
+                    lpos = rpos = 0
+                l_of[j], r_of[j] = lpos, rpos
+                if g is None:
+                    interpolate = False
+                else:
+                    g_of[j] = g
+            left[k], right[k], gamma[k] = l_of[which], r_of[which], g_of[which]
+        if method in ("closest_observation", "lower", "higher", "nearest"):
+            interpolate = False  # (also when every slice is empty and no position was worked out)
+        d_left = torch.from_numpy(left).to(dev)
+        d_right = torch.from_numpy(right).to(dev)
+        d_gamma = torch.from_numpy(gamma).to(dev)
+        status = lib.cpn_nanquantile_sorted(
+            code, src, outer, n, inner, q_arr.size, d_counts.data_ptr(), d_left.data_ptr(), d_right.data_ptr(),
+            d_gamma.data_ptr(), int(interpolate), int(to_dtype == arr.dtype), result.base.ptr(), stream,
+        )
+        _lib.check(status, "cpn_nanquantile_sorted")
+    res = ndarray(result_shape, to_dtype, thunk=result)
+    if out is None:
+        return res
+    converted = res if out.dtype == res.dtype else res.astype(out.dtype)
+    out._thunk.base = converted._thunk.base
+    return out
+
+
+def nanpercentile(
+    a: Any,
+    q: Any,
+    axis: Any = None,
+    out: ndarray | None = None,
+    overwrite_input: bool = False,
+    method: str = "linear",
+    keepdims: bool = False,
+) -> ndarray:
+    """q-th percentile(s) ignoring NaNs: `nanquantile` of q / 100 (`stats_order.py:954-1080`)."""
+    q01 = np.asarray(q) / 100.0
+    return nanquantile(a, q01, axis, out=out, overwrite_input=overwrite_input, method=method, keepdims=keepdims)
+
+
+def nanmedian(a: Any, axis: Any = None, out: ndarray | None = None, overwrite_input: bool = False, keepdims: bool = False) -> ndarray:
+    """Median ignoring NaNs: the 0.5 `nanquantile` with method 'midpoint'
+    (`cupynumeric/_module/stats_avgs_vars.py:445-512`)."""
+    if a is None:
+        raise TypeError("'None' is not suported input to 'nanmedian'")
+    return nanquantile(a, 0.5, axis=axis, out=out, overwrite_input=overwrite_input, keepdims=keepdims, method="midpoint")

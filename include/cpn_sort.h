@@ -299,6 +299,35 @@ int cpn_quantile_sorted(int dtype, const void* sorted, uint64_t outer, uint64_t 
                         int interpolate, void* out, void* stream);
 
 /*
+ * The quantiles of nanquantile / nanpercentile / nanmedian, which ignore NaNs
+ * (cupynumeric/_module/stats_order.py:653-951, cupynumeric/_module/stats_avgs_vars.py:445-512).
+ * `sorted` is a dense [outer][n][inner] array of float16 / float32 / float64 sorted along the middle
+ * axis in NumPy order, i.e. with the NaNs of every slice at its end.
+ *
+ * cpn_count_not_nan_sorted: counts[o][i] (int64) = number of elements of slice (o, i) that are not
+ * NaN, by binary search; replaces count_nonzero(logical_not(isnan(a)), axis) (stats_order.py:879-881).
+ *
+ * cpn_nanquantile_sorted: for quantile q and slice s = (o, i), with left, right (int64) and gamma
+ * (float64) device arrays of num_q * outer * inner entries ([q][o][i]) that the caller has worked
+ * out from counts[s] (stats_order.py:713-746):
+ *   counts[s] == 0      out[q][s] = NaN
+ *   interpolate == 0    out[q][s] = v(left[q][s])
+ *   interpolate != 0    g = gamma[q][s] rounded to the element type; out[q][s] =
+ *                       (1 - g) * v(left[q][s]) + g * v(right[q][s]), every operation rounded in the
+ *                       element type, as the reference evaluates it on arrays of that type (:748-757)
+ * where v(p) is element p of the slice as the reference sees it: it replaces the NaNs by the largest
+ * finite value of the type BEFORE it sorts (:886-887), so in a slice that holds m NaNs the m
+ * positions after its last finite element read as that value and +inf elements follow them.
+ * `out` holds elements of `dtype` when keep_dtype != 0 (the methods that pick samples, and
+ * inverted_cdf), float64 otherwise.  Other dtypes return CPN_ERR_DTYPE.
+ */
+int cpn_count_not_nan_sorted(int dtype, const void* sorted, uint64_t outer, uint64_t n, uint64_t inner,
+                             int64_t* counts, void* stream);
+int cpn_nanquantile_sorted(int dtype, const void* sorted, uint64_t outer, uint64_t n, uint64_t inner,
+                           uint64_t num_q, const int64_t* counts, const int64_t* left, const int64_t* right,
+                           const double* gamma, int interpolate, int keep_dtype, void* out, void* stream);
+
+/*
  * out[r][j] = src[r][indices[r][j]] for `rows` dense rows: src rows hold src_seg elements of
  * elem_bytes (1, 2, 4, 8 or 16) bytes, indices and out rows hold idx_seg elements.  Indices are
  * int64, negative ones count from the end of the row.  An index outside [-src_seg, src_seg)

@@ -438,3 +438,84 @@ def percentile(a, q, axis=None, method: str = "linear", keepdims: bool = False, 
 def median(a, axis=None, keepdims: bool = False, threads: int = 1) -> np.ndarray:
     """`cupynumeric/_module/stats_avgs_vars.py:373-443`."""
     return quantile(a, 0.5, axis=axis, method="midpoint", keepdims=keepdims, threads=threads)
+
+
+def nanquantile(a, q, axis=None, method: str = "linear", keepdims: bool = False, threads: int = 1) -> np.ndarray:
+    """`stats_order.py:763-951` with `nanquantile_impl` (`:653-760`): count the elements of every slice
+    that are not NaN, replace the NaNs by the largest finite value of the type, sort, and per quantile
+    and slice take the position that the estimator gives for that count; weights, `1 - weights`, the
+    two products and the sum are arrays of the input's type (`:708-710,748-757`).  A slice with no
+    element left gives NaN.  With `axis=None` the input is flattened first (NumPy's meaning of it)."""
+    x = np.asarray(a)
+    original_shape = x.shape
+    axes_set = ()
+    if axis is not None and not np.isscalar(axis):
+        axes_set = tuple(int(ax) % x.ndim for ax in axis)
+        if len(axes_set) == 1:
+            real_axis, x_rr = axes_set[0], x
+        else:
+            wanted = sorted(axes_set)
+            first = wanted[0]
+            moved = np.moveaxis(x, wanted, range(first, first + len(wanted)))
+            merged = int(np.prod(moved.shape[first : first + len(wanted)], dtype=np.int64))
+            x_rr = np.ascontiguousarray(moved).reshape(moved.shape[:first] + (merged,) + moved.shape[first + len(wanted) :])
+            real_axis = first
+    else:
+        real_axis, x_rr = axis, x
+        if real_axis is not None:
+            axes_set = (int(real_axis) % x.ndim,)
+            real_axis = axes_set[0]
+    if x_rr.dtype.kind == "c":
+        raise TypeError("input array cannot be of complex type")
+    if real_axis is None:
+        x_rr, real_axis, flat = x_rr.reshape(-1), 0, True
+    else:
+        flat = False
+    counts = np.count_nonzero(~np.isnan(x_rr), axis=real_axis)
+    q_arr = np.asarray(q)
+    arr = sort(np.where(np.isnan(x_rr), np.finfo(x_rr.dtype).max, x_rr), axis=real_axis, threads=threads)
+    to_dtype = arr.dtype if method in ("inverted_cdf", "closest_observation", "lower", "higher", "nearest") else np.dtype(np.float64)
+    plain = tuple(arr.shape[k] for k in range(arr.ndim) if k != real_axis)
+    if keepdims:
+        remaining = (1,) * len(original_shape) if flat else tuple(
+            1 if k in axes_set else original_shape[k] for k in range(len(original_shape)))
+    else:
+        remaining = plain
+    res = np.zeros((*q_arr.shape, *remaining), dtype=to_dtype)
+    gammas = np.zeros(plain, dtype=arr.dtype)
+    lvals = np.zeros(plain, dtype=arr.dtype)
+    rvals = np.zeros(plain, dtype=arr.dtype)
+    for qindex, qv in np.ndenumerate(q_arr):
+        gamma = None
+        for aindex, n in np.ndenumerate(counts):
+            n = int(n)
+            if n == 0:
+                lvals[aindex] = np.nan
+                rvals[aindex] = np.nan
+                continue
+            gamma, left = _quantile_position(method, float(qv), n)
+            right = left + 1
+            if left >= n - 1:
+                left = right = n - 1
+            elif left < 0:
+                left = right = 0
+            lvals[aindex] = arr[(*aindex[:real_axis], left, *aindex[real_axis:])]
+            if gamma is not None:
+                gammas[aindex] = gamma
+                rvals[aindex] = arr[(*aindex[:real_axis], right, *aindex[real_axis:])]
+        with np.errstate(invalid="ignore", over="ignore"):
+            if gamma is None:
+                res[qindex] = lvals.reshape(remaining)
+            else:
+                res[qindex] = ((1 - gammas) * lvals + gammas * rvals).reshape(remaining)
+    return res
+
+
+def nanpercentile(a, q, axis=None, method: str = "linear", keepdims: bool = False, threads: int = 1) -> np.ndarray:
+    """`stats_order.py:954-1080`."""
+    return nanquantile(a, np.asarray(q) / 100.0, axis, method=method, keepdims=keepdims, threads=threads)
+
+
+def nanmedian(a, axis=None, keepdims: bool = False, threads: int = 1) -> np.ndarray:
+    """`cupynumeric/_module/stats_avgs_vars.py:445-512`."""
+    return nanquantile(a, 0.5, axis=axis, method="midpoint", keepdims=keepdims, threads=threads)

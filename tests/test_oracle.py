@@ -378,3 +378,70 @@ def test_quantile_closed_forms():
     assert oracle.quantile(np.array([7]), 0.3, method="weibull") == 7.0
     with pytest.raises(TypeError):
         oracle.quantile(np.array([1 + 2j, 3j]), 0.5)
+
+
+# tests/integration/test_nanquantiles.py:47-58: the reference's own input
+NANQUANTILE_REF_INPUT = np.asarray([[1.0, 2, 2, 40], [1, np.nan, 2, 1], [0, 10, np.nan, np.nan], [np.nan, np.nan, 0, 10],
+                                    [np.nan, np.nan, np.nan, np.nan]])
+
+
+@pytest.mark.parametrize("method", QUANTILE_METHODS)
+def test_nanquantile_matches_numpy_on_the_reference_cases(method):
+    """The oracle's nanquantile / nanpercentile / nanmedian against numpy's on the input, axes and
+    quantiles of tests/integration/test_nanquantiles.py:41-103 and test_nanpercentiles.py (atol 1e-8,
+    exactly for the methods that pick samples), on random float64 / float32 data with NaNs scattered
+    and whole slices of NaN, every axis, keepdims, and axis=None (test_keepdims, :106-111)."""
+    import warnings
+
+    rng = np.random.default_rng(45)
+    rnd = rng.standard_normal((4, 6, 5))
+    rnd[rng.random(rnd.shape) < 0.3] = np.nan
+    rnd[1, :, 2] = np.nan
+    inputs = [NANQUANTILE_REF_INPUT, rnd, rnd.astype(np.float32)]
+    picks = method in ("inverted_cdf", "closest_observation", "lower", "higher", "nearest")
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore", RuntimeWarning)  # NumPy warns about slices of NaN only
+        for arr in inputs:
+            axes_list = (0, 1, (0, 1), (0,), None) + (((0, 2), 2) if arr.ndim == 3 else ())
+            for axes in axes_list:
+                for qs in QUANTILE_REF_QS:
+                    for keepdims in (False, True):
+                        want = np.nanquantile(arr, qs, axis=axes, method=method, keepdims=keepdims)
+                        got = oracle.nanquantile(arr, qs, axis=axes, method=method, keepdims=keepdims)
+                        assert got.shape == want.shape, (method, axes, keepdims)
+                        if arr.dtype == np.float64:
+                            assert got.dtype == want.dtype
+                        else:  # float64 unless the method picks samples (stats_order.py:893-903); NumPy keeps float32
+                            assert got.dtype == (np.float32 if picks else np.float64)
+                        if picks:
+                            assert np.array_equal(got, want, equal_nan=True), (method, axes, qs)
+                        else:
+                            assert np.allclose(got, want, atol=1e-8 if arr.dtype == np.float64 else 1e-5, equal_nan=True), (method, axes, qs)
+                        p = oracle.nanpercentile(arr, np.asarray(qs) * 100.0, axis=axes, method=method, keepdims=keepdims)
+                        assert np.allclose(p, np.nanpercentile(arr, np.asarray(qs) * 100.0, axis=axes, method=method, keepdims=keepdims),
+                                           atol=1e-5, equal_nan=True)
+        for arr in inputs:
+            for axes in (None, 0, -1):
+                assert np.allclose(oracle.nanmedian(arr, axis=axes), np.nanmedian(arr, axis=axes), atol=1e-6, equal_nan=True)
+
+
+def test_nanquantile_closed_forms_and_the_reference_quirks():
+    # no NaN at all: the same positions as quantile (weights in the array's type make no difference for float64)
+    x = np.arange(101, dtype=np.float64)[::-1].copy()
+    assert np.array_equal(oracle.nanquantile(x, [0.0, 0.25, 0.5, 1.0]), [0.0, 25.0, 50.0, 100.0])
+    # NaNs are dropped: the median of {1, 2, 10} and of {4}
+    assert oracle.nanmedian(np.array([np.nan, 10.0, 1.0, np.nan, 2.0])) == 2.0
+    assert np.array_equal(oracle.nanmedian(np.array([[np.nan, 4.0], [np.nan, np.nan]]), axis=1), [4.0, np.nan], equal_nan=True)
+    # float32: the weight 0.3 is rounded to float32 and so is every step (stats_order.py:708-710,748-757)
+    v = np.array([1.0, 2.0, np.nan], dtype=np.float32)
+    g = np.float32(0.3)
+    assert oracle.nanquantile(v, 0.3) == np.float64((np.float32(1) - g) * np.float32(1.0) + g * np.float32(2.0))
+    # NaNs become the largest finite value BEFORE the sort (stats_order.py:886-887), so with +inf in the
+    # same slice the position after the last finite element reads that value, where NumPy reads +inf
+    w = np.array([1.0, np.inf, np.nan])
+    assert oracle.nanquantile(w, 1.0, method="lower") == np.finfo(np.float64).max
+    assert np.nanquantile(w, 1.0, method="lower") == np.inf
+    with pytest.raises(TypeError):
+        oracle.nanquantile(np.array([1 + 2j, np.nan + 0j]), 0.5)
+    with pytest.raises(ValueError):
+        oracle.nanquantile(np.array([1, 2, 3]), 0.5)  # numpy.finfo of an integer type, as in the reference

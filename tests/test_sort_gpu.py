@@ -548,7 +548,9 @@ def test_swapaxes_copy(lib, torch_cuda, elem):
               ((4, 5), 1, 1), ((2, 2, 1, 1, 2, 1, 2), 0, 6),
               # even extents: 2-byte elements move as 32-bit words in 128 x 128 tiles
               ((128, 128), 0, 1), ((130, 258), 0, 1), ((2, 4), 0, 1), ((200, 2), 0, 1), ((6, 4, 10), 0, 2),
-              ((3, 8, 6), 1, 2), ((2, 256, 3, 130), 1, 3), ((514, 126), 1, 0)]
+              ((3, 8, 6), 1, 2), ((2, 256, 3, 130), 1, 3), ((514, 126), 1, 0),
+              # several tiles inside the array (the path without bounds checks) beside edge tiles, batched
+              ((3, 300, 2, 260), 1, 3), ((384, 512), 0, 1), ((2, 129, 383), 1, 2)]
     rng = np.random.default_rng(0)
     for shape, a, b in shapes:
         x = rng.integers(0, 255, int(np.prod(shape)) * np.dtype(elem).itemsize, dtype=np.uint8).view(elem).reshape(shape)
