@@ -87,6 +87,7 @@ void lds_row_sort_kernel(const KeyT* keys_in,
                                                               KeyT* keys_out,
                                                               int64_t* idx_out,
                                                               uint32_t seg,
+                                                              uint64_t row_stride,
                                                               int64_t index_offset,
                                                               uint32_t* status)
 {
@@ -131,7 +132,7 @@ void lds_row_sort_kernel(const KeyT* keys_in,
   const int tid       = threadIdx.x;
   const int lane      = tid & (WAVE - 1);
   const int wave      = tid / WAVE;
-  const uint64_t base = static_cast<uint64_t>(blockIdx.x) * seg;
+  const uint64_t base = static_cast<uint64_t>(blockIdx.x) * row_stride;  // (row_stride == seg: dense rows)
   const bool full     = (seg == TILE);
   // A row shorter than the tile is dealt in equal contiguous shares of whole 64-key rounds, so that
   // every wave works on `rounds` keys per lane and the cost follows the row length, not the tile.

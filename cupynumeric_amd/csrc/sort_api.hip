@@ -56,6 +56,14 @@ static std::atomic<int> g_tile_order{[] {
 
 bool tile_order_single() { return g_tile_order.load(std::memory_order_relaxed) != 0; }
 
+// 1: rows of up to twice the LDS capacity are sorted as two halves and merged; 0: global path
+static std::atomic<int> g_merge_rows{[] {
+  const char* e = getenv("CPN_SORT_MERGE_ROWS");
+  return (e != nullptr && e[0] == '0') ? 0 : 1;
+}()};
+
+bool merge_rows_enabled() { return g_merge_rows.load(std::memory_order_relaxed) != 0; }
+
 static std::atomic<long long> g_spin_limit{static_cast<long long>(LOOKBACK_SPIN_LIMIT)};
 
 uint32_t lookback_spin_limit() { return static_cast<uint32_t>(g_spin_limit.load(std::memory_order_relaxed)); }
@@ -172,6 +180,8 @@ int64_t cpn_set_lookback_spin_limit(int64_t polls)
 }
 
 int cpn_set_tile_order(int single) { return cpn::g_tile_order.exchange(single != 0 ? 1 : 0); }
+
+int cpn_set_merge_rows(int enabled) { return cpn::g_merge_rows.exchange(enabled != 0 ? 1 : 0); }
 
 int64_t cpn_set_wave_row_limit(int64_t limit)
 {

@@ -14,6 +14,7 @@
 #include "onesweep.h"
 #include "profile.h"
 #include "tiny_row_sort.h"
+#include "merge_rows.h"
 #include "wave_row_sort.h"
 
 namespace cpn {
@@ -115,6 +116,24 @@ uint64_t count16_min_row();
 // to send every request down the global path for an A/B run.
 uint64_t lds_row_limit(int key_bytes, bool with_positions);
 
+// Rows longer than the per-row kernels take, up to twice that length: sorted as two halves by the
+// per-row kernel and merged (merge_rows.h) instead of going down the global path.  Real keys of 4
+// and 8 bytes.  Off when cpn_set_merge_rows(0) / CPN_SORT_MERGE_ROWS=0 says so, and whenever the
+// LDS row limit has been lowered (an A/B run that wants the global path gets it).
+bool merge_rows_enabled();
+inline bool merged_rows_apply(int key_bytes, int passes, uint64_t volume, uint64_t seg, bool want_indices)
+{
+  if (!merge_rows_enabled() || (key_bytes != 4 && key_bytes != 8) || passes != key_bytes || volume == 0) {
+    return false;
+  }
+  const uint64_t cap = lds_row_capacity(key_bytes, want_indices);
+  if (lds_row_limit(key_bytes, want_indices) != cap || seg <= cap || seg > 2 * cap) {
+    return false;
+  }
+  const uint64_t chunks = (seg + MERGE_CHUNK_MIN - 1) / MERGE_CHUNK_MIN;
+  return (volume / seg) * chunks < (1ull << 31);  // one workgroup of the merge per chunk of a row
+}
+
 // Element type code (enum cpn_dtype) -> key width and codec.
 struct KeyKind {
   int bytes;  // 0 = unknown code
@@ -152,6 +171,7 @@ struct SortRequest {
   void* temp;
   uint64_t temp_bytes;
   hipStream_t stream;
+  uint64_t row_stride = 0;  // elements between the starts of two rows, in input and outputs; 0: seg (dense rows)
 };
 
 // Workspace layout of the global path.  Everything in [0, zero_bytes) is cleared per call.
@@ -232,6 +252,11 @@ inline uint64_t workspace_bytes(int key_bytes, int passes, uint64_t volume, uint
   if (volume == 0 || seg <= lds_row_limit(key_bytes, want_indices)) {
     return HEADER_BYTES;
   }
+  if (merged_rows_apply(key_bytes, passes, volume, seg, want_indices)) {
+    // the rows with their halves sorted: keys, and the int64 positions of an argsort
+    return HEADER_BYTES + align_up(volume * key_bytes, WORKSPACE_ALIGN) +
+           (want_indices ? align_up(volume * 8, WORKSPACE_ALIGN) : 0);
+  }
   const GlobalLayout L = global_layout(key_bytes, passes, volume, seg, want_values, want_indices, in_place);
   return L.valid ? L.total : 0;
 }
@@ -255,6 +280,45 @@ inline int launch_zero_fill(void* p, uint64_t bytes, hipStream_t stream)
   return CPN_OK;
 }
 
+// ---- rows of up to twice the LDS capacity: two sorted halves, merged ---------------------------
+template <typename KeyT, int CODEC, bool HAS_IDX>
+inline int sort_rows_in_lds(const SortRequest& r);
+
+template <typename KeyT, int CODEC, bool HAS_IDX>
+int sort_rows_merged(const SortRequest& r)
+{
+  const uint64_t n = r.seg, rows = r.volume / n;
+  const uint64_t h = (n + 1) / 2;  // first half; both halves fit the per-row kernel
+  uint8_t* ws      = static_cast<uint8_t*>(r.temp);
+  KeyT* tmp_keys   = reinterpret_cast<KeyT*>(ws + HEADER_BYTES);
+  int64_t* tmp_idx =
+    HAS_IDX ? reinterpret_cast<int64_t*>(ws + HEADER_BYTES + align_up(r.volume * sizeof(KeyT), WORKSPACE_ALIGN)) : nullptr;
+  for (int half = 0; half < 2; ++half) {
+    const uint64_t off = half == 0 ? 0 : h, len = half == 0 ? h : n - h;
+    SortRequest c      = r;
+    c.values_in        = static_cast<const KeyT*>(r.values_in) + off;
+    c.values_out       = tmp_keys + off;
+    c.indices_out      = HAS_IDX ? tmp_idx + off : nullptr;
+    c.seg              = len;
+    c.volume           = rows * len;
+    c.row_stride       = n;
+    c.index_offset     = r.index_offset + static_cast<int64_t>(off);  // positions count from the start of the whole row
+    const int rc       = sort_rows_in_lds<KeyT, CODEC, HAS_IDX>(c);
+    if (rc != CPN_OK) {
+      return rc;
+    }
+  }
+  const uint64_t chunks = (n + merge_chunk(HAS_IDX) - 1) / merge_chunk(HAS_IDX);
+  {
+    ProfileScope prof("merge_halves", r.stream);
+    hipLaunchKernelGGL((merge_halves_kernel<KeyT, CODEC, HAS_IDX>), dim3(static_cast<uint32_t>(rows * chunks)),
+                       dim3(merge_block(HAS_IDX)), 0, r.stream, tmp_keys, tmp_idx, static_cast<KeyT*>(r.values_out), r.indices_out,
+                       static_cast<uint32_t>(n), static_cast<uint32_t>(h), static_cast<uint32_t>(chunks));
+  }
+  CPN_HIP_TRY(hipGetLastError());
+  return CPN_OK;
+}
+
 // ---- per-row LDS path ------------------------------------------------------------------
 template <typename KeyT, int CODEC, bool HAS_IDX, int BLOCK, int ITEMS>
 inline int launch_lds_rows(const SortRequest& r)
@@ -265,7 +329,8 @@ inline int launch_lds_rows(const SortRequest& r)
     hipLaunchKernelGGL((lds_row_sort_kernel<KeyT, CODEC, HAS_IDX, BLOCK, ITEMS>),
                        dim3(static_cast<uint32_t>(rows)), dim3(BLOCK), 0, r.stream,
                        static_cast<const KeyT*>(r.values_in), static_cast<KeyT*>(r.values_out), r.indices_out,
-                       static_cast<uint32_t>(r.seg), r.index_offset, static_cast<uint32_t*>(r.temp));
+                       static_cast<uint32_t>(r.seg), r.row_stride != 0 ? r.row_stride : r.seg, r.index_offset,
+                       static_cast<uint32_t*>(r.temp));
   }
   CPN_HIP_TRY(hipGetLastError());
   return CPN_OK;
@@ -352,6 +417,9 @@ inline int launch_tiny_rows(const SortRequest& r)
 template <typename KeyT, int CODEC, bool HAS_IDX>
 inline int sort_rows_in_lds(const SortRequest& r)
 {
+  if (r.row_stride != 0 && (r.seg <= 4096 || sizeof(KeyT) < 4)) {
+    return CPN_ERR_UNSUPPORTED;  // only the one-workgroup-per-row kernel of 4- and 8-byte keys takes strided rows
+  }
   if (r.volume / r.seg >= (1ull << 31)) {
     return CPN_ERR_UNSUPPORTED;
   }
@@ -684,6 +752,11 @@ int sort_typed(const SortRequest& r)
       }
     }
     return CPN_OK;
+  }
+  if constexpr ((KB == 4 || KB == 8) && KeyTraits<CODEC, KeyT>::NWORDS == 1) {
+    if (merged_rows_apply(KB, PASSES, r.volume, r.seg, has_idx)) {
+      return has_idx ? sort_rows_merged<KeyT, CODEC, true>(r) : sort_rows_merged<KeyT, CODEC, false>(r);
+    }
   }
   const GlobalLayout L = global_layout(KB, PASSES, r.volume, r.seg, r.values_out != nullptr, has_idx, in_place);
   if (L.big) {

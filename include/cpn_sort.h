@@ -90,6 +90,17 @@ int64_t cpn_set_lds_row_limit(int64_t limit);
 int64_t cpn_set_wave_row_limit(int64_t limit);
 
 /*
+ * Process-wide switch: rows longer than the per-row kernels take, up to twice that length (real keys
+ * of 4 and 8 bytes), are sorted as two halves by the per-row kernel and merged (enabled != 0, the
+ * default) or go down the global path like longer rows (0).  Returns the previous setting.  Also
+ * initialised from the environment variable CPN_SORT_MERGE_ROWS (0 switches it off).  Changes the
+ * sizes returned by cpn_local_sort_temp_bytes: do not change it between the size query and the sort.
+ * An A/B switch with no counterpart in the reference, whose segmented radix sort takes every row
+ * length (src/cupynumeric/sort/cub_sort.cuh:81-105).
+ */
+int cpn_set_merge_rows(int enabled);
+
+/*
  * Process-wide tunable: rows of at least `elements` elements on the global path keep their
  * per-row counts, tile descriptors and row positions in 64 bits.  The default and the maximum
  * is 2^30 (shorter rows use 32 bits); a negative value restores the default and the previous

@@ -99,10 +99,15 @@ def test_temp_bytes_layout(lib):
     # only, 14 336 when positions are staged beside them; 16-byte keys 4096
     f64, c128_ = 11, 13
     assert tb(f32, 4 * 16384, 16384, 1, 1, 0) == header and tb(f32, 4 * 16385, 16385, 1, 0, 0) > header
+    assert tb(9, 4 * 16385, 16385, 1, 0, 0) > header  # float16
     assert tb(f64, 4 * 16384, 16384, 1, 0, 0) == header and tb(f64, 4 * 16385, 16385, 1, 0, 0) > header
     assert tb(f64, 4 * 14336, 14336, 0, 1, 0) == header and tb(f64, 4 * 14337, 14337, 0, 1, 0) > header
     assert tb(f64, 4 * 14337, 14337, 1, 0, 0) == header
     assert tb(c128_, 4 * 4096, 4096, 1, 1, 0) == header and tb(c128_, 4 * 4097, 4097, 1, 0, 0) > header
+    # rows of up to twice those lengths (real keys of 4 and 8 bytes): the rows once more, and their positions
+    assert tb(f32, 4 * 20000, 20000, 1, 0, 0) == header + align256(4 * 20000 * 4)
+    assert tb(f64, 4 * 20000, 20000, 0, 1, 0) == header + align256(4 * 20000 * 8) + align256(4 * 20000 * 8)
+    assert tb(f32, 4 * 32769, 32769, 1, 0, 0) > header + align256(4 * 32769 * 4)  # global layout: histograms, descriptors
     n = 1 << 24
     tiles = n // 16384  # 512 threads x 32 keys per tile for keys of up to 4 bytes
 

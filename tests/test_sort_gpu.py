@@ -539,6 +539,62 @@ def test_global_path_skipping_needs_every_row(lib, torch_cuda, global_path):
     check_rows(lib, torch_cuda, x.astype(np.int64), "per-row constant bytes, int64")
 
 
+# ---- rows of up to twice the LDS capacity: two sorted halves, merged -----------------------------------
+@pytest.mark.parametrize("dtype", [np.float32, np.int32, np.uint32, np.float64, np.int64, np.uint64])
+def test_rows_sorted_as_merged_halves(lib, torch_cuda, dtype):
+    """Row lengths on both sides of the range that is sorted as two halves and merged (16 385 ... 32 768;
+    14 337 ... 28 672 for 8-byte keys with positions), odd and even lengths, rows with many ties across
+    the two halves (stability of the merge), sorted, reversed and constant rows, special float values,
+    values and positions together, in place, an index offset; and the same requests with the path
+    switched off give the same bits through the global path."""
+    dt = np.dtype(dtype)
+    rng = np.random.default_rng(dt.num * 7 + 1)
+    lengths = [16385, 16386, 20001, 28672, 28673, 32767, 32768, 32769] + ([14337, 14338] if dt.itemsize == 8 else [])
+    header = lib.cpn_local_sort_temp_bytes(_lib.DTYPE_CODES[dt], 0, 0, 1, 0, 0)
+    for seg in lengths:
+        rows = 5
+        x = make_input(dtype, (rows, seg), seed=seg)
+        x[1] = np.sort(x[1])
+        x[2] = np.sort(x[2])[::-1]
+        if dt.kind == "f":
+            x[3] = rng.integers(0, 6, seg).astype(dtype)                 # six different keys: ties everywhere
+            x[4, ::7] = np.nan
+            x[4, 1::7] = -0.0
+            x[4, 2::7] = 0.0
+        else:
+            x[3] = rng.integers(0, 6, seg).astype(dtype)
+            x[4] = x[4, 0]
+        check_rows(lib, torch_cuda, x, f"{dt} seg={seg}")
+        want_v, want_i = oracle.local_sort(x, argsort=False), oracle.local_sort(x, argsort=True)
+        v, i = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=True, offset=1000)
+        assert_same_bits(v, want_v, f"{dt} seg={seg} values+positions")
+        assert_same_bits(i, want_i + 1000, f"{dt} seg={seg} values+positions, offset")
+        v, _ = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=False, in_place=True)
+        assert_same_bits(v, want_v, f"{dt} seg={seg} in place")
+    # the path is the one that runs: its workspace is the rows once (plus positions), not the global layout
+    code, seg, rows = _lib.DTYPE_CODES[dt], 20000, 4
+    merged_bytes = lib.cpn_local_sort_temp_bytes(code, rows * seg, seg, 1, 0, 0)
+    assert merged_bytes == header + (rows * seg * dt.itemsize + 255) // 256 * 256
+    prev = lib.cpn_set_merge_rows(0)
+    try:
+        assert lib.cpn_local_sort_temp_bytes(code, rows * seg, seg, 1, 0, 0) != merged_bytes
+        x = make_input(dtype, (3, 20001), seed=5)
+        check_rows(lib, torch_cuda, x, f"{dt} global path, merge switched off")
+    finally:
+        lib.cpn_set_merge_rows(prev)
+    assert lib.cpn_local_sort_temp_bytes(code, rows * seg, seg, 1, 0, 0) == merged_bytes
+
+
+def test_merged_rows_many_rows_and_narrow_keys_stay_out(lib, torch_cuda):
+    # many rows: every workgroup of the merge finds its own part of its own row
+    x = make_input(np.float32, (300, 17000), seed=3)
+    check_rows(lib, torch_cuda, x, "300 rows of 17000")
+    # 2-byte, 1-byte and complex keys of such lengths take the global path
+    for dtype in (np.float16, np.uint8, np.complex64):
+        x = make_input(dtype, (3, 17000), seed=4)
+        check_rows(lib, torch_cuda, x, f"{np.dtype(dtype)} rows of 17000")
+
+
 # ---- swapaxes copy ------------------------------------------------------------------------------------
 @pytest.mark.parametrize("elem", [np.uint8, np.float16, np.int32, np.float64, np.complex128])
 def test_swapaxes_copy(lib, torch_cuda, elem):
