@@ -7,8 +7,12 @@
 // merge sort used for rows of at most 400 elements (src/cupynumeric/sort/thrust_sort.cuh:68-122).
 //
 // Digits on which every key of the row agrees are found up front with one AND/OR
-// reduction of the ordered keys and their passes are skipped (the pass would be the
-// identity permutation).
+// reduction and their passes are skipped (the pass would be the identity permutation).
+//
+// All loads of a row are issued before the first use, unconditionally, from offsets clamped into
+// the row: under the branch that also encodes a key the compiler waits for each load before it
+// issues the next, and under per-round uniform branches it copies the whole key array at every
+// join and spills.
 //
 // Wide keys: a row of n keys is almost always put in order by its leading 2*log2(n) or so
 // varying bits.  When more passes than that are due, the kernel first runs only the passes of
@@ -20,12 +24,15 @@
 // the input.
 //
 // Values-only sorts of rows whose keys that tie are the same bits (integers; floats without NaN and
-// -0.0): no order among equal keys shows, so the row need not go through stable passes at all.  It is
-// first split into 8192 ranges of equal width between its smallest and its largest key, one LDS atomic
-// per key on a histogram of 8192 bins, which leaves a handful of keys per bin on evenly or normally
-// distributed data; every key then finds its place inside its bin by counting the smaller keys of the bin.  A row that crowds
-// more than BUCKET_LIMIT keys into one bin (few different keys, tight clusters) goes through the
-// radix passes instead.  Used by the 1024-thread shapes (rows of more than 4096 keys).
+// -0.0): no order among equal keys shows, so the row need not go through stable passes at all.  It
+// is first split into 8192 ranges (bins) of equal width between its smallest and its largest key
+// (4096 for tiles of more than 64 KiB, whose bins share the memory of the digit counters), one LDS
+// atomic per key, which leaves a handful of keys per bin on evenly or normally distributed data; a
+// second atomic puts every key into its bin and tells the key where it went; every key then finds
+// its place inside its bin by counting the keys of the bin that come before it.  A row that
+// crowds more than BUCKET_LIMIT keys into one bin (few different keys, tight clusters) goes
+// through the radix passes instead.  Used by the 1024-thread shapes (rows of more than 4096 real
+// keys of 4 or 8 bytes).
 //
 // Floating-point rows without NaN and without -0.0 (found during the same reduction): on such
 // a row the ordered image of a key is a bijection of its bits, so the keys are replaced by
