@@ -52,11 +52,20 @@
 
 namespace cpn {
 
-// Bins of the split above for a tile of `tile` keys: four per key, 4096 to 8192.
-// (a tile of more than 64 KiB leaves room for 4096 only: they then share the 16 KiB of the digit counters)
-__host__ __device__ constexpr int bucket_bins_log2(int tile, int key_bytes)
+// Bins of the split above: 8192 where they fit beside the row (and the staged positions of an
+// argsort), 4096 (which share the 16 KiB of the digit counters) where that keeps two workgroups on a
+// CU or where nothing more is left of the CU's 160 KiB.
+__host__ __device__ constexpr int bucket_bins_log2(int tile, int key_bytes, bool has_idx)
 {
-  return (tile <= 1024 || tile * key_bytes > 64 * 1024) ? 12 : 13;
+  const int row_bytes = tile * key_bytes + (has_idx ? tile * 2 : 0);
+  constexpr int KIB = 1024;
+  if (row_bytes + 32 * KIB <= 78 * KIB) {
+    return 13;  // two workgroups per CU either way
+  }
+  if (row_bytes + 16 * KIB <= 78 * KIB) {
+    return 12;  // two workgroups per CU only with the smaller table
+  }
+  return row_bytes + 32 * KIB <= 158 * KIB ? 13 : 12;
 }
 // Most keys a bin may hold for the split to be used (each key of a bin is compared with all others).
 constexpr uint32_t BUCKET_LIMIT = 24;
@@ -118,16 +127,16 @@ void lds_row_sort_kernel(const KeyT* keys_in,
   // the split on leading bits: real keys of 4 and 8 bytes, values only
   // (only the 1024-thread shapes, rows of more than 4096 keys: in the smaller shapes the bins cost
   // the LDS that lets many workgroups share a CU, and rows of 1024 float64 keys went from 0.41 to 0.60 ms)
-  constexpr bool BUCKETS_OK = !HAS_IDX && NW == 1 && sizeof(KeyT) >= 4 && sizeof(KeyT) <= 8 && BLOCK == 1024 &&
+  constexpr bool BUCKETS_OK = NW == 1 && sizeof(KeyT) >= 4 && sizeof(KeyT) <= 8 && BLOCK == 1024 &&
                               (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT);
-  constexpr int BINS_LOG2   = bucket_bins_log2(TILE, sizeof(KeyT));
+  constexpr int BINS_LOG2   = bucket_bins_log2(TILE, sizeof(KeyT), HAS_IDX);
   constexpr int BINS        = 1 << BINS_LOG2;
   constexpr int BINS_PER_THREAD = BINS / BLOCK;
   static_assert(!BUCKETS_OK || (BINS_PER_THREAD >= 4 && BINS_PER_THREAD % 4 == 0), "a thread scans whole 16-byte chunks");
 
   // (padded where the split is compiled in: its walk over a bin reads up to BUCKET_LIMIT keys past the bin's end)
   __shared__ __align__(16) KeyT s_keys[TILE + (BUCKETS_OK ? BUCKET_PAD : 0)];
-  __shared__ IdxS s_idx[HAS_IDX ? TILE : 1];
+  __shared__ IdxS s_idx[HAS_IDX ? TILE + (BUCKETS_OK ? BUCKET_PAD : 0) : 1];
   // the per-wave digit counters of the radix passes and the bins of the split share their memory
   // (the split is over, or given up, before the first radix pass clears its counters)
   constexpr int CTR_WORDS = (BUCKETS_OK && BINS > WAVES * RADIX) ? BINS : WAVES * RADIX;
@@ -313,7 +322,11 @@ void lds_row_sort_kernel(const KeyT* keys_in,
   }
   if constexpr (BUCKETS_OK) {
     static_assert(!BUCKETS_OK || !IMAGES_OK, "the split works on the keys' own bits");
-    if (free_first && __builtin_popcount(active) >= 2) {  // uniform
+    // Sorts that carry positions take the split too: a key's place inside its bin then counts the
+    // smaller keys and the equal ones of lower position, which is the stable order; the keys' own
+    // comparison has to be the sort order, so float rows with a NaN or a -0.0 stay out here as well.
+    const bool split_ok = HAS_IDX ? (CODEC != CODEC_FLOAT || any_special == 0) : free_first;
+    if (split_ok && __builtin_popcount(active) >= 2) {  // uniform
       using NT = typename NativeKey<CODEC, sizeof(KeyT)>::type;  // float, double or the integer type
       auto native = [](KeyT k) -> NT {
         NT v;
@@ -452,13 +465,22 @@ void lds_row_sort_kernel(const KeyT* keys_in,
         }
         __syncthreads();
         // every key into its bin, in whatever order the atomics hand out
-        uint32_t self[ITEMS];  // where this thread's key i went
+        // (without positions a key remembers where it went: that breaks the ties of the walk below;
+        // with positions the positions do, and the registers are needed elsewhere)
+        uint32_t self[HAS_IDX ? 1 : ITEMS];
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {
-          self[i] = 0;
+          if constexpr (!HAS_IDX) {
+            self[i] = 0;
+          }
           if (round_runs(i) && holds(i)) {
-            self[i]         = atomicAdd(&s_bins[bin[i]], 1u);
-            s_keys[self[i]] = key[i];
+            const uint32_t went = atomicAdd(&s_bins[bin[i]], 1u);
+            s_keys[went]        = key[i];
+            if constexpr (HAS_IDX) {
+              s_idx[went] = static_cast<IdxS>(idx[i]);
+            } else {
+              self[i] = went;
+            }
           }
         }
         __syncthreads();
@@ -470,7 +492,9 @@ void lds_row_sort_kernel(const KeyT* keys_in,
         // LDS reads in flight instead of one; a read past the end of a bin fetches a key of a later
         // bin, or of the padding, and is not counted.  Eight at a time, not all: the walk's state for
         // 16 keys does not fit the registers of a 1024-thread workgroup.)
-        constexpr int GROUP = ITEMS < 8 ? ITEMS : 8;
+        // (with positions: ties go by the position the key came from, read from LDS beside the key, and
+        // four keys walk at a time)
+        constexpr int GROUP = HAS_IDX ? (ITEMS % 4 == 0 ? 4 : 2) : (ITEMS < 8 ? ITEMS : 8);
         static_assert(ITEMS % GROUP == 0, "whole groups");
 #pragma unroll
         for (int g = 0; g < ITEMS; g += GROUP) {
@@ -487,7 +511,9 @@ void lds_row_sort_kernel(const KeyT* keys_in,
               const uint32_t end = s_bins[bin[i]];
               from[k]            = (bin[i] == 0) ? 0u : s_bins[bin[i] - 1];  // start of the bin
               len[k]             = end - from[k];
-              self[i] -= from[k];
+              if constexpr (!HAS_IDX) {
+                self[i] -= from[k];
+              }
               longest = len[k] > longest ? len[k] : longest;
             }
           }
@@ -495,12 +521,16 @@ void lds_row_sort_kernel(const KeyT* keys_in,
           auto walk = [&](auto every_round) {
             for (uint32_t j = 0; j < longest; ++j) {
               KeyT other[GROUP];
+              uint32_t other_idx[HAS_IDX ? GROUP : 1];
 #pragma unroll
               for (int k = 0; k < GROUP; ++k) {
                 if (!decltype(every_round)::value && !round_runs(g + k)) {
                   break;
                 }
                 other[k] = s_keys[from[k] + j];
+                if constexpr (HAS_IDX) {
+                  other_idx[k] = s_idx[from[k] + j];
+                }
               }
 #pragma unroll
               for (int k = 0; k < GROUP; ++k) {
@@ -509,7 +539,12 @@ void lds_row_sort_kernel(const KeyT* keys_in,
                 }
                 const NT a = native(other[k]), b = native(key[g + k]);
                 // (bitwise, not short-circuit: no branch between the reads of a round)
-                const bool first = (a < b) | ((a == b) & (j < self[g + k]));
+                bool first;
+                if constexpr (HAS_IDX) {
+                  first = (a < b) | ((a == b) & (other_idx[k] < idx[g + k]));
+                } else {
+                  first = (a < b) | ((a == b) & (j < self[g + k]));
+                }
                 before[k] += (first & (j < len[k])) ? 1u : 0u;
               }
             }
@@ -521,14 +556,17 @@ void lds_row_sort_kernel(const KeyT* keys_in,
           }
 #pragma unroll
           for (int k = 0; k < GROUP; ++k) {
-            self[g + k] = from[k] + before[k];  // where the key belongs
+            bin[g + k] = from[k] + before[k];  // where the key belongs (its bin number is no longer needed)
           }
         }
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {
           if (round_runs(i) && holds(i)) {
-            s_keys[self[i]] = key[i];
+            s_keys[bin[i]] = key[i];
+            if constexpr (HAS_IDX) {
+              s_idx[bin[i]] = static_cast<IdxS>(idx[i]);
+            }
           }
         }
         __syncthreads();
@@ -536,6 +574,9 @@ void lds_row_sort_kernel(const KeyT* keys_in,
         for (int i = 0; i < ITEMS; ++i) {
           if (holds(i)) {
             key[i] = s_keys[woff + i * WAVE];
+            if constexpr (HAS_IDX) {
+              idx[i] = s_idx[woff + i * WAVE];
+            }
           }
         }
         todo     = 0;      // sorted: no radix pass is left

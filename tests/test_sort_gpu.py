@@ -197,14 +197,23 @@ def test_lds_rows_split_on_leading_bits(lib, torch_cuda, dtype):
         assert_same_bits(got, want, f"{dt} seg={seg}")
         got, _ = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=False, in_place=True)
         assert_same_bits(got, want, f"{dt} seg={seg} in place")
-    # groups of equal keys of every size around the limit of a bin
-    for group in (2, 23, 24, 25, 40):
-        seg = 4096
-        base = rng.permutation(seg // group + 1).astype(dtype)
-        x = np.repeat(base, group)[:seg].reshape(1, seg).copy()
-        rng.shuffle(x[0])
-        got, _ = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=False)
-        assert_same_bits(got, np.sort(x, axis=-1, kind="stable"), f"{dt} groups of {group}")
+        # sorts that carry positions take the split as well: ties go by position, which is the stable order
+        want_i = np.argsort(x, axis=-1, kind="stable")
+        _, got_i = abi_sort(lib, torch_cuda, x, want_values=False, want_indices=True)
+        assert_same_bits(got_i, want_i, f"{dt} seg={seg} argsort")
+        got, got_i = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=True, offset=7)
+        assert_same_bits(got, want, f"{dt} seg={seg} values with positions")
+        assert_same_bits(got_i, want_i + 7, f"{dt} seg={seg} positions with values")
+    # groups of equal keys of every size around the limit of a bin (24; 48 where 4096 bins serve up to 16 384 keys)
+    for seg, groups in ((8192, (2, 23, 24, 25, 40)), (16384, (24, 47, 48, 49, 100))):
+        for group in groups:
+            base = rng.permutation(seg // group + 1).astype(dtype)
+            x = np.repeat(base, group)[:seg].reshape(1, seg).copy()
+            rng.shuffle(x[0])
+            got, _ = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=False)
+            assert_same_bits(got, np.sort(x, axis=-1, kind="stable"), f"{dt} seg={seg} groups of {group}")
+            _, got_i = abi_sort(lib, torch_cuda, x, want_values=False, want_indices=True)
+            assert_same_bits(got_i, np.argsort(x, axis=-1, kind="stable"), f"{dt} seg={seg} groups of {group}, argsort")
 
 
 @pytest.mark.parametrize("dtype", [np.int32, np.uint32, np.float32])
