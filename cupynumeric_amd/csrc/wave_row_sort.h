@@ -103,8 +103,8 @@ __device__ __forceinline__ T wave_all_or(T v)
 template <int CODEC, typename KeyT, bool HAS_IDX, int ITEMS>
 __host__ __device__ constexpr bool wave_split_ok()
 {
-  return !HAS_IDX && sizeof(KeyT) == 4 && ITEMS <= 8 &&
-         (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT);
+  (void)HAS_IDX;  // with positions too: ties inside a range then go by position, the stable order
+  return sizeof(KeyT) == 4 && ITEMS <= 8 && (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT);
 }
 // ranges (bins) of the split for a tile of `tile` keys; their counters share the memory of the
 // 256 digit counters of the radix passes
@@ -186,7 +186,7 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
         vary_and[n] &= w[i][n];
         vary_or[n] |= w[i][n];
       }
-      if constexpr (CODEC == CODEC_FLOAT && !HAS_IDX) {
+      if constexpr (CODEC == CODEC_FLOAT && (!HAS_IDX || wave_split_ok<CODEC, KeyT, HAS_IDX, ITEMS>())) {
         special = special | is_nan_or_negative_zero(raw);
       }
     } else {
@@ -244,7 +244,13 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
   const bool free_first = !HAS_IDX && (OW::BIJECT || plain_floats);
   bool first_running    = true;
   if constexpr (SPLIT_OK) {
-    if (free_first && __builtin_popcount(active) >= 3) {  // uniform for the wave; fewer varying digits: the passes are cheap
+    // (with positions: the ranges are steps of the value, which a NaN does not have, so float rows
+    // with a NaN, or a -0.0, which the same test reports, keep the passes)
+    bool split_ok = free_first;
+    if constexpr (HAS_IDX) {
+      split_ok = (CODEC != CODEC_FLOAT) || (__builtin_amdgcn_ballot_w64(special) == 0);
+    }
+    if (split_ok && __builtin_popcount(active) >= 3) {  // uniform for the wave; fewer varying digits: the passes are cheap
       // smallest and largest image of the row (image order is key order)
       uint32_t lo = 0xFFFFFFFFu, hi = 0;
 #pragma unroll
@@ -321,13 +327,21 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
         }
         __builtin_amdgcn_wave_barrier();
         // every key into its range, in whatever order the atomics hand out
-        uint32_t self[ITEMS];  // where this lane's key i went
+        auto pos_of = [&](int i) -> uint32_t { return (pos2[i / 2] >> (16 * (i % 2))) & 0xFFFFu; };
+        uint32_t self[HAS_IDX ? 1 : ITEMS];  // where this lane's key i went (without positions: breaks the ties below)
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {
-          self[i] = 0;
+          if constexpr (!HAS_IDX) {
+            self[i] = 0;
+          }
           if (full || (i * WAVE + lane < seg)) {
-            self[i]                   = atomicAdd(&ctr[bin[i]], 1u);
-            s_words[wave][0][self[i]] = w[i][0];
+            const uint32_t went    = atomicAdd(&ctr[bin[i]], 1u);
+            s_words[wave][0][went] = w[i][0];
+            if constexpr (HAS_IDX) {
+              s_pos[wave][went] = static_cast<uint16_t>(pos_of(i));
+            } else {
+              self[i] = went;
+            }
           }
         }
         __builtin_amdgcn_wave_barrier();
@@ -344,21 +358,33 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
           if (full || (i * WAVE + lane < seg)) {
             from[i] = (bin[i] == 0) ? 0u : ctr[bin[i] - 1];
             len[i]  = ctr[bin[i]] - from[i];
-            self[i] -= from[i];
+            if constexpr (!HAS_IDX) {
+              self[i] -= from[i];
+            }
             longest = len[i] > longest ? len[i] : longest;
           }
         }
         for (uint32_t j = 0; j < longest; ++j) {
           uint32_t other[ITEMS];
+          uint32_t other_pos[HAS_IDX ? ITEMS : 1];
 #pragma unroll
           for (int i = 0; i < ITEMS; ++i) {
             const uint32_t at = from[i] + j;
-            other[i]          = s_words[wave][0][at < static_cast<uint32_t>(TILE) ? at : static_cast<uint32_t>(TILE - 1)];
+            const uint32_t in = at < static_cast<uint32_t>(TILE) ? at : static_cast<uint32_t>(TILE - 1);
+            other[i]          = s_words[wave][0][in];
+            if constexpr (HAS_IDX) {
+              other_pos[i] = s_pos[wave][in];
+            }
           }
 #pragma unroll
           for (int i = 0; i < ITEMS; ++i) {
             // (bitwise, not short-circuit: no branch between the reads of a round)
-            const bool first = (other[i] < w[i][0]) | ((other[i] == w[i][0]) & (j < self[i]));
+            bool first;
+            if constexpr (HAS_IDX) {
+              first = (other[i] < w[i][0]) | ((other[i] == w[i][0]) & (other_pos[i] < pos_of(i)));
+            } else {
+              first = (other[i] < w[i][0]) | ((other[i] == w[i][0]) & (j < self[i]));
+            }
             before[i] += (first & (j < len[i])) ? 1u : 0u;
           }
         }
@@ -367,6 +393,9 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
         for (int i = 0; i < ITEMS; ++i) {
           if (full || (i * WAVE + lane < seg)) {
             s_words[wave][0][from[i] + before[i]] = w[i][0];
+            if constexpr (HAS_IDX) {
+              s_pos[wave][from[i] + before[i]] = static_cast<uint16_t>(pos_of(i));
+            }
           }
         }
         __builtin_amdgcn_wave_barrier();
@@ -374,6 +403,10 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
         for (int i = 0; i < ITEMS; ++i) {
           if (full || (i * WAVE + lane < seg)) {
             w[i][0] = s_words[wave][0][i * WAVE + lane];
+            if constexpr (HAS_IDX) {
+              const uint32_t p = s_pos[wave][i * WAVE + lane];
+              pos2[i / 2]      = (i % 2 == 0) ? ((pos2[i / 2] & 0xFFFF0000u) | p) : ((pos2[i / 2] & 0xFFFFu) | (p << 16));
+            }
           }
         }
         __builtin_amdgcn_wave_barrier();

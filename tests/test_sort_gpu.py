@@ -251,10 +251,25 @@ def test_wave_rows_split_into_ranges(lib, torch_cuda, dtype):
         assert_same_bits(got, want, f"{dt} seg={seg}")
         got, _ = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=False, in_place=True)
         assert_same_bits(got, want, f"{dt} seg={seg} in place")
+        # with positions the split runs as well and ties go by position; rows with zeros and NaNs keep the passes
+        want_i = np.argsort(x, axis=-1, kind="stable")
+        _, got_i = abi_sort(lib, torch_cuda, x, want_values=False, want_indices=True)
+        assert_same_bits(got_i, want_i, f"{dt} seg={seg} argsort")
+        got, got_i = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=True, offset=3)
+        assert_same_bits(got, want, f"{dt} seg={seg} values with positions")
+        assert_same_bits(got_i, want_i + 3, f"{dt} seg={seg} positions with values")
+        if dt.kind == "f":
+            y = x.copy()
+            y[0, ::5] = np.nan
+            y[1, ::4] = -0.0
+            y[1, 1::4] = 0.0
+            check_rows(lib, torch_cuda, y, f"{dt} seg={seg} rows with NaN and zeros")
     big = rng.standard_normal((20000, 128)).astype(np.float32).view(np.uint32).view(dtype) if dt.kind != "f" else \
         rng.standard_normal((20000, 128)).astype(dtype)
     got, _ = abi_sort(lib, torch_cuda, big, want_values=True, want_indices=False)
     assert_same_bits(got, np.sort(big, axis=-1, kind="stable"), f"{dt} many rows of 128")
+    _, got_i = abi_sort(lib, torch_cuda, big, want_values=False, want_indices=True)
+    assert_same_bits(got_i, np.argsort(big, axis=-1, kind="stable"), f"{dt} many rows of 128, argsort")
 
 
 def test_lds_many_short_rows(lib, torch_cuda):
