@@ -31,8 +31,11 @@
 // second atomic puts every key into its bin and tells the key where it went; every key then finds
 // its place inside its bin by counting the keys of the bin that come before it.  A row that
 // crowds more than BUCKET_LIMIT keys into one bin (few different keys, tight clusters) goes
-// through the radix passes instead.  Used by the 1024-thread shapes (rows of more than 4096 real
-// keys of 4 or 8 bytes).
+// through the radix passes instead.  Used by every shape of at least 128 threads, for real keys of
+// 4 or 8 bytes (4-byte keys in rows of up to 1024 are sorted by one wave each, wave_row_sort.h, which
+// has the same path); two bins per key for rows of up to 2048 keys.  Sorts that carry positions take
+// it as well: the position a key came from is staged beside the key and breaks the ties inside a
+// bin, which makes the result the stable order.
 //
 // Floating-point rows without NaN and without -0.0 (found during the same reduction): on such
 // a row the ordered image of a key is a bijection of its bits, so the keys are replaced by
@@ -59,6 +62,9 @@ __host__ __device__ constexpr int bucket_bins_log2(int tile, int key_bytes, bool
 {
   const int row_bytes = tile * key_bytes + (has_idx ? tile * 2 : 0);
   constexpr int KIB = 1024;
+  if (tile <= 2048) {
+    return tile <= 1024 ? 11 : 12;  // two bins per key
+  }
   if (row_bytes + 32 * KIB <= 78 * KIB) {
     return 13;  // two workgroups per CU either way
   }
@@ -127,7 +133,11 @@ void lds_row_sort_kernel(const KeyT* keys_in,
   // the split on leading bits: real keys of 4 and 8 bytes, values only
   // (only the 1024-thread shapes, rows of more than 4096 keys: in the smaller shapes the bins cost
   // the LDS that lets many workgroups share a CU, and rows of 1024 float64 keys went from 0.41 to 0.60 ms)
-  constexpr bool BUCKETS_OK = NW == 1 && sizeof(KeyT) >= 4 && sizeof(KeyT) <= 8 && BLOCK == 1024 &&
+  // (every shape of at least 128 threads: measured on 2^26 keys, passes / split: rows of 1024 float64 0.35 / 0.30 ms,
+  // 2048 float64 0.47 / 0.34, 4096 float64 0.50 / 0.37, 1500 float32 0.48 / 0.30, 2048 float32 0.36 / 0.25,
+  // 4096 int32 0.35 / 0.30; with positions 2048 float32 0.43 / 0.32, 2048 float64 0.55 / 0.40 ms)
+  constexpr bool BUCKETS_SHAPE = BLOCK >= 128 && ITEMS >= 8;
+  constexpr bool BUCKETS_OK = NW == 1 && sizeof(KeyT) >= 4 && sizeof(KeyT) <= 8 && BUCKETS_SHAPE &&
                               (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT);
   constexpr int BINS_LOG2   = bucket_bins_log2(TILE, sizeof(KeyT), HAS_IDX);
   constexpr int BINS        = 1 << BINS_LOG2;
@@ -235,7 +245,7 @@ void lds_row_sort_kernel(const KeyT* keys_in,
     }
   }
   const int any_special = __syncthreads_or(special);
-  const bool images     = IMAGES_OK && (any_special == 0);
+  bool images           = IMAGES_OK && (any_special == 0);
   // Sorts that return keys only: the first pass to run need not be stable.  Keys that tie in every
   // digit are the same bits (float rows with a NaN or a -0.0, where different bits tie, are left
   // out; so are complex keys), so nothing shows in which order that pass leaves equal digits, and
@@ -312,16 +322,7 @@ void lds_row_sort_kernel(const KeyT* keys_in,
     }
     KT::words(k, w);
   };
-  if constexpr (IMAGES_OK) {
-    if (images) {
-#pragma unroll
-      for (int i = 0; i < ITEMS; ++i) {
-        key[i] = sign_flip(key[i]);
-      }
-    }
-  }
   if constexpr (BUCKETS_OK) {
-    static_assert(!BUCKETS_OK || !IMAGES_OK, "the split works on the keys' own bits");
     // Sorts that carry positions take the split too: a key's place inside its bin then counts the
     // smaller keys and the equal ones of lower position, which is the stable order; the keys' own
     // comparison has to be the sort order, so float rows with a NaN or a -0.0 stay out here as well.
@@ -379,7 +380,7 @@ void lds_row_sort_kernel(const KeyT* keys_in,
       __syncthreads();
       // (every lane takes the extremes of one wave, four exchanges inside each group of 16 lanes
       // merge them; minimum and maximum do not mind seeing a wave several times)
-      static_assert(WAVES == 16, "one wave per lane of a 16-lane group");
+      static_assert(WAVES <= WAVE && (WAVES & (WAVES - 1)) == 0, "one wave per lane of a group of WAVES lanes");
       lo = s_ext[lane % WAVES];
       hi = s_ext[WAVES + lane % WAVES];
 #pragma unroll
@@ -581,6 +582,16 @@ void lds_row_sort_kernel(const KeyT* keys_in,
         }
         todo     = 0;      // sorted: no radix pass is left
         shortcut = false;
+      }
+    }
+  }
+  // (after the split, which works on the keys' own bits; a row that the split has sorted needs no images)
+  images = images && todo != 0;
+  if constexpr (IMAGES_OK) {
+    if (images) {
+#pragma unroll
+      for (int i = 0; i < ITEMS; ++i) {
+        key[i] = sign_flip(key[i]);
       }
     }
   }

@@ -93,8 +93,8 @@ __device__ __forceinline__ T wave_all_or(T v)
   return v;
 }
 
-// Values-only sorts of real 4-byte keys whose ties are the same bits (integers; floats without NaN
-// and -0.0) need no stable passes: the row is split into ranges of equal width between its smallest
+// Sorts of real 4-byte keys whose ties are the same bits (integers; floats without NaN and -0.0) or
+// whose ties can go by the position carried with every key (argsort) need no stable passes: the row is split into ranges of equal width between its smallest
 // and largest key, two per key, with one LDS atomic per key, and every key then counts the smaller
 // keys of its range (the same idea as in the one-workgroup-per-row kernel, lds_row_sort.h, here
 // within one wave and without any barrier).  A row that crowds a range takes the radix passes.
