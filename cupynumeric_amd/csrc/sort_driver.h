@@ -471,9 +471,11 @@ inline int sort_rows_in_lds(const SortRequest& r)
     return launch_lds_rows<KeyT, CODEC, HAS_IDX, 1024, 4>(r);  // lds_row_capacity(16) == 4096
   } else {
     if (r.seg <= 4096) {
-      // eight keys per thread when a thread also carries positions or 8-byte keys (10-25 % faster
-      // than sixteen there), sixteen for plain sorts of narrower keys
-      if constexpr (HAS_IDX || sizeof(KeyT) == 8) {
+      // eight keys per thread when a thread also carries positions (10-25 % faster than sixteen) and
+      // for keys of 4 and 8 bytes, whose rows are split into value ranges (twice the waves per CU:
+      // 2^26 float32 keys in rows of 4096 0.33 -> 0.27 ms, of 2049 0.57 -> 0.42); sixteen for plain
+      // sorts of 1- and 2-byte keys
+      if constexpr (HAS_IDX || sizeof(KeyT) >= 4) {
         return launch_lds_rows<KeyT, CODEC, HAS_IDX, 512, 8>(r);
       } else {
         return launch_lds_rows<KeyT, CODEC, HAS_IDX, 256, 16>(r);
