@@ -62,8 +62,13 @@ __host__ __device__ constexpr int bucket_bins_log2(int tile, int key_bytes, bool
 {
   const int row_bytes = tile * key_bytes + (has_idx ? tile * 2 : 0);
   constexpr int KIB = 1024;
-  if (tile <= 2048) {
-    return tile <= 1024 ? 11 : 12;  // two bins per key
+  if (tile <= 4096) {
+    // One bin per key; two for plain sorts of 4-byte keys.  More bins shorten the walks and cost LDS,
+    // i.e. workgroups per CU, which weighs more.  Measured on 2^26 keys, two / one / half a bin per key:
+    // rows of 1024 float64 0.28 / 0.26 / 0.26 ms (four per key: 0.43), 2048 float64 0.34 / 0.28 / 0.30,
+    // 4096 float64 0.38 / 0.32 / 0.33, 4096 float32 with positions 0.39 / 0.34 / 0.41, and plain
+    // 4096 float32 0.275 / 0.281 / 0.327, 2048 float32 0.259 / 0.266 / 0.302.
+    return (tile <= 1024 ? 10 : (tile <= 2048 ? 11 : 12)) + ((key_bytes == 4 && !has_idx) ? 1 : 0);
   }
   if (row_bytes + 32 * KIB <= 78 * KIB) {
     return 13;  // two workgroups per CU either way
