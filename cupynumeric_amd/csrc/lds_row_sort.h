@@ -58,7 +58,7 @@ namespace cpn {
 // Bins of the split above: 8192 where they fit beside the row (and the staged positions of an
 // argsort), 4096 (which share the 16 KiB of the digit counters) where that keeps two workgroups on a
 // CU or where nothing more is left of the CU's 160 KiB.
-__host__ __device__ constexpr int bucket_bins_log2(int tile, int key_bytes, bool has_idx)
+__host__ __device__ constexpr int bucket_bins_log2(int tile, int key_bytes, bool has_idx, int block)
 {
   const int row_bytes = tile * key_bytes + (has_idx ? tile * 2 : 0);
   constexpr int KIB = 1024;
@@ -75,6 +75,11 @@ __host__ __device__ constexpr int bucket_bins_log2(int tile, int key_bytes, bool
   }
   if (row_bytes + 16 * KIB <= 78 * KIB) {
     return 12;  // two workgroups per CU only with the smaller table
+  }
+  if (block <= 512 && row_bytes + 8 * KIB <= 78 * KIB) {
+    // 8192 eight-byte keys on 512 threads: a quarter of a bin per key, and two workgroups per CU
+    // (1024 threads with more than 64 registers each have a CU to themselves anyway)
+    return 11;
   }
   return row_bytes + 32 * KIB <= 158 * KIB ? 13 : 12;
 }
@@ -144,7 +149,7 @@ void lds_row_sort_kernel(const KeyT* keys_in,
   constexpr bool BUCKETS_SHAPE = BLOCK >= 128 && ITEMS >= 8;
   constexpr bool BUCKETS_OK = NW == 1 && sizeof(KeyT) >= 4 && sizeof(KeyT) <= 8 && BUCKETS_SHAPE &&
                               (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT);
-  constexpr int BINS_LOG2   = bucket_bins_log2(TILE, sizeof(KeyT), HAS_IDX);
+  constexpr int BINS_LOG2   = bucket_bins_log2(TILE, sizeof(KeyT), HAS_IDX, BLOCK);
   constexpr int BINS        = 1 << BINS_LOG2;
   constexpr int BINS_PER_THREAD = BINS / BLOCK;
   static_assert(!BUCKETS_OK || (BINS_PER_THREAD >= 4 && BINS_PER_THREAD % 4 == 0), "a thread scans whole 16-byte chunks");
@@ -500,7 +505,7 @@ void lds_row_sort_kernel(const KeyT* keys_in,
         // 16 keys does not fit the registers of a 1024-thread workgroup.)
         // (with positions: ties go by the position the key came from, read from LDS beside the key, and
         // four keys walk at a time)
-        constexpr int GROUP = HAS_IDX ? (ITEMS % 4 == 0 ? 4 : 2) : (ITEMS < 8 ? ITEMS : 8);
+        constexpr int GROUP = HAS_IDX ? (ITEMS % 4 == 0 ? 4 : 2) : (ITEMS < 8 ? ITEMS : (ITEMS % 8 == 0 ? 8 : (ITEMS % 4 == 0 ? 4 : 2)));
         static_assert(ITEMS % GROUP == 0, "whole groups");
 #pragma unroll
         for (int g = 0; g < ITEMS; g += GROUP) {
