@@ -127,11 +127,11 @@ def make_config(name: str, log2n: int | None = None, rows: int | None = None) ->
 # Row lengths on either side of every length at which the library changes kernels (--edges): key type,
 # operation, lengths whose successor is timed too; 2^26 keys per run.
 EDGE_LENGTHS = (
-    ("float32", "sort", (32, 1024, 2048, 4096, 8192, 16384, 32768)),
-    ("float64", "sort", (512, 2048, 4096, 8192, 16384, 32768)),
+    ("float32", "sort", (32, 1024, 2048, 4096, 6144, 8192, 12288, 16384, 32768, 65536)),
+    ("float64", "sort", (512, 2048, 4096, 6144, 8192, 16384, 32768, 65536, 1048576)),
     ("float16", "sort", (4096, 8192, 16384)),
-    ("float32", "argsort", (4096, 8192, 16384, 32768)),
-    ("float64", "argsort", (4096, 8192, 14336, 28672)),
+    ("float32", "argsort", (4096, 6144, 8192, 16384, 32768, 65536)),
+    ("float64", "argsort", (4096, 6144, 8192, 14336, 28672, 57344, 458752)),
 )
 
 
@@ -746,13 +746,17 @@ def run_sort_workload(name: str, steps: int, warmup: int, log2n=None, rows=None,
     for label in ("histogram", "virtual_histogram", "distinct_sweep"):
         if label in by_label and cfg["x"].nbytes >= (1 << 26) and max(by_label[label]) < 0.02:
             by_label[label + "_skipped"] = by_label.pop(label)
-    merged_halves = "merge_halves" in by_label  # rows of up to twice the LDS capacity: two half-row sorts and a merge
+    merged_halves = "merge_halves" in by_label  # rows longer than the LDS capacity: sorted pieces, merged level by level
     alg = algorithmic_bytes(cfg, job.uses_lds_rows or merged_halves, passes_run)
+    merge_levels = 0
     if merged_halves:
         n, kb, pos = cfg["x"].size, cfg["x"].dtype.itemsize, (8 if cfg["op"] == "argsort" else 0)
+        merge_levels = round(len(by_label["merge_halves"]) / profile_steps)
         dominant = "lds_row_sort"
-        alg[dominant] = (n // 2) * (kb + kb + pos)  # per launch: half of every row read, written with its positions
-        alg["merge_halves"] = n * (kb + pos) + n * (pos if pos else kb)
+        alg[dominant] = n * (kb + kb + pos)  # every piece read, written with its positions
+        # per launch, averaged over the levels: all but the last read and write keys and positions, the
+        # last one writes the requested output only
+        alg["merge_halves"] = ((2 * merge_levels - 1) * n * (kb + pos) + n * (pos if pos else kb)) / merge_levels
     elif job.uses_lds_rows:  # whichever of the per-row kernels the row length selects
         dominant = next(k for k in ROW_KERNELS if k in by_label)
         alg[dominant] = alg["lds_row_sort"]
@@ -791,7 +795,7 @@ def run_sort_workload(name: str, steps: int, warmup: int, log2n=None, rows=None,
         "ms_per_step_min": float(np.min(per_step)),
         "dtype": {1: "u8", 2: "u16", 4: "u32", 8: "u64"}[cfg["x"].dtype.itemsize],
         "config": {"workload": cfg["workload"], "keys": int(cfg["x"].size), "op": cfg["op"],
-                   "path": ("lds_row_sort on half rows + merge_halves" if merged_halves else dominant)
+                   "path": (f"lds_row_sort on {1 << merge_levels} pieces of a row + {merge_levels} x merge_halves" if merged_halves else dominant)
                    if (job.uses_lds_rows or merged_halves) else f"onesweep, 8-bit digits, {passes_run} passes ran",
                    "workspace_bytes": int(job.temp_bytes)},
         "roofline": roofline,

@@ -118,8 +118,10 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(lds_row_w
 void lds_row_sort_kernel(const KeyT* keys_in,
                                                               KeyT* keys_out,
                                                               int64_t* idx_out,
-                                                              uint32_t seg,
+                                                              uint32_t piece_len,
                                                               uint64_t row_stride,
+                                                              uint32_t pieces,
+                                                              uint32_t last_piece_len,
                                                               int64_t index_offset,
                                                               uint32_t* status)
 {
@@ -168,7 +170,18 @@ void lds_row_sort_kernel(const KeyT* keys_in,
   const int tid       = threadIdx.x;
   const int lane      = tid & (WAVE - 1);
   const int wave      = tid / WAVE;
-  const uint64_t base = static_cast<uint64_t>(blockIdx.x) * row_stride;  // (row_stride == seg: dense rows)
+  // A workgroup sorts one piece of a row: the whole row (pieces == 1; row_stride == piece_len where the
+  // rows are dense), or, for rows that are merged afterwards, piece number blockIdx.x % pieces of row
+  // blockIdx.x / pieces; the last piece of a row may be shorter, and positions count from the row's start.
+  uint32_t seg  = piece_len;
+  uint64_t base = static_cast<uint64_t>(blockIdx.x) * row_stride;
+  if (pieces > 1) {
+    const uint32_t row   = blockIdx.x / pieces;
+    const uint32_t piece = blockIdx.x - row * pieces;
+    base                 = static_cast<uint64_t>(row) * row_stride + static_cast<uint64_t>(piece) * piece_len;
+    index_offset += static_cast<int64_t>(piece) * piece_len;
+    seg = piece + 1 == pieces ? last_piece_len : piece_len;
+  }
   const bool full     = (seg == TILE);
   // A row shorter than the tile is dealt in equal contiguous shares of whole 64-key rounds, so that
   // every wave works on `rounds` keys per lane and the cost follows the row length, not the tile.

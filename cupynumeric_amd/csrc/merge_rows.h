@@ -1,13 +1,14 @@
-// Rows a little too long for the per-row kernels: every row is sorted as two halves by the
-// one-workgroup-per-row kernel (each half fits the LDS of a CU) and the halves are merged here.
+// Rows too long for the per-row kernels: every row is cut into 2^levels pieces of equal length (the
+// last one may be shorter), each sorted by the one-workgroup-per-row kernel (a piece fits the LDS of
+// a CU), and neighbouring pieces are merged here, level by level, until the row is one run.
 // One read and one write of HBM per element and step, against one pass per key byte, per-row
 // histograms and tiles that end at every row on the global path.
 //
-// Stands, for rows of up to twice the LDS capacity, where the reference runs
-// cub::DeviceSegmentedRadixSort (src/cupynumeric/sort/cub_sort.cuh:81-105,153-182).
+// Stands, for these rows, where the reference runs cub::DeviceSegmentedRadixSort
+// (src/cupynumeric/sort/cub_sort.cuh:81-105,153-182).
 //
-// The merge is stable: of two keys that tie, the one from the first half (the lower positions of
-// the row) comes first, and inside a half the stable row sort has kept input order.
+// The merge is stable: of two keys that tie, the one from the first piece of a pair (the lower
+// positions of the row) comes first, and inside a piece the stable row sort has kept input order.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -18,7 +19,10 @@
 
 namespace cpn {
 
-constexpr int MERGE_ITEMS = 8;
+#ifndef CPN_MERGE_ITEMS
+#define CPN_MERGE_ITEMS 8
+#endif
+constexpr int MERGE_ITEMS = CPN_MERGE_ITEMS;
 // Threads of a workgroup, which merges MERGE_ITEMS outputs per thread: 512 for keys alone (the
 // kernel's time is trips to memory, so large chunks: 2^26 float32 keys in rows of 16 385 0.26 -> 0.23 ms
 // against 256), 256 when int64 positions are staged beside the keys (56 KiB of LDS with 512 left two
@@ -27,17 +31,90 @@ __host__ __device__ constexpr int merge_block(bool has_idx) { return has_idx ? 2
 __host__ __device__ constexpr int merge_chunk(bool has_idx) { return merge_block(has_idx) * MERGE_ITEMS; }
 constexpr int MERGE_CHUNK_MIN = 256 * MERGE_ITEMS;  // the smaller of the two: bounds the grid
 
-// keys / idx: the rows with both halves sorted, [rows][n]; half 0 is [0, h), half 1 [h, n).
-// idx holds the final int64 row positions of the elements (those of half 1 already count from h).
-// keys_out may be nullptr (index-only sorts), idx / idx_out are nullptr unless HAS_IDX.
+// Where a workgroup of the merge starts: blockIdx.x -> row, pair of pieces in the row, chunk of the pair's outputs.
+struct MergeChunk {
+  uint64_t first;  // of the pair, in keys / idx and in the outputs
+  uint32_t len_a, len_b;  // the two pieces (len_b == 0: nothing to merge with)
+  uint32_t d0;            // first merged output of the chunk, counted inside the pair
+};
+__device__ inline MergeChunk merge_chunk_of(
+  uint32_t block, uint32_t n, uint32_t piece, uint32_t chunks_per_pair, uint32_t pairs_per_row, uint32_t chunk_len)
+{
+  uint64_t row;
+  uint32_t pair, chunk;
+  if (pairs_per_row == 1) {
+    row   = block / chunks_per_pair;
+    pair  = 0;
+    chunk = block - static_cast<uint32_t>(row * chunks_per_pair);
+  } else {
+    const uint32_t per_row = pairs_per_row * chunks_per_pair;
+    row                    = block / per_row;
+    const uint32_t rest    = block - static_cast<uint32_t>(row * per_row);
+    pair                   = rest / chunks_per_pair;
+    chunk                  = rest - pair * chunks_per_pair;
+  }
+  const uint64_t start = 2ull * pair * piece;  // of this pair in its row; start < n
+  const uint32_t left  = n - static_cast<uint32_t>(start);
+  MergeChunk c;
+  c.first = row * n + start;
+  c.len_a = left < piece ? left : piece;
+  c.len_b = left - c.len_a < piece ? left - c.len_a : piece;
+  c.d0    = chunk * chunk_len;
+  return c;
+}
+
+// How many of the outputs before a chunk come from the first piece of its pair, for every chunk
+// of the merge launch that follows (one thread each): the smallest i with !(a[i] <= b[d0 - 1 - i]).
+// Done ahead of the merge because a search inside its workgroups, with one candidate per thread,
+// touched a cache line per candidate, four times the lines of the chunk itself.
+constexpr int MERGE_SPLIT_BLOCK = 256;
+template <typename KeyT, int CODEC>
+__global__ __launch_bounds__(MERGE_SPLIT_BLOCK) void merge_split_kernel(const KeyT* __restrict__ keys,
+                                                                        uint32_t* __restrict__ splits,
+                                                                        uint32_t n,
+                                                                        uint32_t piece,
+                                                                        uint32_t chunks_per_pair,
+                                                                        uint32_t pairs_per_row,
+                                                                        uint32_t chunk_len,
+                                                                        uint32_t chunks_total)
+{
+  const uint32_t g = blockIdx.x * MERGE_SPLIT_BLOCK + threadIdx.x;
+  if (g >= chunks_total) {
+    return;
+  }
+  const MergeChunk c = merge_chunk_of(g, n, piece, chunks_per_pair, pairs_per_row, chunk_len);
+  const uint32_t d   = c.d0 < c.len_a + c.len_b ? c.d0 : c.len_a + c.len_b;  // (chunks past the end of a short pair)
+  const KeyT* a      = keys + c.first;
+  const KeyT* b      = a + c.len_a;
+  uint32_t lo = d > c.len_b ? d - c.len_b : 0u, hi = d < c.len_a ? d : c.len_a;
+  while (lo < hi) {
+    const uint32_t mid = (lo + hi) / 2;
+    if (ordered_bits<CODEC, KeyT>(a[mid]) <= ordered_bits<CODEC, KeyT>(b[d - 1 - mid])) {
+      lo = mid + 1;
+    } else {
+      hi = mid;
+    }
+  }
+  splits[g] = lo;
+}
+
+// keys / idx: the rows, [rows][n], every row in sorted pieces of `piece` elements: [0, piece),
+// [piece, 2 piece), ... (the last one ends at n).  Pieces 2p and 2p + 1 of a row are merged into
+// [2p piece, (2p + 2) piece) of the outputs; a piece without a partner is copied.
+// idx holds the final int64 row positions of the elements (they count from the start of the row).
+// keys_out may be nullptr (index-only sorts, last level), idx / idx_out are nullptr unless HAS_IDX.
+// splits: merge_split_kernel's output for this launch.
+// Grid: rows x pairs_per_row x chunks_per_pair workgroups, chunks_per_pair = ceil(2 piece / merge_chunk).
 template <typename KeyT, int CODEC, bool HAS_IDX>
 __global__ __launch_bounds__(merge_block(HAS_IDX)) void merge_halves_kernel(const KeyT* __restrict__ keys,
                                                                     const int64_t* __restrict__ idx,
                                                                     KeyT* __restrict__ keys_out,
                                                                     int64_t* __restrict__ idx_out,
+                                                                    const uint32_t* __restrict__ splits,
                                                                     uint32_t n,
-                                                                    uint32_t h,
-                                                                    uint32_t chunks_per_row)
+                                                                    uint32_t piece,
+                                                                    uint32_t chunks_per_pair,
+                                                                    uint32_t pairs_per_row)
 {
   constexpr int MERGE_BLOCK = merge_block(HAS_IDX);
   constexpr int MERGE_CHUNK = merge_chunk(HAS_IDX);
@@ -45,55 +122,24 @@ __global__ __launch_bounds__(merge_block(HAS_IDX)) void merge_halves_kernel(cons
   __shared__ int64_t s_idx[HAS_IDX ? MERGE_CHUNK : 1];
   __shared__ uint16_t s_src[HAS_IDX ? MERGE_CHUNK : 1];
 
-  const int tid        = threadIdx.x;
-  const uint64_t row   = blockIdx.x / chunks_per_row;
-  const uint32_t chunk = blockIdx.x - static_cast<uint32_t>(row * chunks_per_row);
-  const KeyT* a        = keys + row * n;  // first half, len_a keys
-  const KeyT* b        = a + h;           // second half, len_b keys
-  const uint32_t len_a = h, len_b = n - h;
-  const uint32_t d0    = chunk * MERGE_CHUNK;
-  const uint32_t d1    = (d0 + MERGE_CHUNK < n) ? d0 + MERGE_CHUNK : n;
+  const int tid      = threadIdx.x;
+  const MergeChunk c = merge_chunk_of(blockIdx.x, n, piece, chunks_per_pair, pairs_per_row, MERGE_CHUNK);
+  const uint32_t len_a = c.len_a, len_b = c.len_b, d0 = c.d0;
+  const uint32_t h = len_a;  // the second piece starts here
+  if (d0 >= len_a + len_b) {
+    return;  // (the whole workgroup: the last pair of a row may be short)
+  }
+  const bool ends      = d0 + MERGE_CHUNK >= len_a + len_b;  // the pair ends in this chunk
+  const uint32_t d1    = ends ? len_a + len_b : d0 + MERGE_CHUNK;
+  const uint64_t first = c.first;
+  const KeyT* a        = keys + first;  // first piece, len_a keys
 
   auto image = [](KeyT k) { return ordered_bits<CODEC, KeyT>(k); };
 
-  // How many of the first d merged keys come from the first half: the smallest i with
-  // !(a[i] <= b[d - 1 - i]).  The whole workgroup looks for it, one candidate per thread and round, for both
-  // ends of its chunk in the same rounds (two rounds for halves of up to 65 536 keys: every round
-  // is a trip to memory, which is what this kernel's time is made of, hence the large chunks).
-  uint32_t lo[2], hi[2];
-  const uint32_t dd[2] = {d0, d1};
-#pragma unroll
-  for (int e = 0; e < 2; ++e) {
-    lo[e] = dd[e] > len_b ? dd[e] - len_b : 0u;
-    hi[e] = dd[e] < len_a ? dd[e] : len_a;
-  }
-  while (lo[0] < hi[0] || lo[1] < hi[1]) {  // uniform
-    uint32_t step[2];
-    int below[2];
-#pragma unroll
-    for (int e = 0; e < 2; ++e) {
-      step[e]             = (hi[e] - lo[e] + MERGE_BLOCK - 1) / MERGE_BLOCK;
-      const uint32_t cand = lo[e] + static_cast<uint32_t>(tid) * step[e];
-      below[e]            = 0;
-      if (cand < hi[e]) {
-        below[e] = image(a[cand]) <= image(b[dd[e] - 1 - cand]) ? 1 : 0;
-      }
-    }
-#pragma unroll
-    for (int e = 0; e < 2; ++e) {
-      const uint32_t k = static_cast<uint32_t>(__syncthreads_count(below[e]));  // candidates before the split: a prefix
-      if (lo[e] < hi[e]) {
-        if (k == 0) {
-          hi[e] = lo[e];
-        } else {
-          const uint32_t new_hi = lo[e] + k * step[e];
-          lo[e]                 = lo[e] + (k - 1) * step[e] + 1;
-          hi[e]                 = new_hi < hi[e] ? new_hi : hi[e];
-        }
-      }
-    }
-  }
-  const uint32_t a0 = lo[0], a1 = lo[1];
+  // how many of the outputs before the chunk, and before the next one, come from the first piece
+  // (merge_split_kernel; the next chunk of the pair is the next workgroup)
+  const uint32_t a0 = splits[blockIdx.x];
+  const uint32_t a1 = ends ? len_a : splits[blockIdx.x + 1];
   const uint32_t b0 = d0 - a0, b1 = d1 - a1;
   const uint32_t na = a1 - a0, nb = b1 - b0, total = d1 - d0;
 
@@ -109,7 +155,7 @@ __global__ __launch_bounds__(merge_block(HAS_IDX)) void merge_halves_kernel(cons
       const uint32_t src = jj < na ? a0 + jj : h + b0 + (jj - na);
       v[k]               = a[src];
       if constexpr (HAS_IDX) {
-        p[k] = idx[row * n + src];
+        p[k] = idx[first + src];
       }
     }
 #pragma unroll
@@ -142,7 +188,7 @@ __global__ __launch_bounds__(merge_block(HAS_IDX)) void merge_halves_kernel(cons
   // the heads of both runs stay in registers; a step reads only the successor of the key it took
   // (positions past the end of a run are clamped: their keys are read and never taken)
   KeyT head_a = s_key[ia < na ? ia : (na != 0 ? na - 1 : 0)];
-  KeyT head_b = s_key[na + (ib < nb ? ib : (nb != 0 ? nb - 1 : 0))];
+  KeyT head_b = s_key[nb != 0 ? na + (ib < nb ? ib : nb - 1) : 0];
 #pragma unroll
   for (int k = 0; k < MERGE_ITEMS; ++k) {
     out_key[k] = KeyT{};
@@ -170,7 +216,7 @@ __global__ __launch_bounds__(merge_block(HAS_IDX)) void merge_halves_kernel(cons
     }
   }
   __syncthreads();
-  const uint64_t out_base = row * n + d0;
+  const uint64_t out_base = first + d0;
 #pragma unroll
   for (int k = 0; k < MERGE_ITEMS; ++k) {
     const uint32_t j = static_cast<uint32_t>(tid) + k * MERGE_BLOCK;

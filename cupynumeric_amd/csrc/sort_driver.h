@@ -116,22 +116,46 @@ uint64_t count16_min_row();
 // to send every request down the global path for an A/B run.
 uint64_t lds_row_limit(int key_bytes, bool with_positions);
 
-// Rows longer than the per-row kernels take, up to twice that length: sorted as two halves by the
-// per-row kernel and merged (merge_rows.h) instead of going down the global path.  Real keys of 4
-// and 8 bytes.  Off when cpn_set_merge_rows(0) / CPN_SORT_MERGE_ROWS=0 says so, and whenever the
-// LDS row limit has been lowered (an A/B run that wants the global path gets it).
+// Rows longer than the per-row kernels take: cut into 2^levels pieces that the per-row kernel sorts,
+// merged pairwise level by level (merge_rows.h) instead of going down the global path.  Real keys
+// of 4 and 8 bytes.  Off when cpn_set_merge_rows(0) / CPN_SORT_MERGE_ROWS=0 says so, and whenever
+// the LDS row limit has been lowered (an A/B run that wants the global path gets it).
+// merge_levels_limit: the most levels for which this beats the global path, whose cost is one pass
+// per key byte whatever the row length, while every level here is one read and one write of the rows.
 bool merge_rows_enabled();
-inline bool merged_rows_apply(int key_bytes, int passes, uint64_t volume, uint64_t seg, bool want_indices)
+int merge_levels_limit(int key_bytes, bool want_indices);
+// Levels of merging for rows of seg elements: 0 = the request does not take this path.
+inline int merged_row_levels(int key_bytes, int passes, uint64_t volume, uint64_t seg, bool want_indices)
 {
   if (!merge_rows_enabled() || (key_bytes != 4 && key_bytes != 8) || passes != key_bytes || volume == 0) {
-    return false;
+    return 0;
   }
   const uint64_t cap = lds_row_capacity(key_bytes, want_indices);
-  if (lds_row_limit(key_bytes, want_indices) != cap || seg <= cap || seg > 2 * cap) {
-    return false;
+  if (lds_row_limit(key_bytes, want_indices) != cap || seg <= cap) {
+    return 0;
   }
-  const uint64_t chunks = (seg + MERGE_CHUNK_MIN - 1) / MERGE_CHUNK_MIN;
-  return (volume / seg) * chunks < (1ull << 31);  // one workgroup of the merge per chunk of a row
+  const int limit = merge_levels_limit(key_bytes, want_indices);
+  int levels      = 1;
+  while ((cap << levels) < seg) {
+    if (++levels > limit) {
+      return 0;
+    }
+  }
+  if (levels > limit) {
+    return 0;
+  }
+  // one workgroup of a merge per chunk of a pair of pieces, one of the per-row kernel per piece
+  const uint64_t per_row = (seg + MERGE_CHUNK_MIN - 1) / MERGE_CHUNK_MIN + (1ull << levels);
+  return (volume / seg) * per_row < (1ull << 31) ? levels : 0;
+}
+// Length of the pieces (the last one of a row may be shorter).
+inline uint64_t merged_row_piece(uint64_t seg, int levels) { return (seg + (1ull << levels) - 1) >> levels; }
+// Bytes of the table of chunk starts that a level of merging reads (one word per workgroup of the
+// largest merge launch; every level reuses it).
+inline uint64_t merged_row_split_bytes(uint64_t volume, uint64_t seg, int levels)
+{
+  const uint64_t per_row = (seg + MERGE_CHUNK_MIN - 1) / MERGE_CHUNK_MIN + (1ull << levels);
+  return align_up((volume / seg) * per_row * sizeof(uint32_t), WORKSPACE_ALIGN);
 }
 
 // Element type code (enum cpn_dtype) -> key width and codec.
@@ -172,6 +196,10 @@ struct SortRequest {
   uint64_t temp_bytes;
   hipStream_t stream;
   uint64_t row_stride = 0;  // elements between the starts of two rows, in input and outputs; 0: seg (dense rows)
+  // Rows sorted piece by piece (and merged afterwards): every row is `pieces` pieces of seg elements,
+  // the last one of last_seg; volume / seg still counts the rows.
+  uint32_t pieces   = 1;
+  uint32_t last_seg = 0;
 };
 
 // Workspace layout of the global path.  Everything in [0, zero_bytes) is cleared per call.
@@ -252,10 +280,12 @@ inline uint64_t workspace_bytes(int key_bytes, int passes, uint64_t volume, uint
   if (volume == 0 || seg <= lds_row_limit(key_bytes, want_indices)) {
     return HEADER_BYTES;
   }
-  if (merged_rows_apply(key_bytes, passes, volume, seg, want_indices)) {
-    // the rows with their halves sorted: keys, and the int64 positions of an argsort
-    return HEADER_BYTES + align_up(volume * key_bytes, WORKSPACE_ALIGN) +
-           (want_indices ? align_up(volume * 8, WORKSPACE_ALIGN) : 0);
+  if (const int levels = merged_row_levels(key_bytes, passes, volume, seg, want_indices); levels != 0) {
+    // the rows with their pieces sorted: keys, and the int64 positions of an argsort; twice that
+    // where the levels of merging go back and forth between two copies
+    const uint64_t copy =
+      align_up(volume * key_bytes, WORKSPACE_ALIGN) + (want_indices ? align_up(volume * 8, WORKSPACE_ALIGN) : 0);
+    return HEADER_BYTES + merged_row_split_bytes(volume, seg, levels) + (levels >= 2 ? 2 : 1) * copy;
   }
   const GlobalLayout L = global_layout(key_bytes, passes, volume, seg, want_values, want_indices, in_place);
   return L.valid ? L.total : 0;
@@ -280,42 +310,62 @@ inline int launch_zero_fill(void* p, uint64_t bytes, hipStream_t stream)
   return CPN_OK;
 }
 
-// ---- rows of up to twice the LDS capacity: two sorted halves, merged ---------------------------
+// ---- rows longer than the LDS capacity: sorted pieces, merged pairwise --------------------------
 template <typename KeyT, int CODEC, bool HAS_IDX>
 inline int sort_rows_in_lds(const SortRequest& r);
 
 template <typename KeyT, int CODEC, bool HAS_IDX>
-int sort_rows_merged(const SortRequest& r)
+int sort_rows_merged(const SortRequest& r, int levels)
 {
   const uint64_t n = r.seg, rows = r.volume / n;
-  const uint64_t h = (n + 1) / 2;  // first half; both halves fit the per-row kernel
-  uint8_t* ws      = static_cast<uint8_t*>(r.temp);
-  KeyT* tmp_keys   = reinterpret_cast<KeyT*>(ws + HEADER_BYTES);
-  int64_t* tmp_idx =
-    HAS_IDX ? reinterpret_cast<int64_t*>(ws + HEADER_BYTES + align_up(r.volume * sizeof(KeyT), WORKSPACE_ALIGN)) : nullptr;
-  for (int half = 0; half < 2; ++half) {
-    const uint64_t off = half == 0 ? 0 : h, len = half == 0 ? h : n - h;
-    SortRequest c      = r;
-    c.values_in        = static_cast<const KeyT*>(r.values_in) + off;
-    c.values_out       = tmp_keys + off;
-    c.indices_out      = HAS_IDX ? tmp_idx + off : nullptr;
-    c.seg              = len;
-    c.volume           = rows * len;
-    c.row_stride       = n;
-    c.index_offset     = r.index_offset + static_cast<int64_t>(off);  // positions count from the start of the whole row
-    const int rc       = sort_rows_in_lds<KeyT, CODEC, HAS_IDX>(c);
+  const uint64_t q        = merged_row_piece(n, levels);
+  const uint32_t pieces   = 1u << levels;  // (pieces - 1) * q < n: the last piece is never empty
+  const uint64_t key_copy = align_up(r.volume * sizeof(KeyT), WORKSPACE_ALIGN);
+  const uint64_t copy     = key_copy + (HAS_IDX ? align_up(r.volume * 8, WORKSPACE_ALIGN) : 0);
+  uint32_t* splits        = reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(r.temp) + HEADER_BYTES);
+  uint8_t* ws             = static_cast<uint8_t*>(r.temp) + HEADER_BYTES + merged_row_split_bytes(r.volume, n, levels);
+  // the copy that level `done` (0: the sorted pieces) leaves its rows in; the last level writes the outputs
+  auto keys_of = [&](int done) { return reinterpret_cast<KeyT*>(ws + ((levels - 1 - done) % 2) * copy); };
+  auto idx_of  = [&](int done) {
+    return HAS_IDX ? reinterpret_cast<int64_t*>(ws + ((levels - 1 - done) % 2) * copy + key_copy) : nullptr;
+  };
+  {
+    SortRequest c = r;
+    c.values_out  = keys_of(0);
+    c.indices_out = idx_of(0);
+    c.seg         = q;
+    c.volume      = rows * q;
+    c.row_stride  = n;
+    c.pieces      = pieces;
+    c.last_seg    = static_cast<uint32_t>(n - (pieces - 1) * q);
+    const int rc  = sort_rows_in_lds<KeyT, CODEC, HAS_IDX>(c);
     if (rc != CPN_OK) {
       return rc;
     }
   }
-  const uint64_t chunks = (n + merge_chunk(HAS_IDX) - 1) / merge_chunk(HAS_IDX);
-  {
-    ProfileScope prof("merge_halves", r.stream);
-    hipLaunchKernelGGL((merge_halves_kernel<KeyT, CODEC, HAS_IDX>), dim3(static_cast<uint32_t>(rows * chunks)),
-                       dim3(merge_block(HAS_IDX)), 0, r.stream, tmp_keys, tmp_idx, static_cast<KeyT*>(r.values_out), r.indices_out,
-                       static_cast<uint32_t>(n), static_cast<uint32_t>(h), static_cast<uint32_t>(chunks));
+  for (int level = 1; level <= levels; ++level) {
+    const uint64_t piece  = q << (level - 1);
+    const uint32_t pairs  = pieces >> level;
+    const uint64_t chunks = (2 * piece + merge_chunk(HAS_IDX) - 1) / merge_chunk(HAS_IDX);
+    const bool last       = level == levels;
+    const uint32_t grid   = static_cast<uint32_t>(rows * pairs * chunks);
+    {
+      ProfileScope prof("merge_split", r.stream);
+      hipLaunchKernelGGL((merge_split_kernel<KeyT, CODEC>), dim3((grid + MERGE_SPLIT_BLOCK - 1) / MERGE_SPLIT_BLOCK),
+                         dim3(MERGE_SPLIT_BLOCK), 0, r.stream, keys_of(level - 1), splits, static_cast<uint32_t>(n),
+                         static_cast<uint32_t>(piece), static_cast<uint32_t>(chunks), pairs,
+                         static_cast<uint32_t>(merge_chunk(HAS_IDX)), grid);
+    }
+    CPN_HIP_TRY(hipGetLastError());
+    {
+      ProfileScope prof("merge_halves", r.stream);
+      hipLaunchKernelGGL((merge_halves_kernel<KeyT, CODEC, HAS_IDX>), dim3(grid), dim3(merge_block(HAS_IDX)), 0, r.stream,
+                         keys_of(level - 1), idx_of(level - 1), last ? static_cast<KeyT*>(r.values_out) : keys_of(level),
+                         last ? r.indices_out : idx_of(level), splits, static_cast<uint32_t>(n), static_cast<uint32_t>(piece),
+                         static_cast<uint32_t>(chunks), pairs);
+    }
+    CPN_HIP_TRY(hipGetLastError());
   }
-  CPN_HIP_TRY(hipGetLastError());
   return CPN_OK;
 }
 
@@ -327,9 +377,10 @@ inline int launch_lds_rows(const SortRequest& r)
   {
     ProfileScope prof("lds_row_sort", r.stream);
     hipLaunchKernelGGL((lds_row_sort_kernel<KeyT, CODEC, HAS_IDX, BLOCK, ITEMS>),
-                       dim3(static_cast<uint32_t>(rows)), dim3(BLOCK), 0, r.stream,
+                       dim3(static_cast<uint32_t>(rows * r.pieces)), dim3(BLOCK), 0, r.stream,
                        static_cast<const KeyT*>(r.values_in), static_cast<KeyT*>(r.values_out), r.indices_out,
-                       static_cast<uint32_t>(r.seg), r.row_stride != 0 ? r.row_stride : r.seg, r.index_offset,
+                       static_cast<uint32_t>(r.seg), r.row_stride != 0 ? r.row_stride : r.seg, r.pieces,
+                       r.pieces > 1 ? r.last_seg : static_cast<uint32_t>(r.seg), r.index_offset,
                        static_cast<uint32_t*>(r.temp));
   }
   CPN_HIP_TRY(hipGetLastError());
@@ -420,7 +471,7 @@ inline int sort_rows_in_lds(const SortRequest& r)
   if (r.row_stride != 0 && (r.seg <= 4096 || sizeof(KeyT) < 4)) {
     return CPN_ERR_UNSUPPORTED;  // only the one-workgroup-per-row kernel of 4- and 8-byte keys takes strided rows
   }
-  if (r.volume / r.seg >= (1ull << 31)) {
+  if (r.volume / r.seg * r.pieces >= (1ull << 31)) {
     return CPN_ERR_UNSUPPORTED;
   }
   if (r.seg <= 32 && r.seg <= wave_row_limit()) {
@@ -777,8 +828,8 @@ int sort_typed(const SortRequest& r)
     return CPN_OK;
   }
   if constexpr ((KB == 4 || KB == 8) && KeyTraits<CODEC, KeyT>::NWORDS == 1) {
-    if (merged_rows_apply(KB, PASSES, r.volume, r.seg, has_idx)) {
-      return has_idx ? sort_rows_merged<KeyT, CODEC, true>(r) : sort_rows_merged<KeyT, CODEC, false>(r);
+    if (const int levels = merged_row_levels(KB, PASSES, r.volume, r.seg, has_idx); levels != 0) {
+      return has_idx ? sort_rows_merged<KeyT, CODEC, true>(r, levels) : sort_rows_merged<KeyT, CODEC, false>(r, levels);
     }
   }
   const GlobalLayout L = global_layout(KB, PASSES, r.volume, r.seg, r.values_out != nullptr, has_idx, in_place);

@@ -90,15 +90,18 @@ int64_t cpn_set_lds_row_limit(int64_t limit);
 int64_t cpn_set_wave_row_limit(int64_t limit);
 
 /*
- * Process-wide switch: rows longer than the per-row kernels take, up to twice that length (real keys
- * of 4 and 8 bytes), are sorted as two halves by the per-row kernel and merged (enabled != 0, the
- * default) or go down the global path like longer rows (0).  Returns the previous setting.  Also
- * initialised from the environment variable CPN_SORT_MERGE_ROWS (0 switches it off).  Changes the
- * sizes returned by cpn_local_sort_temp_bytes: do not change it between the size query and the sort.
+ * Process-wide switch: rows longer than the per-row kernels take (real keys of 4 and 8 bytes) are cut
+ * into 2, 4, ... pieces that the per-row kernel sorts and that are then merged pairwise, level by
+ * level, as long as that is cheaper than the global path's one pass per key byte (mode 1, the default:
+ * up to 6 levels for 8-byte keys, 5 with positions, i.e. rows of up to 1 048 576 and 458 752 keys;
+ * 2 levels for 4-byte keys, rows of up to 65 536), or all go down the global path (mode 0).  A mode N >= 2 allows up to N - 1 levels for every key (A/B runs); a
+ * negative mode restores the default.  Returns the previous mode.  Also initialised from the
+ * environment variable CPN_SORT_MERGE_ROWS.  Changes the sizes returned by
+ * cpn_local_sort_temp_bytes: do not change it between the size query and the sort.
  * An A/B switch with no counterpart in the reference, whose segmented radix sort takes every row
  * length (src/cupynumeric/sort/cub_sort.cuh:81-105).
  */
-int cpn_set_merge_rows(int enabled);
+int cpn_set_merge_rows(int mode);
 
 /*
  * Process-wide tunable: rows of at least `elements` elements on the global path keep their

@@ -104,10 +104,29 @@ def test_temp_bytes_layout(lib):
     assert tb(f64, 4 * 14336, 14336, 0, 1, 0) == header and tb(f64, 4 * 14337, 14337, 0, 1, 0) > header
     assert tb(f64, 4 * 14337, 14337, 1, 0, 0) == header
     assert tb(c128_, 4 * 4096, 4096, 1, 1, 0) == header and tb(c128_, 4 * 4097, 4097, 1, 0, 0) > header
-    # rows of up to twice those lengths (real keys of 4 and 8 bytes): the rows once more, and their positions
-    assert tb(f32, 4 * 20000, 20000, 1, 0, 0) == header + align256(4 * 20000 * 4)
-    assert tb(f64, 4 * 20000, 20000, 0, 1, 0) == header + align256(4 * 20000 * 8) + align256(4 * 20000 * 8)
-    assert tb(f32, 4 * 32769, 32769, 1, 0, 0) > header + align256(4 * 32769 * 4)  # global layout: histograms, descriptors
+    # longer rows of real keys of 4 and 8 bytes, merged from sorted pieces: a table of chunk starts (one word
+    # per 2048 outputs of a row and per piece), the rows once more and their positions; both twice from two
+    # levels of merging on; up to 2 levels for 4-byte keys, 6 for 8-byte keys (5 with positions)
+    def table(rows, seg, levels):
+        return align256(rows * ((seg + 2047) // 2048 + (1 << levels)) * 4)
+
+    assert tb(f32, 4 * 20000, 20000, 1, 0, 0) == header + table(4, 20000, 1) + align256(4 * 20000 * 4)
+    assert tb(f64, 4 * 20000, 20000, 0, 1, 0) == header + table(4, 20000, 1) + align256(4 * 20000 * 8) + align256(4 * 20000 * 8)
+    assert tb(f32, 4 * 32769, 32769, 1, 0, 0) == header + table(4, 32769, 2) + 2 * align256(4 * 32769 * 4)
+    assert tb(f32, 4 * 65536, 65536, 1, 1, 0) == header + table(4, 65536, 2) + 2 * (align256(4 * 65536 * 4) + align256(4 * 65536 * 8))
+    assert tb(f32, 4 * 65537, 65537, 1, 0, 0) == header + 4 * 4 * 256 * 4 + 4 * 20 * 256 * 4 + align256(4 * 65537 * 4)  # global layout: histograms, tile descriptors, one key buffer
+    assert tb(f64, 2 * (1 << 20), 1 << 20, 1, 0, 0) == header + table(2, 1 << 20, 6) + 2 * align256(2 * (1 << 20) * 8)
+    assert tb(f64, 2 * 458752, 458752, 0, 1, 0) == header + table(2, 458752, 5) + 4 * align256(2 * 458752 * 8)
+    prev = lib.cpn_set_merge_rows(0)
+    try:
+        assert lib.cpn_set_merge_rows(0) == 0
+        assert tb(f32, 4 * 20000, 20000, 1, 0, 0) != header + table(4, 20000, 1) + align256(4 * 20000 * 4)
+        lib.cpn_set_merge_rows(2)  # one level for every key
+        assert tb(f32, 4 * 20000, 20000, 1, 0, 0) == header + table(4, 20000, 1) + align256(4 * 20000 * 4)
+        assert tb(f32, 4 * 32769, 32769, 1, 0, 0) != header + table(4, 32769, 2) + 2 * align256(4 * 32769 * 4)
+    finally:
+        lib.cpn_set_merge_rows(prev)
+    assert lib.cpn_set_merge_rows(-1) == 1 and lib.cpn_set_merge_rows(1) == 1
     n = 1 << 24
     tiles = n // 16384  # 512 threads x 32 keys per tile for keys of up to 4 bytes
 

@@ -567,14 +567,16 @@ def test_global_path_skipping_needs_every_row(lib, torch_cuda, global_path):
 # ---- rows of up to twice the LDS capacity: two sorted halves, merged -----------------------------------
 @pytest.mark.parametrize("dtype", [np.float32, np.int32, np.uint32, np.float64, np.int64, np.uint64])
 def test_rows_sorted_as_merged_halves(lib, torch_cuda, dtype):
-    """Row lengths on both sides of the range that is sorted as two halves and merged (16 385 ... 32 768;
-    14 337 ... 28 672 for 8-byte keys with positions), odd and even lengths, rows with many ties across
-    the two halves (stability of the merge), sorted, reversed and constant rows, special float values,
+    """Row lengths on both sides of the ranges that are sorted in 2, 4 and 8 pieces and merged (up to
+    16 384 keys a piece; 14 336 for 8-byte keys with positions), odd and even lengths, rows with many ties
+    across the pieces (stability of the merge), sorted, reversed and constant rows, special float values,
     values and positions together, in place, an index offset; and the same requests with the path
     switched off give the same bits through the global path."""
     dt = np.dtype(dtype)
     rng = np.random.default_rng(dt.num * 7 + 1)
-    lengths = [16385, 16386, 20001, 28672, 28673, 32767, 32768, 32769] + ([14337, 14338] if dt.itemsize == 8 else [])
+    lengths = [16385, 16386, 20001, 28672, 28673, 32767, 32768, 32769, 40003, 57344, 57345, 65535, 65536, 65537]
+    if dt.itemsize == 8:
+        lengths += [14337, 14338, 114688, 114689, 131072, 131073]
     header = lib.cpn_local_sort_temp_bytes(_lib.DTYPE_CODES[dt], 0, 0, 1, 0, 0)
     for seg in lengths:
         rows = 5
@@ -596,10 +598,15 @@ def test_rows_sorted_as_merged_halves(lib, torch_cuda, dtype):
         assert_same_bits(i, want_i + 1000, f"{dt} seg={seg} values+positions, offset")
         v, _ = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=False, in_place=True)
         assert_same_bits(v, want_v, f"{dt} seg={seg} in place")
-    # the path is the one that runs: its workspace is the rows once (plus positions), not the global layout
+    # the path is the one that runs: its workspace is the table of chunk starts and the rows once (plus
+    # positions; twice from two levels of merging on), not the global layout
     code, seg, rows = _lib.DTYPE_CODES[dt], 20000, 4
     merged_bytes = lib.cpn_local_sort_temp_bytes(code, rows * seg, seg, 1, 0, 0)
-    assert merged_bytes == header + (rows * seg * dt.itemsize + 255) // 256 * 256
+    table = (rows * ((seg + 2047) // 2048 + 2) * 4 + 255) // 256 * 256
+    assert merged_bytes == header + table + (rows * seg * dt.itemsize + 255) // 256 * 256
+    table = (rows * ((40000 + 2047) // 2048 + 4) * 4 + 255) // 256 * 256
+    assert lib.cpn_local_sort_temp_bytes(code, rows * 40000, 40000, 1, 1, 0) == \
+        header + table + 2 * ((rows * 40000 * dt.itemsize + 255) // 256 * 256 + (rows * 40000 * 8 + 255) // 256 * 256)
     prev = lib.cpn_set_merge_rows(0)
     try:
         assert lib.cpn_local_sort_temp_bytes(code, rows * seg, seg, 1, 0, 0) != merged_bytes
