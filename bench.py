@@ -654,7 +654,7 @@ def run_consumer(args) -> dict:
 
 
 # -------------------------------------------------------------------------------------------------
-ROW_KERNELS = ("tiny_row_sort", "wave_row_sort", "lds_row_sort", "count16_row_sort")
+ROW_KERNELS = ("bitonic_row_sort", "tiny_row_sort", "wave_row_sort", "lds_row_sort", "count16_row_sort")
 
 
 def verify_result(job: GpuJob, cfg: dict) -> str:

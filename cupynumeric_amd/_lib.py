@@ -59,6 +59,7 @@ PROTOTYPES: dict[str, tuple] = {
     "cpn_set_virtual_digit_threshold": (c_int64, [c_int64]),
     "cpn_set_wave_row_limit": (c_int64, [c_int64]),
     "cpn_set_merge_rows": (c_int, [c_int]),
+    "cpn_set_bitonic_rows": (c_int, [c_int]),
     "cpn_set_tile_order": (c_int, [c_int]),
     "cpn_dtype_size": (c_uint64, [c_int]),
     "cpn_key_order_bits": (c_uint64, [c_int, c_uint64]),

@@ -78,6 +78,14 @@ int merge_levels_limit(int key_bytes, bool want_indices)
   return key_bytes == 8 ? (want_indices ? 5 : 6) : 2;
 }
 
+// 1: rows of 2 ... 64 real keys go through the bitonic network; 0: through the ranking kernels
+static std::atomic<int> g_bitonic_rows{[] {
+  const char* e = getenv("CPN_SORT_BITONIC_ROWS");
+  return (e != nullptr && e[0] == '0') ? 0 : 1;
+}()};
+
+bool bitonic_rows_enabled() { return g_bitonic_rows.load(std::memory_order_relaxed) != 0; }
+
 static std::atomic<long long> g_spin_limit{static_cast<long long>(LOOKBACK_SPIN_LIMIT)};
 
 uint32_t lookback_spin_limit() { return static_cast<uint32_t>(g_spin_limit.load(std::memory_order_relaxed)); }
@@ -194,6 +202,8 @@ int64_t cpn_set_lookback_spin_limit(int64_t polls)
 }
 
 int cpn_set_tile_order(int single) { return cpn::g_tile_order.exchange(single != 0 ? 1 : 0); }
+
+int cpn_set_bitonic_rows(int enabled) { return cpn::g_bitonic_rows.exchange(enabled != 0 ? 1 : 0); }
 
 int cpn_set_merge_rows(int mode) { return cpn::g_merge_rows.exchange(mode < 0 ? 1 : mode); }
 

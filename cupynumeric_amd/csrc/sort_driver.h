@@ -14,6 +14,7 @@
 #include "onesweep.h"
 #include "profile.h"
 #include "tiny_row_sort.h"
+#include "bitonic_row_sort.h"
 #include "merge_rows.h"
 #include "wave_row_sort.h"
 
@@ -101,6 +102,10 @@ __host__ __device__ constexpr int key_passes(int key_bytes, int codec)
 {
   return codec == CODEC_COMPLEX ? key_bytes + 1 : key_bytes;
 }
+
+// Rows of 2 ... 64 real keys go through the bitonic network (bitonic_row_sort.h)
+// unless CPN_SORT_BITONIC_ROWS=0 in the environment sends them to the ranking kernels (A/B runs).
+bool bitonic_rows_enabled();
 
 // Row length up to which one wavefront (instead of one workgroup) sorts a row; at most 1024.
 // Changed by cpn_set_wave_row_limit / CPN_SORT_WAVE_ROW_LIMIT for A/B runs.
@@ -448,6 +453,22 @@ inline int launch_wave_rows(const SortRequest& r)
 }
 
 template <typename KeyT, int CODEC, bool HAS_IDX, int S>
+inline int launch_bitonic_rows(const SortRequest& r)
+{
+  const uint64_t rows           = r.volume / r.seg;
+  const uint64_t rows_per_block = (256 / WAVE) * (WAVE / S);
+  const uint64_t blocks         = (rows + rows_per_block - 1) / rows_per_block;
+  {
+    ProfileScope prof("bitonic_row_sort", r.stream);
+    hipLaunchKernelGGL((bitonic_row_sort_kernel<KeyT, CODEC, HAS_IDX, S>), dim3(static_cast<uint32_t>(blocks)), dim3(256),
+                       0, r.stream, static_cast<const KeyT*>(r.values_in), static_cast<KeyT*>(r.values_out),
+                       r.indices_out, static_cast<uint32_t>(r.seg), rows, r.index_offset, static_cast<uint32_t*>(r.temp));
+  }
+  CPN_HIP_TRY(hipGetLastError());
+  return CPN_OK;
+}
+
+template <typename KeyT, int CODEC, bool HAS_IDX, int S>
 inline int launch_tiny_rows(const SortRequest& r)
 {
   const uint64_t rows          = r.volume / r.seg;
@@ -473,6 +494,24 @@ inline int sort_rows_in_lds(const SortRequest& r)
   }
   if (r.volume / r.seg * r.pieces >= (1ull << 31)) {
     return CPN_ERR_UNSUPPORTED;
+  }
+  if constexpr (sizeof(KeyT) <= 8 && (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT)) {
+    // real keys, rows of 2 ... 64: a bitonic network between the lanes of a wavefront
+    if (r.seg >= 2 && r.seg <= 64 && r.seg <= wave_row_limit() && bitonic_rows_enabled()) {
+      if (r.seg <= 2) {
+        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 2>(r);
+      } else if (r.seg <= 4) {
+        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 4>(r);
+      } else if (r.seg <= 8) {
+        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 8>(r);
+      } else if (r.seg <= 16) {
+        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 16>(r);
+      } else if (r.seg <= 32) {
+        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 32>(r);
+      } else {
+        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 64>(r);
+      }
+    }
   }
   if (r.seg <= 32 && r.seg <= wave_row_limit()) {
     if (r.seg <= 1) {

@@ -90,6 +90,16 @@ int64_t cpn_set_lds_row_limit(int64_t limit);
 int64_t cpn_set_wave_row_limit(int64_t limit);
 
 /*
+ * Process-wide switch: rows of 2 ... 64 real keys of up to 8 bytes are sorted by a bitonic network
+ * between the lanes of a wavefront (enabled != 0, the default) or by the ranking kernels that take
+ * the other key types of that length (0).  Returns the previous setting.  Also initialised from the
+ * environment variable CPN_SORT_BITONIC_ROWS (0 switches it off).  Does not affect workspace sizes.
+ * An A/B switch with no counterpart in the reference, which merge-sorts (segment id, value) tuples
+ * for short rows (src/cupynumeric/sort/thrust_sort.cuh:68-122).
+ */
+int cpn_set_bitonic_rows(int enabled);
+
+/*
  * Process-wide switch: rows longer than the per-row kernels take (real keys of 4 and 8 bytes) are cut
  * into 2, 4, ... pieces that the per-row kernel sorts and that are then merged pairwise, level by
  * level, as long as that is cheaper than the global path's one pass per key byte (mode 1, the default:

@@ -273,6 +273,58 @@ def test_wave_rows_split_into_ranges(lib, torch_cuda, dtype):
     assert_same_bits(got_i, np.argsort(big, axis=-1, kind="stable"), f"{dt} many rows of 128, argsort")
 
 
+REAL_DTYPES = [np.bool_, np.int8, np.uint8, np.int16, np.uint16, np.float16, np.int32, np.uint32, np.float32,
+               np.int64, np.uint64, np.float64]
+
+
+@pytest.mark.parametrize("dtype", REAL_DTYPES)
+def test_rows_of_up_to_64_keys_through_the_bitonic_network(lib, torch_cuda, dtype):
+    """Rows of 2 ... 64 real keys: every length (every number of slots per row, full and partly filled),
+    row counts that leave the last wavefront partly empty, rows of equal keys, of two keys, sorted and
+    reversed rows, NaNs of several payloads and zeros of both signs (ties go by position: the stable
+    order), the extreme values of the type (the image that padding slots hold), values and positions
+    together, in place, an index offset; and the ranking kernels give the same bits with the network
+    switched off."""
+    dt = np.dtype(dtype)
+    rng = np.random.default_rng(dt.num * 13 + 5)
+    for seg in list(range(2, 66)):
+        rows = 1 + (seg * 7) % 23 if seg % 3 else 200 + seg
+        x = make_input(dtype, (rows, seg), seed=seg)
+        x[0] = x[0, 0]
+        if rows > 4:
+            x[1] = np.sort(x[1])
+            x[2] = np.sort(x[2])[::-1]
+            x[3] = np.where(rng.random(seg) < 0.5, x[3, 0], x[3, -1])
+        if rows > 6:
+            if dt.kind == "f":
+                x[4, ::3] = np.nan
+                x[4, 1::3] = -0.0
+                x[4, 2::3] = 0.0
+                x[5] = np.where(rng.random(seg) < 0.3, np.inf, x[5])
+                x[5, ::4] = -np.inf
+                x[6, ::2] = np.finfo(dtype).max
+                nan_bits = x[4].view(f"u{dt.itemsize}")
+                nan_bits[::6] |= 1  # another NaN payload
+            elif dt.kind in "iu":
+                x[4, ::2] = np.iinfo(dtype).max
+                x[5, ::2] = np.iinfo(dtype).min
+                x[6] = rng.integers(0, 3, seg).astype(dtype)
+        want_v, want_i = check_rows(lib, torch_cuda, x, f"{dt} seg={seg}")
+        if seg in (2, 3, 17, 32, 33, 64):
+            v, i = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=True, offset=-5)
+            assert_same_bits(v, want_v, f"{dt} seg={seg} values+positions")
+            assert_same_bits(i, want_i - 5, f"{dt} seg={seg} values+positions, offset")
+            v, _ = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=False, in_place=True)
+            assert_same_bits(v, want_v, f"{dt} seg={seg} in place")
+    prev = lib.cpn_set_bitonic_rows(0)
+    try:
+        for seg in (2, 20, 32, 33, 64):
+            check_rows(lib, torch_cuda, make_input(dtype, (77, seg), seed=seg), f"{dt} seg={seg}, ranking kernels")
+    finally:
+        assert lib.cpn_set_bitonic_rows(prev) == 0
+    assert lib.cpn_set_bitonic_rows(1) == 1
+
+
 def test_lds_many_short_rows(lib, torch_cuda):
     for dtype, shape in [(np.float64, (3000, 37)), (np.int8, (5000, 5)), (np.float16, (700, 401)), (np.uint32, (129, 1024))]:
         check_rows(lib, torch_cuda, make_input(dtype, shape, seed=11), f"{np.dtype(dtype)} {shape}")
