@@ -103,7 +103,7 @@ __host__ __device__ constexpr int key_passes(int key_bytes, int codec)
   return codec == CODEC_COMPLEX ? key_bytes + 1 : key_bytes;
 }
 
-// Rows of 2 ... 64 real keys go through the bitonic network (bitonic_row_sort.h)
+// Rows of 2 ... 128 real keys go through the bitonic network (bitonic_row_sort.h)
 // unless CPN_SORT_BITONIC_ROWS=0 in the environment sends them to the ranking kernels (A/B runs).
 bool bitonic_rows_enabled();
 
@@ -456,7 +456,7 @@ template <typename KeyT, int CODEC, bool HAS_IDX, int S>
 inline int launch_bitonic_rows(const SortRequest& r)
 {
   const uint64_t rows           = r.volume / r.seg;
-  const uint64_t rows_per_block = (256 / WAVE) * (WAVE / S);
+  const uint64_t rows_per_block = (256 / WAVE) * (S >= WAVE ? 1 : WAVE / S);
   const uint64_t blocks         = (rows + rows_per_block - 1) / rows_per_block;
   {
     ProfileScope prof("bitonic_row_sort", r.stream);
@@ -496,8 +496,8 @@ inline int sort_rows_in_lds(const SortRequest& r)
     return CPN_ERR_UNSUPPORTED;
   }
   if constexpr (sizeof(KeyT) <= 8 && (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT)) {
-    // real keys, rows of 2 ... 64: a bitonic network between the lanes of a wavefront
-    if (r.seg >= 2 && r.seg <= 64 && r.seg <= wave_row_limit() && bitonic_rows_enabled()) {
+    // real keys, rows of 2 ... 128: a bitonic network between the lanes of a wavefront
+    if (r.seg >= 2 && r.seg <= 128 && r.seg <= wave_row_limit() && bitonic_rows_enabled()) {
       if (r.seg <= 2) {
         return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 2>(r);
       } else if (r.seg <= 4) {
@@ -508,8 +508,10 @@ inline int sort_rows_in_lds(const SortRequest& r)
         return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 16>(r);
       } else if (r.seg <= 32) {
         return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 32>(r);
-      } else {
+      } else if (r.seg <= 64) {
         return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 64>(r);
+      } else {
+        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 128>(r);
       }
     }
   }

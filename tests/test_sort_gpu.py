@@ -278,8 +278,9 @@ REAL_DTYPES = [np.bool_, np.int8, np.uint8, np.int16, np.uint16, np.float16, np.
 
 
 @pytest.mark.parametrize("dtype", REAL_DTYPES)
-def test_rows_of_up_to_64_keys_through_the_bitonic_network(lib, torch_cuda, dtype):
-    """Rows of 2 ... 64 real keys: every length (every number of slots per row, full and partly filled),
+def test_rows_of_up_to_128_keys_through_the_bitonic_network(lib, torch_cuda, dtype):
+    """Rows of 2 ... 128 real keys: every length (every number of slots per row, full and partly filled,
+    one and two elements per lane),
     row counts that leave the last wavefront partly empty, rows of equal keys, of two keys, sorted and
     reversed rows, NaNs of several payloads and zeros of both signs (ties go by position: the stable
     order), the extreme values of the type (the image that padding slots hold), values and positions
@@ -287,7 +288,7 @@ def test_rows_of_up_to_64_keys_through_the_bitonic_network(lib, torch_cuda, dtyp
     switched off."""
     dt = np.dtype(dtype)
     rng = np.random.default_rng(dt.num * 13 + 5)
-    for seg in list(range(2, 66)):
+    for seg in list(range(2, 70)) + [95, 96, 97, 100, 126, 127, 128, 129]:
         rows = 1 + (seg * 7) % 23 if seg % 3 else 200 + seg
         x = make_input(dtype, (rows, seg), seed=seg)
         x[0] = x[0, 0]
@@ -310,7 +311,7 @@ def test_rows_of_up_to_64_keys_through_the_bitonic_network(lib, torch_cuda, dtyp
                 x[5, ::2] = np.iinfo(dtype).min
                 x[6] = rng.integers(0, 3, seg).astype(dtype)
         want_v, want_i = check_rows(lib, torch_cuda, x, f"{dt} seg={seg}")
-        if seg in (2, 3, 17, 32, 33, 64):
+        if seg in (2, 3, 17, 32, 33, 64, 65, 100, 128):
             v, i = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=True, offset=-5)
             assert_same_bits(v, want_v, f"{dt} seg={seg} values+positions")
             assert_same_bits(i, want_i - 5, f"{dt} seg={seg} values+positions, offset")
@@ -318,7 +319,7 @@ def test_rows_of_up_to_64_keys_through_the_bitonic_network(lib, torch_cuda, dtyp
             assert_same_bits(v, want_v, f"{dt} seg={seg} in place")
     prev = lib.cpn_set_bitonic_rows(0)
     try:
-        for seg in (2, 20, 32, 33, 64):
+        for seg in (2, 20, 32, 33, 64, 65, 128):
             check_rows(lib, torch_cuda, make_input(dtype, (77, seg), seed=seg), f"{dt} seg={seg}, ranking kernels")
     finally:
         assert lib.cpn_set_bitonic_rows(prev) == 0
