@@ -136,8 +136,8 @@ inline int merged_row_levels(int key_bytes, int passes, uint64_t volume, uint64_
     return 0;
   }
   const uint64_t cap = lds_row_capacity(key_bytes, want_indices);
-  if (lds_row_limit(key_bytes, want_indices) != cap || seg <= cap) {
-    return 0;
+  if (lds_row_limit(key_bytes, want_indices) != cap || seg <= cap || seg >= (1ull << 31)) {
+    return 0;  // (the merge kernels count inside a row in 32 bits)
   }
   const int limit = merge_levels_limit(key_bytes, want_indices);
   int levels      = 1;
