@@ -707,8 +707,11 @@ inline int sort_global(const SortRequest& r, const GlobalLayout& L)
       ProfileScope prof("histogram_scan", r.stream);
       const uint64_t n_hist = L.rows * PASSES;
       uint64_t sgrid        = (n_hist + SCAN_BLOCK / WAVE - 1) / (SCAN_BLOCK / WAVE);
-      if (sgrid > 1024) {
-        sgrid = 1024;
+      // Every workgroup ends with one atomic on the same word (the last one makes the plan), and those
+      // queue: 4092 histograms on 1023 workgroups took 0.087 ms, on 64 workgroups 0.021 ms.
+      const uint64_t sgrid_cap = n_hist / 64 < 64 ? 64 : (n_hist / 64 > 1024 ? 1024 : n_hist / 64);
+      if (sgrid > sgrid_cap) {
+        sgrid = sgrid_cap;
       }
       hipLaunchKernelGGL((histogram_scan_kernel<OffT>), dim3(static_cast<uint32_t>(sgrid)), dim3(SCAN_BLOCK), 0,
                          r.stream, hist, varying, r.seg, static_cast<uint32_t>(PASSES), n_hist,
