@@ -530,8 +530,11 @@ inline int sort_rows_in_lds(const SortRequest& r)
       return launch_tiny_rows<KeyT, CODEC, HAS_IDX, 32>(r);
     }
   }
-  // (keys of 8 bytes and more hold too many registers per lane at 16 items: 512 there)
-  if (r.seg <= wave_row_limit() && (sizeof(KeyT) < 8 || r.seg <= 512)) {
+  // (keys of 8 bytes and more hold too many registers per lane at 16 items: 512 there; and for 4-byte
+  // keys the workgroup kernel with its split into value ranges is the faster one from 513 on: 2^26
+  // float32 keys in rows of 513 0.63 -> 0.38 ms, of 1024 0.34 -> 0.23, argsort of rows of 1024 0.44 -> 0.31;
+  // rows of 1024 float16 keys 0.17 against 0.20 ms, of single bytes 0.067 against 0.081)
+  if (r.seg <= wave_row_limit() && (sizeof(KeyT) < 4 || r.seg <= 512)) {
     if (r.seg <= 64) {
       return launch_wave_rows<KeyT, CODEC, HAS_IDX, 1>(r);
     } else if (r.seg <= 128) {
