@@ -70,7 +70,10 @@ __host__ __device__ constexpr int bucket_bins_log2(int tile, int key_bytes, bool
     // 4096 float32 0.275 / 0.281 / 0.327, 2048 float32 0.259 / 0.266 / 0.302.
     // (The shapes of 12 keys per thread, tiles of 1536 and 3072 keys, keep the table of the next smaller
     // power of two: 1.33 bins per key; with 2.67 rows of 3072 float32 keys took 0.37 ms instead of 0.25.)
-    return (tile <= 1024 ? 10 : (tile <= 2048 ? 11 : 12)) + ((key_bytes == 4 && !has_idx && tile % 3 != 0) ? 1 : 0);
+    // (The one-wave shape of 768 keys: 512 bins for plain sorts, 2^26 float32 keys in rows of 513 0.25 ms
+    // against 0.28 with 1024 bins; 1024 with positions, 0.305 against 0.32 ms for rows of 768.)
+    return (tile <= 1024 ? 10 : (tile <= 2048 ? 11 : 12)) + ((key_bytes == 4 && !has_idx && tile % 3 != 0) ? 1 : 0) -
+           ((tile <= 768 && !has_idx) ? 1 : 0);
   }
   if (row_bytes + 32 * KIB <= 78 * KIB) {
     return 13;  // two workgroups per CU either way
@@ -150,7 +153,7 @@ void lds_row_sort_kernel(const KeyT* keys_in,
   // (every shape of at least 128 threads: measured on 2^26 keys, passes / split: rows of 1024 float64 0.35 / 0.30 ms,
   // 2048 float64 0.47 / 0.34, 4096 float64 0.50 / 0.37, 1500 float32 0.48 / 0.30, 2048 float32 0.36 / 0.25,
   // 4096 int32 0.35 / 0.30; with positions 2048 float32 0.43 / 0.32, 2048 float64 0.55 / 0.40 ms)
-  constexpr bool BUCKETS_SHAPE = BLOCK >= 128 && ITEMS >= 8;
+  constexpr bool BUCKETS_SHAPE = BLOCK >= 64 && ITEMS >= 8;  // (64 x 12: one wavefront per row of 513 ... 768 keys)
   constexpr bool BUCKETS_OK = NW == 1 && sizeof(KeyT) >= 4 && sizeof(KeyT) <= 8 && BUCKETS_SHAPE &&
                               (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT);
   constexpr int BINS_LOG2   = bucket_bins_log2(TILE, sizeof(KeyT), HAS_IDX, BLOCK);
