@@ -62,6 +62,9 @@ __host__ __device__ constexpr int bucket_bins_log2(int tile, int key_bytes, bool
 {
   const int row_bytes = tile * key_bytes + (has_idx ? tile * 2 : 0);
   constexpr int KIB = 1024;
+  if (tile <= 256) {
+    return 8;  // one bin per key
+  }
   if (tile <= 4096) {
     // One bin per key; two for plain sorts of 4-byte keys.  More bins shorten the walks and cost LDS,
     // i.e. workgroups per CU, which weighs more.  Measured on 2^26 keys, two / one / half a bin per key:
@@ -153,7 +156,7 @@ void lds_row_sort_kernel(const KeyT* keys_in,
   // (every shape of at least eight keys per thread: measured on 2^26 keys, passes / split: rows of 1024 float64 0.35 / 0.30 ms,
   // 2048 float64 0.47 / 0.34, 4096 float64 0.50 / 0.37, 1500 float32 0.48 / 0.30, 2048 float32 0.36 / 0.25,
   // 4096 int32 0.35 / 0.30; with positions 2048 float32 0.43 / 0.32, 2048 float64 0.55 / 0.40 ms)
-  constexpr bool BUCKETS_SHAPE = BLOCK >= 64 && ITEMS >= 8;  // (64 x 12: one wavefront per row of 513 ... 768 keys)
+  constexpr bool BUCKETS_SHAPE = BLOCK >= 64 && ITEMS >= 4;  // (64 x 4 ... 64 x 12: one wavefront per row of up to 768 keys)
   constexpr bool BUCKETS_OK = NW == 1 && sizeof(KeyT) >= 4 && sizeof(KeyT) <= 8 && BUCKETS_SHAPE &&
                               (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT);
   constexpr int BINS_LOG2   = bucket_bins_log2(TILE, sizeof(KeyT), HAS_IDX, BLOCK);

@@ -530,16 +530,22 @@ inline int sort_rows_in_lds(const SortRequest& r)
       return launch_tiny_rows<KeyT, CODEC, HAS_IDX, 32>(r);
     }
   }
-  // (keys of 8 bytes and more hold too many registers per lane at 16 items: 512 there; and for 4-byte
-  // keys the workgroup kernel with its split into value ranges is the faster one from 513 on: 2^26
-  // float32 keys in rows of 513 0.63 -> 0.38 ms, of 1024 0.34 -> 0.23, argsort of rows of 1024 0.44 -> 0.31;
-  // rows of 1024 float16 keys 0.17 against 0.20 ms, of single bytes 0.067 against 0.081)
   if ((sizeof(KeyT) == 4 || sizeof(KeyT) == 8) && r.seg > 256 && r.seg <= 512 && CODEC != CODEC_COMPLEX) {
     // real keys of 4 and 8 bytes: the workgroup kernel in a one-wave shape, eight keys per lane, split into
     // value ranges, ahead of the one-wave ranking kernel: 2^26 float64 keys in rows of 512 0.32 -> 0.23 ms,
     // of 257 0.57 -> 0.40; float32 rows of 512 0.24 -> 0.21, argsort 0.31 -> 0.29
     return launch_lds_rows<KeyT, CODEC, HAS_IDX, 64, 8>(r);
   }
+  if ((sizeof(KeyT) == 4 || sizeof(KeyT) == 8) && r.seg > 128 && r.seg <= 256 && CODEC != CODEC_COMPLEX) {
+    // (the same with four keys per lane: float32 rows of 256 0.27 -> 0.22 ms, float64 rows of 256 0.35 -> 0.29,
+    // of 129 0.69 -> 0.52, with positions 0.72 -> 0.45)
+    return launch_lds_rows<KeyT, CODEC, HAS_IDX, 64, 4>(r);
+  }
+  // The one-wave ranking kernel: keys of 1 and 2 bytes up to 1024, the others up to 512 (keys of 8 bytes
+  // and more hold too many registers per lane at 16 items, and for 4-byte keys the workgroup kernel with
+  // its split into value ranges is the faster one: 2^26 float32 keys in rows of 513 0.63 -> 0.38 ms, of
+  // 1024 0.34 -> 0.23, argsort of rows of 1024 0.44 -> 0.31; rows of 1024 float16 keys 0.17 against
+  // 0.20 ms, of single bytes 0.067 against 0.081).  Real keys of 4 and 8 bytes have left above.
   if (r.seg <= wave_row_limit() && (sizeof(KeyT) < 4 || r.seg <= 512)) {
     if (r.seg <= 64) {
       return launch_wave_rows<KeyT, CODEC, HAS_IDX, 1>(r);

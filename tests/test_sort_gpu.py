@@ -153,7 +153,7 @@ def test_random_module_and_flatten():
 
 
 # ---- per-row LDS path: every dtype, lengths around every workgroup-shape boundary -------------------
-LDS_LENGTHS = [1, 2, 3, 63, 64, 65, 255, 256, 257, 300, 511, 512, 513, 600, 767, 768, 769, 1000, 1023, 1024, 1025, 1535, 1536, 1537, 3071, 3072, 3073, 4095, 4096, 4097, 6143, 6144, 6145, 8191,
+LDS_LENGTHS = [1, 2, 3, 63, 64, 65, 129, 130, 200, 255, 256, 257, 300, 511, 512, 513, 600, 767, 768, 769, 1000, 1023, 1024, 1025, 1535, 1536, 1537, 3071, 3072, 3073, 4095, 4096, 4097, 6143, 6144, 6145, 8191,
                8192, 8193, 12000, 12287, 12288, 12289, 14335, 14336, 14337, 16383, 16384, 16385]
 
 
@@ -173,7 +173,7 @@ def test_lds_rows_split_on_leading_bits(lib, torch_cuda, dtype):
     the limit (the radix passes take over), all lengths of the row kernels that have the path."""
     rng = np.random.default_rng(np.dtype(dtype).itemsize * 31 + np.dtype(dtype).num)
     dt = np.dtype(dtype)
-    for seg in (257, 300, 512, 513, 700, 768, 769, 1024, 1025, 1500, 1536, 1537, 2048, 2049, 3000, 3072, 3073, 4095, 4096, 4097, 6000, 6144, 6145, 8192, 8193, 12000, 12288,
+    for seg in (129, 200, 256, 257, 300, 512, 513, 700, 768, 769, 1024, 1025, 1500, 1536, 1537, 2048, 2049, 3000, 3072, 3073, 4095, 4096, 4097, 6000, 6144, 6145, 8192, 8193, 12000, 12288,
                 12289, 16384):
         rows = 7
         if dt.kind == "f":
@@ -206,7 +206,7 @@ def test_lds_rows_split_on_leading_bits(lib, torch_cuda, dtype):
         assert_same_bits(got, want, f"{dt} seg={seg} values with positions")
         assert_same_bits(got_i, want_i + 7, f"{dt} seg={seg} positions with values")
     # groups of equal keys of every size around the limit of a bin (24; 48 where a bin holds four keys on average)
-    for seg, groups in ((512, (23, 24, 25)), (768, (23, 24, 25)), (1536, (23, 24, 25)), (3072, (23, 24, 25)), (6144, (23, 24, 25)), (8192, (2, 23, 24, 25, 40, 47, 48, 49)), (12288, (24, 25, 48, 49)),
+    for seg, groups in ((256, (23, 24, 25)), (512, (23, 24, 25)), (768, (23, 24, 25)), (1536, (23, 24, 25)), (3072, (23, 24, 25)), (6144, (23, 24, 25)), (8192, (2, 23, 24, 25, 40, 47, 48, 49)), (12288, (24, 25, 48, 49)),
                         (16384, (24, 47, 48, 49, 100))):
         for group in groups:
             base = rng.permutation(seg // group + 1).astype(dtype)
