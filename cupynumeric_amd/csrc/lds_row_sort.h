@@ -31,9 +31,8 @@
 // second atomic puts every key into its bin and tells the key where it went; every key then finds
 // its place inside its bin by counting the keys of the bin that come before it.  A row that
 // crowds more than BUCKET_LIMIT keys into one bin (few different keys, tight clusters) goes
-// through the radix passes instead.  Used by every shape of at least eight keys per thread, for real
-// keys of 4 or 8 bytes (rows of up to 512 such keys are sorted by one wave each, wave_row_sort.h, which
-// has the same path for 4-byte keys); the number of bins is bucket_bins_log2.  Sorts that carry positions take
+// through the radix passes instead.  Used by every shape of at least four keys per thread, for real
+// keys of 4 or 8 bytes (the one-wave ranking kernel, wave_row_sort.h, has the same path for 4-byte keys); the number of bins is bucket_bins_log2.  Sorts that carry positions take
 // it as well: the position a key came from is staged beside the key and breaks the ties inside a
 // bin, which makes the result the stable order.
 //
@@ -153,7 +152,7 @@ void lds_row_sort_kernel(const KeyT* keys_in,
   // the split on leading bits: real keys of 4 and 8 bytes, values only
   // (only the 1024-thread shapes, rows of more than 4096 keys: in the smaller shapes the bins cost
   // the LDS that lets many workgroups share a CU, and rows of 1024 float64 keys went from 0.41 to 0.60 ms)
-  // (every shape of at least eight keys per thread: measured on 2^26 keys, passes / split: rows of 1024 float64 0.35 / 0.30 ms,
+  // (every shape of at least four keys per thread: measured on 2^26 keys, passes / split: rows of 1024 float64 0.35 / 0.30 ms,
   // 2048 float64 0.47 / 0.34, 4096 float64 0.50 / 0.37, 1500 float32 0.48 / 0.30, 2048 float32 0.36 / 0.25,
   // 4096 int32 0.35 / 0.30; with positions 2048 float32 0.43 / 0.32, 2048 float64 0.55 / 0.40 ms)
   constexpr bool BUCKETS_SHAPE = BLOCK >= 64 && ITEMS >= 4;  // (64 x 4 ... 64 x 12: one wavefront per row of up to 768 keys)
