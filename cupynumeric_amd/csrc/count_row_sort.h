@@ -25,8 +25,12 @@ constexpr int COUNT16_WORDS = 32768;  // 65 536 bins, two 16-bit counters per wo
 // Shortest row given to this kernel: below it the fixed cost of clearing and scanning 65 536 bins
 // outweighs the cheaper ranking (CPN_SORT_COUNT16_MIN_ROW in the environment overrides it).
 // Measured on float16 rows, 2^26 keys in all, radix row kernel / this kernel: rows of 3000 0.25 / 0.36 ms,
-// 4096 0.23 / 0.30, 4097 0.47 / 0.40, 5000 0.25 / 0.18, 8192 0.33 / 0.21, 16 384 0.41 / 0.18 ms.
-constexpr uint32_t COUNT16_MIN_ROW = 4097;
+// 4096 0.23 / 0.30; against the radix kernel's 512-thread shapes of 12 and 16 keys per thread (two workgroups
+// per CU): 4097 0.27 / 0.39, 5000 0.22 / 0.28, 6144 0.185 / 0.23, 6145 0.24 / 0.32, 8192 0.18 / 0.20; and
+// against its 1024-thread shapes above: 8193 0.42 / 0.38, 12 288 0.35 / 0.21, 16 384 0.33 / 0.19 ms.
+// So the counting starts where the 512-thread shapes end (count16_long_rows_kernel); the kernel for rows of
+// up to 8192 keys, count16_rows_kernel, runs only when the environment lowers this value.
+constexpr uint32_t COUNT16_MIN_ROW = 8193;
 
 // Word of the histogram that holds bin `bin`.  Words are kept in 16-byte chunks and the chunk index is
 // XOR-swizzled so that the scan, in which every thread walks 8 consecutive chunks of its own,
