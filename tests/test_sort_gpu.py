@@ -327,6 +327,55 @@ def test_rows_of_up_to_128_keys_through_the_bitonic_network(lib, torch_cuda, dty
     assert lib.cpn_set_bitonic_rows(1) == 1
 
 
+COUNT16_CHILD = r"""
+import numpy as np
+import cupynumeric_amd as num
+from cupynumeric_amd import _lib
+lib = _lib.load()
+rng = np.random.default_rng(5)
+for dtype in (np.float16, np.int16, np.uint16):
+    for seg in (4097, 6000, 8191, 8192):
+        if dtype == np.float16:
+            x = rng.standard_normal((5, seg)).astype(dtype)
+            x[1, ::5] = np.nan
+            x[1, 1::5] = -0.0
+            x[1, 2::5] = 0.0
+            x[2] = x[2, 0]
+            b = x[3].view(np.uint16)
+            b[::7] = 0xFE01  # negative NaN with a payload
+        else:
+            info = np.iinfo(dtype)
+            x = rng.integers(info.min, info.max, (5, seg), dtype=dtype, endpoint=True)
+            x[2] = x[2, 0]
+        lib.cpn_profile_enable(1)
+        _lib.profile_collect()
+        got = np.asarray(num.sort(num.array(x)))
+        labels = {k for k, _ in _lib.profile_collect()}
+        lib.cpn_profile_enable(0)
+        assert "count16_row_sort" in labels, (dtype, seg, labels)
+        want = np.sort(x, axis=-1, kind="stable")
+        u = np.uint16
+        assert np.array_equal(got.view(u), want.view(u)), (dtype, seg)
+print("ok")
+"""
+
+
+def test_counting_kernel_for_rows_of_up_to_8192_keys_behind_its_switch(torch_cuda):
+    """Plain sorts of 4097 ... 8192 two-byte keys take the radix shapes by default; the counting kernel
+    for such rows runs when CPN_SORT_COUNT16_MIN_ROW, read when the library is loaded, lowers its
+    threshold: a child process with that setting sorts rows with NaNs of both signs, payloads, zeros
+    of both signs and constant rows, checks the bits against NumPy's stable sort and that the counting
+    kernel is the one that ran."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, CPN_SORT_COUNT16_MIN_ROW="4097", PYTHONPATH=root + os.pathsep + os.environ.get("PYTHONPATH", ""))
+    out = subprocess.run([sys.executable, "-c", COUNT16_CHILD], env=env, cwd=root, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stdout[-1000:] + out.stderr[-3000:]
+
+
 def test_lds_many_short_rows(lib, torch_cuda):
     for dtype, shape in [(np.float64, (3000, 37)), (np.int8, (5000, 5)), (np.float16, (700, 401)), (np.uint32, (129, 1024))]:
         check_rows(lib, torch_cuda, make_input(dtype, shape, seed=11), f"{np.dtype(dtype)} {shape}")
