@@ -625,9 +625,10 @@ inline int sort_rows_in_lds(const SortRequest& r)
         // (4-12 % on 2- and 4-byte keys); one-pass sorts of single bytes prefer fewer barriers
         if constexpr (sizeof(KeyT) == 1) {
           return launch_lds_rows<KeyT, CODEC, HAS_IDX, 512, 16>(r);
-        } else if constexpr (sizeof(KeyT) == 2 && !HAS_IDX) {
-          // plain sorts of 2-byte keys: two passes in 512-thread shapes, two workgroups per CU, ahead of the
-          // counting kernel up to here (2^26 float16 keys in rows of 4097 0.39 -> 0.27 ms, of 8192 0.20 -> 0.18)
+        } else if constexpr (sizeof(KeyT) == 2) {
+          // 2-byte keys: two passes in 512-thread shapes, two workgroups per CU; for plain sorts ahead of the
+          // counting kernel up to here (2^26 float16 keys in rows of 4097 0.39 -> 0.27 ms, of 8192 0.20 -> 0.18;
+          // with positions, against 1024 threads x 8 keys: rows of 6144 0.40 -> 0.36, of 8192 0.35 -> 0.32)
           if (r.seg <= 6144) {
             return launch_lds_rows<KeyT, CODEC, HAS_IDX, 512, 12>(r);
           }
