@@ -159,6 +159,53 @@ def run_edges() -> dict:
             "unit": "ms", "n_gpus": 1, "data": "synthetic", "edges": table}
 
 
+def run_edges_compact() -> dict:
+    """The same row lengths as --edges on input generated on the device (normal float32 / float16, uniform
+    float64), fastest of 7 single steps through the C ABI, every result checked against torch's stable sort;
+    reports, per key type and operation, the largest step between a row length and its successor and every
+    step above 1.5."""
+    import torch
+
+    out = {}
+    ok = True
+    for dt, op, lengths in EDGE_LENGTHS:
+        kb = np.dtype(dt).itemsize
+        data = device_random(torch, (1 << 26) + (1 << 21), dt, seed=10, law="uniform" if dt == "float64" else "normal")
+        steps = []
+        for n in lengths:
+            rows = (1 << 26) // n
+            ms = []
+            for seg in (n, n + 1):
+                job = GpuJob(dict(x_dev=data[: rows * seg * kb], shape=(rows, seg), dtype=dt, op=op, axis=-1))
+                for _ in range(2):
+                    job.step()
+                best = float("inf")
+                for _ in range(7):
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    job.step()
+                    e1.record()
+                    torch.cuda.synchronize()
+                    best = min(best, e0.elapsed_time(e1))
+                job.check_status()
+                got = job.d_idx.view(torch.uint8) if op == "argsort" else job.d_val
+                ok = ok and verify_against_torch(torch, got, job.d_in, (rows, seg), dt, op, -1) == "ok"
+                ms.append(best)
+                del job, got
+                torch.cuda.empty_cache()
+            steps.append({"row_length": n, "ms_below": round(ms[0], 4), "ms_above": round(ms[1], 4),
+                          "step": round((ms[1] / (rows * (n + 1))) / (ms[0] / (rows * n)), 2)})
+        worst = max(steps, key=lambda e: e["step"])
+        out[f"{dt} {op}"] = {"worst": worst, "above_1.5": [e for e in steps if e["step"] > 1.5 and e is not worst],
+                             "edges_timed": len(steps)}
+        del data
+        torch.cuda.empty_cache()
+    out["verify"] = "ok" if ok else "FAILED"
+    out["what"] = ("rows of n and n + 1 keys for every n at which the library changes kernels, 2^26 keys per sort; "
+                   "step = time per key above / time per key below")
+    return out
+
+
 def algorithmic_bytes(cfg: dict, lds_limit_rows: bool, passes_run: int | None = None) -> dict:
     """Bytes the algorithm has to move, per kernel kind.  `kb` key bytes, `ib` = 4-byte row
     positions between passes (rows shorter than 2^30) and 8-byte int64 on the final write.
@@ -257,7 +304,10 @@ def measure_device_rates(torch) -> dict:
 
 
 class GpuJob:
-    """Device buffers and the call sequence of one workload, through the C ABI."""
+    """Device buffers and the call sequence of one workload, through the C ABI: a sort or argsort
+    along any axis of a dense array (other axes than the last: transposed copy, last-axis sort,
+    transposed copy back, as `sort_swapped` does).  `cfg["x"]` is the host input, or `cfg["x_dev"]`
+    a device byte tensor that already holds it (then `cfg["shape"]` and `cfg["dtype"]` describe it)."""
 
     def __init__(self, cfg: dict):
         import torch
@@ -270,20 +320,29 @@ class GpuJob:
         if not torch.cuda.is_available():
             raise RuntimeError("bench.py needs a HIP device")
         dev = torch.device("cuda:0")
-        x = cfg["x"]
         self.cfg = cfg
-        self.code = _lib.DTYPE_CODES[x.dtype]
-        self.kb = x.dtype.itemsize
+        if cfg.get("x_dev") is not None:
+            self.d_in = cfg["x_dev"]
+            self.shape = tuple(cfg["shape"])
+            self.np_dtype = np.dtype(cfg["dtype"])
+        else:
+            x = cfg["x"]
+            self.shape = x.shape
+            self.np_dtype = x.dtype
+            self.d_in = torch.from_numpy(x.reshape(-1).view(np.uint8)).to(dev)
+        self.code = _lib.DTYPE_CODES[self.np_dtype]
+        self.kb = self.np_dtype.itemsize
         self.argsort = cfg["op"] == "argsort"
-        self.transposed = cfg["axis"] == 0
-        self.shape = x.shape
-        self.volume = x.size
-        self.seg = x.shape[0] if self.transposed else x.shape[-1]
-        self.d_in = torch.from_numpy(x.reshape(-1).view(np.uint8)).to(dev)
+        ndim = len(self.shape)
+        self.axis = cfg["axis"] % ndim
+        self.transposed = self.axis != ndim - 1
+        self.volume = int(np.prod(self.shape, dtype=np.int64))
+        self.seg = self.shape[self.axis]
         self.d_val = None if self.argsort else torch.empty_like(self.d_in)
         self.d_idx = torch.empty(self.volume, dtype=torch.int64, device=dev) if self.argsort else None
         self.d_tr = torch.empty_like(self.d_in) if self.transposed else None
-        in_place = self.transposed  # the transposed copy is sorted in place, as sort_swapped does
+        self.d_idx_tr = torch.empty_like(self.d_idx) if (self.transposed and self.argsort) else None
+        in_place = self.transposed and not self.argsort  # the transposed copy is sorted in place, as sort_swapped does
         self.temp_bytes = self.lib.cpn_local_sort_temp_bytes(
             self.code, self.volume, self.seg, int(not self.argsort), int(self.argsort), int(in_place)
         )
@@ -291,19 +350,28 @@ class GpuJob:
         self.stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
         # rows that fit the per-row LDS kernel need nothing but the workspace header
         self.uses_lds_rows = self.temp_bytes == self.lib.cpn_local_sort_temp_bytes(self.code, 0, 0, 1, 0, 0)
+        if self.transposed:
+            moved = list(self.shape)
+            moved[self.axis], moved[-1] = moved[-1], moved[self.axis]
+            self.c_shape = (ctypes.c_int64 * ndim)(*self.shape)
+            self.c_shape_moved = (ctypes.c_int64 * ndim)(*moved)
 
     def step(self) -> None:
         lib, ck = self.lib, self._lib_mod.check
         if self.transposed:
-            r, c = self.shape
-            shape = (ctypes.c_int64 * 2)(r, c)
-            ck(lib.cpn_swapaxes_copy(self.kb, self.d_in.data_ptr(), self.d_tr.data_ptr(), shape, 2, 0, 1, self.stream),
-               "cpn_swapaxes_copy")
-            ck(lib.cpn_local_sort(self.code, self.d_tr.data_ptr(), self.d_tr.data_ptr(), None, self.volume, self.seg,
-                                  0, 1, self.temp.data_ptr(), self.temp_bytes, self.stream), "cpn_local_sort")
-            shape_t = (ctypes.c_int64 * 2)(c, r)
-            ck(lib.cpn_swapaxes_copy(self.kb, self.d_tr.data_ptr(), self.d_val.data_ptr(), shape_t, 2, 0, 1,
-                                     self.stream), "cpn_swapaxes_copy")
+            ndim, last = len(self.shape), len(self.shape) - 1
+            ck(lib.cpn_swapaxes_copy(self.kb, self.d_in.data_ptr(), self.d_tr.data_ptr(), self.c_shape, ndim, self.axis,
+                                     last, self.stream), "cpn_swapaxes_copy")
+            if self.argsort:
+                ck(lib.cpn_local_sort(self.code, self.d_tr.data_ptr(), None, self.d_idx_tr.data_ptr(), self.volume,
+                                      self.seg, 0, 1, self.temp.data_ptr(), self.temp_bytes, self.stream), "cpn_local_sort")
+                ck(lib.cpn_swapaxes_copy(8, self.d_idx_tr.data_ptr(), self.d_idx.data_ptr(), self.c_shape_moved, ndim,
+                                         self.axis, last, self.stream), "cpn_swapaxes_copy")
+            else:
+                ck(lib.cpn_local_sort(self.code, self.d_tr.data_ptr(), self.d_tr.data_ptr(), None, self.volume, self.seg,
+                                      0, 1, self.temp.data_ptr(), self.temp_bytes, self.stream), "cpn_local_sort")
+                ck(lib.cpn_swapaxes_copy(self.kb, self.d_tr.data_ptr(), self.d_val.data_ptr(), self.c_shape_moved, ndim,
+                                         self.axis, last, self.stream), "cpn_swapaxes_copy")
         else:
             ck(lib.cpn_local_sort(
                 self.code, self.d_in.data_ptr(), None if self.argsort else self.d_val.data_ptr(),
@@ -316,7 +384,7 @@ class GpuJob:
     def result(self) -> np.ndarray:
         if self.argsort:
             return self.d_idx.cpu().numpy().reshape(self.shape)
-        return self.d_val.cpu().numpy().view(self.cfg["x"].dtype).reshape(self.shape)
+        return self.d_val.cpu().numpy().view(self.np_dtype).reshape(self.shape)
 
 
 def verify_sample(job: GpuJob, cfg: dict) -> str:
@@ -810,6 +878,150 @@ def run_sort_workload(name: str, steps: int, warmup: int, log2n=None, rows=None,
     return fields, cfg, job
 
 
+# -------------------------------------------------------------------------------------------------
+# the reference's own sort microbenchmark, through the public API and through the C ABI
+# -------------------------------------------------------------------------------------------------
+TORCH_DTYPES = {"float16": "float16", "float32": "float32", "float64": "float64", "int32": "int32", "int64": "int64"}
+
+# examples/microbenchmarks/sort_bench.py:44-51: the six variants; :104-105: the two dtypes
+MICRO_VARIANTS = ("sort-1D", "argsort-1D", "sort-2D-flat", "argsort-2D-flat", "sort-2D-skinny", "argsort-2D-skinny")
+MICRO_DTYPES = ("float32", "float64")
+
+
+def micro_shape(variant: str, size: int) -> tuple[int, ...]:
+    """Array shape of a variant at `size` (examples/microbenchmarks/sort_bench.py:54-68)."""
+    import math
+
+    if variant.endswith("-1D"):
+        return (size,)
+    a, b = math.ceil(math.pow(size, 1 / 4)), math.ceil(math.pow(size, 3 / 4))
+    return (a, b) if variant.endswith("-2D-flat") else (b, a)
+
+
+def device_random(torch, count: int, dtype: str, seed: int, law: str = "uniform"):
+    """`count` seeded random elements of `dtype` generated on the device, as a byte tensor: uniform in
+    [0, 1) (what the reference's benchmarks sort, examples/_benchmark/random_array.py:43-49) or
+    standard normal."""
+    g = torch.Generator(device="cuda:0")
+    g.manual_seed(seed)
+    tdt = getattr(torch, TORCH_DTYPES[dtype])
+    gen_dt = torch.float32 if tdt == torch.float16 else tdt
+    x = torch.empty(count, dtype=gen_dt, device="cuda:0")
+    if law == "uniform":
+        x.uniform_(0.0, 1.0, generator=g)
+    else:
+        x.normal_(generator=g)
+    return x.to(tdt).view(torch.uint8)
+
+
+def verify_against_torch(torch, result_bytes, input_bytes, shape, dtype: str, op: str, axis: int) -> str:
+    """Element for element against torch's stable sort of the same device input along `axis` (values equal
+    or both NaN; indices equal: the stable argsort is unique)."""
+    tdt = getattr(torch, TORCH_DTYPES[dtype])
+    x = input_bytes.view(tdt).view(shape)
+    ref = torch.sort(x, dim=axis, stable=True)
+    if op == "argsort":
+        same = result_bytes.view(torch.int64).view(shape) == ref.indices
+    else:
+        got = result_bytes.view(tdt).view(shape)
+        same = (got == ref.values) | ((got != got) & (ref.values != ref.values))
+    bad = int((~same).sum())
+    del ref
+    return "ok" if bad == 0 else f"FAILED: {bad} elements differ from torch.sort(stable=True)"
+
+
+def timed_calls(torch, fn, runs: int, warmup: int) -> float:
+    """The reference's timed loop (examples/_benchmark/timer.py:199-241): `warmup` untimed calls, then
+    `runs` calls between a start and a stop that waits for the device; calls are ordered by the stream
+    they are issued on (the reference's fence), the host does not wait between them.  Returns
+    milliseconds per call, host wall clock."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(runs):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / runs
+
+
+def time_case(torch, num, input_bytes, shape, dtype: str, op: str, axis: int, runs: int, warmup: int,
+              verify: bool = True) -> dict:
+    """One case both ways: through the public API (`cupynumeric.sort(x, axis)` / `argsort`: result and
+    workspace allocated per call, status bookkeeping included) and through the C ABI (`cpn_local_sort`
+    and `cpn_swapaxes_copy` with outputs and workspace allocated beforehand)."""
+    from cupynumeric_amd._thunk import DeviceArray
+
+    a = num.ndarray(shape, np.dtype(dtype), thunk=DeviceArray.from_device(input_bytes, shape, dtype))
+    api_fn = (lambda: num.argsort(a, axis)) if op == "argsort" else (lambda: num.sort(a, axis))
+    api_ms = timed_calls(torch, api_fn, runs, warmup)
+    out = {"shape": list(shape), "api_ms": round(api_ms, 5)}
+    if verify:
+        res = api_fn()
+        out["verify"] = verify_against_torch(torch, res._thunk.base.device(), input_bytes, shape, dtype, op, axis)
+        del res
+    torch.cuda.empty_cache()
+    job = GpuJob(dict(x_dev=input_bytes, shape=shape, dtype=dtype, op=op, axis=axis))
+    abi_ms = timed_calls(torch, job.step, runs, warmup)
+    job.check_status()
+    if verify:
+        got = job.d_idx.view(torch.uint8) if op == "argsort" else job.d_val
+        v = verify_against_torch(torch, got, input_bytes, shape, dtype, op, axis)
+        if v != "ok" or out["verify"] != "ok":
+            out["verify"] = f"api: {out['verify']}; abi: {v}"
+    out["abi_ms"] = round(abi_ms, 5)
+    out["api_over_abi"] = round(api_ms / abi_ms, 3)
+    out["keys_per_s_api"] = int(np.prod(shape, dtype=np.int64)) / (api_ms * 1e-3)
+    del job
+    torch.cuda.empty_cache()
+    return out
+
+
+def run_reference_microbenchmarks(log2size: int = 28, runs: int = 5, warmup: int = 2) -> dict:
+    """The plan of the reference's sort microbenchmark (examples/microbenchmarks/sort_bench.py:44-68,
+    104-130) at size 2^log2size: six variants x float32 / float64, `np.sort(x, -1)` / `np.argsort(x, -1)`
+    on uniform [0, 1) input, each through the public API and through the C ABI; sort-1D / argsort-1D of
+    float32 for sizes 2^10 ... 2^26 (the regime of examples/sort.py and of the reference's CI, which runs
+    the suite at size 1000); and two sorts along other axes than the last."""
+    import torch
+
+    import cupynumeric as num
+
+    size = 1 << log2size
+    cases = {}
+    for k, dtype in enumerate(MICRO_DTYPES):
+        data = device_random(torch, size, dtype, seed=11 + k)
+        for variant in MICRO_VARIANTS:
+            op = variant.split("-")[0]
+            cases[f"{variant}:{dtype}"] = time_case(torch, num, data, micro_shape(variant, size), dtype, op, -1, runs, warmup)
+        del data
+        torch.cuda.empty_cache()
+    sweep = {}
+    data = device_random(torch, 1 << 26, "float32", seed=13)
+    for log2s in range(10, 27, 2):
+        n = 1 << log2s
+        reps = 200 if log2s <= 18 else (50 if log2s <= 22 else 10)
+        for op in ("sort", "argsort"):
+            part = data[: 4 * n]
+            r = time_case(torch, num, part, (n,), "float32", op, -1, reps, 5, verify=True)
+            sweep[f"{op}-1D:2^{log2s}"] = {"api_us": round(r["api_ms"] * 1e3, 2), "abi_us": round(r["abi_ms"] * 1e3, 2),
+                                          "api_over_abi": r["api_over_abi"], "verify": r["verify"]}
+    del data
+    torch.cuda.empty_cache()
+    axes = {}
+    data = device_random(torch, 1 << 28, "float32", seed=14)
+    axes["argsort axis 0 of (8192, 8192) float32"] = time_case(
+        torch, num, data[: 4 * 8192 * 8192], (8192, 8192), "float32", "argsort", 0, runs, warmup)
+    axes["sort axis 1 of (256, 512, 2048) float32"] = time_case(
+        torch, num, data, (256, 512, 2048), "float32", "sort", 1, runs, warmup)
+    del data
+    torch.cuda.empty_cache()
+    ok = all(c["verify"] == "ok" for group in (cases, sweep, axes) for c in group.values())
+    return {"size": f"2^{log2size}", "runs": runs, "warmup": warmup, "input": "uniform [0, 1), generated on the device, seeded",
+            "timing": "host wall clock around `runs` calls, device synchronised before the first and after the last",
+            "cases": cases, "sizes_1d_float32": sweep, "other_axes": axes, "verify": "ok" if ok else "FAILED"}
+
+
 # the other workloads reported beside the headline: the baseline's configs and the reference's own
 # 2-D microbenchmark shapes
 ALL_CONFIGS = ("c1", "c3", "c4", "c5", "flat", "skinny")
@@ -835,12 +1047,18 @@ def main() -> None:
     ap.add_argument("--edges", action="store_true",
                     help="instead of a workload: time rows of length n and n + 1 for every n at which the "
                          "library changes kernels (EDGE_LENGTHS), one JSON line")
+    ap.add_argument("--micro", action="store_true",
+                    help="instead of a workload: the reference's sort microbenchmark matrix (six variants x float32 / "
+                         "float64), the 1-D sizes 2^10 ... 2^26 and two sorts along other axes, each through the public "
+                         "API and through the C ABI; one JSON line")
+    ap.add_argument("--micro-log2size", type=int, default=28, help="size of the microbenchmark matrix, 2^L elements")
     ap.add_argument("--log2n", type=int, default=None, help="shrink a 1-D workload to 2^L keys")
     ap.add_argument("--rows", type=int, default=None, help="shrink a 2-D workload to this many rows")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-all-configs", action="store_true",
-                    help="the default run (c2 at full size) also times the other workloads, 10 steps each, and "
-                         "reports them under all_configs; this switch leaves them out")
+                    help="the default run (c2 at full size) also times the other workloads, 10 steps each "
+                         "(all_configs), the reference's microbenchmark matrix through the public API and the C ABI "
+                         "(sort_bench) and the row-length edges (edges); this switch leaves them out")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy, the known-size kernel that "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -850,6 +1068,10 @@ def main() -> None:
 
     if args.edges:
         print(json.dumps(run_edges()))
+        return
+    if args.micro:
+        print(json.dumps({"metric": "ms per call, the reference's sort microbenchmark, public API and C ABI", "unit": "ms",
+                          "n_gpus": 1, "data": "synthetic", "sort_bench": run_reference_microbenchmarks(args.micro_log2size)}))
         return
     if args.config in CONSUMERS:
         print(json.dumps(run_consumer(args)))
@@ -907,6 +1129,8 @@ def main() -> None:
             del j
             torch.cuda.empty_cache()
         line["all_configs"] = others
+        line["sort_bench"] = run_reference_microbenchmarks()
+        line["edges"] = run_edges_compact()
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(cfg)
     print(json.dumps(line))

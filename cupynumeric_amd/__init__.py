@@ -183,10 +183,10 @@ def unique(
 
 
 def take_along_axis(a: Any, indices: Any, axis: int | None) -> ndarray:
-    """Values of `a` at `indices` along `axis` (`cupynumeric/_module/indexing.py:657-770`), for the
-    case the reference's TAKE task covers: every dimension other than `axis` agrees between `a`
-    and `indices` (no broadcasting).  `axis=None` flattens `a` and wants 1-D indices.  Indices out
-    of range raise IndexError."""
+    """Values of `a` at `indices` along `axis` (`cupynumeric/_module/indexing.py:657-770`): every
+    dimension other than `axis` agrees between `a` and `indices` or is 1 on one side (NumPy's
+    broadcasting; shapes that do not broadcast raise IndexError, as in NumPy).  `axis=None` flattens
+    `a` and wants 1-D indices.  Indices out of range raise IndexError from this call."""
     from numpy.lib.array_utils import normalize_axis_index
 
     a = convert_to_ndarray(a)
@@ -205,10 +205,6 @@ def take_along_axis(a: Any, indices: Any, axis: int | None) -> ndarray:
 
     if a.ndim != indices.ndim:
         raise ValueError("`indices` and `a` must have the same number of dimensions")
-    others_a = a.shape[:computed_axis] + a.shape[computed_axis + 1 :]
-    others_i = indices.shape[:computed_axis] + indices.shape[computed_axis + 1 :]
-    if others_a != others_i:
-        raise NotImplementedError("take_along_axis: broadcasting between `a` and `indices` is not supported")
     if indices.dtype != np.dtype(np.int64):
         indices = indices.astype(np.int64)
 

@@ -67,6 +67,23 @@ class ndarray:
             out = out.astype(dtype)
         return out
 
+    def __getitem__(self, key: Any) -> "ndarray":
+        """`a[indices]` for a 1-D array and a 1-D integer array of positions (a cuPyNumeric or NumPy
+        array, or a list), negative positions counting from the end: the indexing that the reference's
+        sort tests apply to `argsort` results (`tests/integration/test_argsort.py:243-245`; advanced
+        indexing in the reference, `cupynumeric/_array/array.py:1236-1263`).  A position out of range
+        raises IndexError when data next reaches the host, not from this call, so that the stream
+        keeps running.  Other kinds of index are not provided."""
+        if isinstance(key, list):
+            key = np.asarray(key, dtype=np.int64) if len(key) == 0 else np.asarray(key)
+        if isinstance(key, np.ndarray):
+            key = convert_to_ndarray(key)
+        if not isinstance(key, ndarray) or key.ndim != 1 or self.ndim != 1 or not np.issubdtype(key.dtype, np.integer):
+            raise NotImplementedError(
+                "only a[indices] with a 1-D integer index array on a 1-D array is provided by this package"
+            )
+        return self.take_1d(key)
+
     def flatten(self, order: str = "C") -> "ndarray":
         """Dense 1-D copy (C order)."""
         if order not in ("C", "K", "A"):
@@ -143,7 +160,7 @@ class ndarray:
         """`a.take(indices)` for 1-D `a` and 1-D integer `indices`: what `searchsorted` does with
         its `sorter` (`cupynumeric/_array/array.py:3766`)."""
         idx = indices if indices.dtype == np.dtype(np.int64) else indices.astype(np.int64)
-        thunk = self._thunk.take_along_last_axis(idx._thunk)
+        thunk = self._thunk.take_along_last_axis(idx._thunk, check="deferred")
         return ndarray(thunk.shape, thunk.dtype, thunk=thunk)
 
     def searchsorted(self, v: Any, side: str = "left", sorter: Any = None) -> "ndarray":

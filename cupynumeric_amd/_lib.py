@@ -45,6 +45,9 @@ CPN_ERR_DEVICE = -7
 CPN_ERR_UNSUPPORTED = -8
 CPN_ERR_SCRATCH = -9
 
+# include/cpn_sort.h: options of cpn_local_sort_ex
+CPN_SORT_SINGLE_TICKET = 1
+
 # include/cpn_sort.h: workspace of cpn_local_sort_static
 STATIC_SCRATCH_BYTES = 64 << 20
 
@@ -67,6 +70,11 @@ PROTOTYPES: dict[str, tuple] = {
     "cpn_local_sort": (
         c_int,
         [c_int, c_void_p, c_void_p, c_void_p, c_uint64, c_uint64, c_int64, c_int, c_void_p, c_uint64, c_void_p],
+    ),
+    "cpn_local_sort_ex": (
+        c_int,
+        [c_int, c_void_p, c_void_p, c_void_p, c_uint64, c_uint64, c_int64, c_int, ctypes.c_uint32, c_void_p, c_uint64,
+         c_void_p],
     ),
     "cpn_local_sort_static": (
         c_int, [c_int, c_void_p, c_void_p, c_void_p, c_uint64, c_uint64, c_int64, c_int, c_void_p, c_void_p]
@@ -92,6 +100,11 @@ PROTOTYPES: dict[str, tuple] = {
     ),
     "cpn_take_along_last_axis": (
         c_int, [c_int, c_void_p, c_void_p, c_void_p, c_uint64, c_uint64, c_uint64, c_void_p, c_void_p]
+    ),
+    "cpn_take_along_last_axis_broadcast": (
+        c_int,
+        [c_int, c_void_p, c_void_p, c_void_p, c_int, ctypes.POINTER(c_uint64), ctypes.POINTER(c_uint64),
+         ctypes.POINTER(c_uint64), c_uint64, c_uint64, c_void_p, c_void_p],
     ),
     "cpn_lexsort_pack": (
         c_int,

@@ -78,9 +78,9 @@ def sort_task(output: "DeviceArray", input: "DeviceArray", argsort: bool, stable
         raise NotImplementedError(f"cpn_local_sort: no workspace layout for dtype={input.dtype}, shape={input.shape}")
     stream = ctypes.c_void_p(runtime.stream_handle())
 
-    def issue():
+    def issue(options: int = 0):
         temp = runtime.empty_bytes(temp_bytes)
-        status = lib.cpn_local_sort(
+        status = lib.cpn_local_sort_ex(
             code,
             values_in,
             values_out,
@@ -89,6 +89,7 @@ def sort_task(output: "DeviceArray", input: "DeviceArray", argsort: bool, stable
             seg,
             0,  # rect.lo[last] of a single-GPU launch (`src/cupynumeric/sort/sort.cu:1851`)
             int(stable),
+            options,
             temp.data_ptr(),
             temp_bytes,
             stream,
@@ -106,14 +107,11 @@ def sort_task(output: "DeviceArray", input: "DeviceArray", argsort: bool, stable
         return
     status = lib.cpn_local_sort_check(temp.data_ptr(), stream)
     if status == _lib.CPN_ERR_DEVICE and not in_place:
-        # once more, from a fresh workspace, with the tiles handed out through one counter: that order
-        # does not depend on every XCD taking part (the input was not touched: it is not the output)
-        previous = lib.cpn_set_tile_order(1)
-        try:
-            temp = issue()
-            status = lib.cpn_local_sort_check(temp.data_ptr(), stream)
-        finally:
-            lib.cpn_set_tile_order(previous)
+        # once more, from a fresh workspace, with the tiles of this one call handed out through one
+        # counter: that order does not depend on every XCD taking part (the input was not touched: it
+        # is not the output).  Nothing process-wide changes, so other threads sort on undisturbed.
+        temp = issue(_lib.CPN_SORT_SINGLE_TICKET)
+        status = lib.cpn_local_sort_check(temp.data_ptr(), stream)
     _lib.check(status, "cpn_local_sort")
 
 
@@ -227,12 +225,12 @@ def lexsort_deferred(keys: "list[DeviceArray]", axis: int) -> "DeviceArray":
         if len(group) == 1 and indices is None:
             key_reordered = group[0]  # first key: nothing to reorder, no need to pack
         elif group[0].dtype.kind == "c":
-            key_reordered = group[0].take_along_last_axis(indices)
+            key_reordered = group[0].take_along_last_axis(indices, check="trusted")
         else:
             key_reordered = _pack_keys(group, indices)
         order = DeviceArray(key_reordered.shape, dtype="int64")
         sort_task(order, key_reordered, True, True)
-        indices = order if indices is None else indices.take_along_last_axis(order)
+        indices = order if indices is None else indices.take_along_last_axis(order, check="trusted")
 
     if axis != last:
         indices = indices.swapaxes_copy(last, axis)

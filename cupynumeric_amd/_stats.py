@@ -330,6 +330,7 @@ def nanquantile(
         d_counts = torch.empty(slices, dtype=torch.int64, device=dev)
         _lib.check(lib.cpn_count_not_nan_sorted(code, src, outer, n, inner, d_counts.data_ptr(), stream),
                    "cpn_count_not_nan_sorted")
+        runtime.flush_status()  # a failed sort must not reach the host through the counts
         counts = d_counts.cpu().numpy()  # (synchronises: the positions below depend on the counts)
         # positions and weights per quantile and slice, worked out once per different count
         # (`stats_order.py:713-746`)

@@ -74,6 +74,19 @@ class DeviceArray:
         host = np.array(arr, dtype=dt, order="C", copy=True)
         return cls(host.shape, dt, Storage(host.nbytes, host=host))
 
+    @classmethod
+    def from_device(cls, buf: "torch.Tensor", shape: tuple[int, ...], dtype: Any) -> "DeviceArray":
+        """An array over device memory that already holds its dense row-major data: `buf` is a
+        contiguous torch tensor on the GPU (any element type) of exactly the array's bytes.  The
+        memory is shared, not copied."""
+        dt = check_dtype(dtype)
+        raw = buf.reshape(-1).view(runtime.torch.uint8)
+        out = cls(shape, dt, Storage(raw.numel()))
+        if raw.numel() != out.size * dt.itemsize or not raw.is_cuda:
+            raise ValueError("from_device: the buffer must be device memory of exactly shape x dtype bytes")
+        out.base._dev = raw
+        return out
+
     @property
     def ndim(self) -> int:
         return len(self.shape)
@@ -143,37 +156,66 @@ class DeviceArray:
         _lib.check(status, "cpn_swapaxes_copy")
         return out
 
-    def take_along_last_axis(self, indices: "DeviceArray") -> "DeviceArray":
+    def take_along_last_axis(self, indices: "DeviceArray", check: str = "now") -> "DeviceArray":
         """`take_along_axis(self, indices, axis=-1)` for arrays whose leading dimensions agree
-        (`cupynumeric/_module/indexing.py:648-760`; the TAKE task's no-broadcast case)."""
+        (`cupynumeric/_module/indexing.py:648-760`; the TAKE task's no-broadcast case).
+
+        `check`: what happens to the kernel's out-of-bounds flag.  "now": read back before returning
+        (one stream synchronisation; the public `take_along_axis` raises IndexError from the call, as
+        the reference does); "deferred": reported with the next host read (`runtime.flush_status`), so
+        that the stream keeps running; "trusted": no flag at all, for indices that this package
+        produced itself (the argsorts inside `lexsort`)."""
         if indices.dtype != np.dtype(np.int64):
             raise TypeError("`indices` must be an int64 array")
         if self.ndim != indices.ndim or self.ndim == 0:
             raise ValueError("`indices` and `a` must have the same number of dimensions")
-        if self.shape[:-1] != indices.shape[:-1]:
-            raise ValueError("take_along_last_axis: leading dimensions must agree")
-        out = DeviceArray(indices.shape, self.dtype)
+        lead_a, lead_i = self.shape[:-1], indices.shape[:-1]
+        if any(m != n and m != 1 and n != 1 for m, n in zip(lead_a, lead_i)):
+            raise IndexError(
+                "shape mismatch: indexing arrays could not be broadcast together with shapes "
+                f"{self.shape} {indices.shape} (every dimension but the axis must agree or be 1)"
+            )
+        lead_out = tuple(max(m, n) if min(m, n) != 0 else 0 for m, n in zip(lead_a, lead_i))
+        out = DeviceArray(lead_out + indices.shape[-1:], self.dtype)
         if out.size == 0:
             return out
         if self.shape[-1] == 0:
             raise IndexError("index out of bounds: cannot take from an empty axis")
         lib = _lib.load()
-        rows = indices.size // indices.shape[-1]
-        flag = runtime.zero_flag()
-        status = lib.cpn_take_along_last_axis(
-            self.dtype.itemsize,
-            self.base.ptr(),
-            indices.base.ptr(),
-            out.base.ptr(),
-            rows,
-            self.shape[-1],
-            indices.shape[-1],
-            flag.data_ptr(),
-            ctypes.c_void_p(runtime.stream_handle()),
-        )
+        if runtime.check_mode == "off":
+            check = "trusted"
+        elif runtime.check_mode == "eager" and check == "deferred":
+            check = "now"
+        flag = runtime.zero_flag() if check != "trusted" else None
+        flag_ptr = flag.data_ptr() if flag is not None else None
+        stream = ctypes.c_void_p(runtime.stream_handle())
+        if lead_a == lead_i:
+            status = lib.cpn_take_along_last_axis(
+                self.dtype.itemsize, self.base.ptr(), indices.base.ptr(), out.base.ptr(), out.size // indices.shape[-1],
+                self.shape[-1], indices.shape[-1], flag_ptr, stream,
+            )
+        else:
+            # rows per step of each leading dimension on either side: the dense stride, 0 where broadcast
+            def row_strides(lead: tuple[int, ...]) -> list[int]:
+                strides, run = [0] * len(lead), 1
+                for d in range(len(lead) - 1, -1, -1):
+                    strides[d] = run if lead[d] != 1 else 0
+                    run *= lead[d]
+                return strides
+
+            n = len(lead_out)
+            u64 = ctypes.c_uint64 * max(n, 1)
+            status = lib.cpn_take_along_last_axis_broadcast(
+                self.dtype.itemsize, self.base.ptr(), indices.base.ptr(), out.base.ptr(), n, u64(*lead_out),
+                u64(*row_strides(lead_a)), u64(*row_strides(lead_i)), self.shape[-1], indices.shape[-1], flag_ptr, stream,
+            )
         _lib.check(status, "cpn_take_along_last_axis")
-        if runtime.check_mode != "off" and int(flag.item()) != 0:
-            raise IndexError("index out of bounds in take_along_axis")
+        if check == "deferred":
+            runtime.defer_flag(flag, "index")
+        elif check == "now":
+            runtime.flush_status()  # (errors of earlier work first: the read below synchronises anyway)
+            if int(flag.item()) != 0:
+                raise IndexError("index out of bounds in take_along_axis")
         return out
 
     # -- the sort entry point ---------------------------------------------------------------
@@ -294,6 +336,7 @@ class DeviceArray:
         )
         _lib.check(status, "cpn_unique")
         if runtime.check_mode != "off":  # (reading the count below synchronises anyway)
+            runtime.flush_status()  # errors of earlier work first
             _lib.check(lib.cpn_local_sort_check(temp.data_ptr(), stream), "cpn_unique")
         n_unique = int(count.item())
         return DeviceArray((n_unique,), self.dtype, out.base)

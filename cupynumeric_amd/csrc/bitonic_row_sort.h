@@ -1,6 +1,6 @@
 // Rows of up to 64 elements of real keys of up to 8 bytes, one element per lane and 64/S rows per
-// wavefront (S = slots per row, the next power of two), and rows of up to 128 keys of up to 4
-// bytes, two elements per lane and one row per wavefront, sorted by a bitonic network of
+// wavefront (S = slots per row, the next power of two), and rows of 65 ... 128 such keys, two
+// elements per lane and one row per wavefront, sorted by a bitonic network of
 // compare-exchanges between lanes.  What is compared is (order-preserving image of the key,
 // position in the row) as one unsigned word (an image and a position word for 8-byte keys), so
 // that no two are equal: the network, which is not stable by itself, then yields exactly the
@@ -49,9 +49,10 @@ __device__ __forceinline__ uint64_t lane_xor(uint64_t v)
   return (static_cast<uint64_t>(hi) << 32) | lo;
 }
 
-// 8-byte keys: the image and the position side by side, compared image first (one element per
-// lane only: two per lane measured slower than the ranking kernel, 0.62 against 0.49 ms for 2^26
-// float64 keys in rows of 128).
+// 8-byte keys: the image and the position side by side, compared image first.  Two elements per
+// lane (rows of 65 ... 128) pay off for them as well once the select between two words is written
+// member by member (below): 2^26 float64 keys in rows of 128 0.49 ms through the ranking kernel,
+// 0.42 ms here (0.62 ms while the select went through memory).
 struct ImagePos {
   uint64_t image;
   uint64_t pos;  // (64 bits so that the struct has no padding; 32 of them travel)

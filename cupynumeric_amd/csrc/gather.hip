@@ -60,6 +60,71 @@ static int launch_take(const void* src, const int64_t* idx, void* out, uint64_t 
   return CPN_OK;
 }
 
+// The same gather when the leading dimensions of `src` and `idx` broadcast against each other
+// (NumPy's take_along_axis lets every dimension but the axis be 1 on either side): the row of the
+// source and of the indices that belong to an output row follow from the row's coordinates and a
+// stride per dimension, 0 where that side is broadcast.
+constexpr int TAKE_MAX_LEAD = 7;
+struct TakeLead {
+  int ndim;
+  uint64_t shape[TAKE_MAX_LEAD];       // leading dimensions of the output
+  uint64_t src_stride[TAKE_MAX_LEAD];  // rows of src per step in that dimension (0: broadcast)
+  uint64_t idx_stride[TAKE_MAX_LEAD];  // rows of idx per step
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void take_last_axis_broadcast_kernel(const T* __restrict__ src,
+                                                                        const int64_t* __restrict__ idx,
+                                                                        T* __restrict__ out,
+                                                                        uint64_t total,
+                                                                        uint64_t src_seg,
+                                                                        uint64_t idx_seg,
+                                                                        TakeLead lead,
+                                                                        uint32_t* oob_flag)
+{
+  const uint64_t stride = static_cast<uint64_t>(gridDim.x) * blockDim.x;
+  bool bad              = false;
+  for (uint64_t o = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x; o < total; o += stride) {
+    uint64_t row = o / idx_seg;
+    const uint64_t j = o - row * idx_seg;
+    uint64_t src_row = 0, idx_row = 0;
+    for (int d = lead.ndim - 1; d >= 0; --d) {
+      const uint64_t c = row % lead.shape[d];
+      row /= lead.shape[d];
+      src_row += c * lead.src_stride[d];
+      idx_row += c * lead.idx_stride[d];
+    }
+    int64_t k = idx[idx_row * idx_seg + j];
+    if (k < 0) {
+      k += static_cast<int64_t>(src_seg);
+    }
+    if (k < 0 || static_cast<uint64_t>(k) >= src_seg) {
+      bad = true;
+    } else {
+      out[o] = src[src_row * src_seg + static_cast<uint64_t>(k)];
+    }
+  }
+  if (bad && oob_flag != nullptr) {
+    __hip_atomic_store(oob_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+template <typename T>
+static int launch_take_broadcast(const void* src, const int64_t* idx, void* out, uint64_t rows, uint64_t src_seg,
+                                 uint64_t idx_seg, const TakeLead& lead, uint32_t* oob_flag, hipStream_t stream)
+{
+  const uint64_t total = rows * idx_seg;
+  uint64_t grid        = (total + 255) / 256;
+  if (grid > (1u << 20)) {
+    grid = 1u << 20;
+  }
+  ProfileScope prof("take_last_axis", stream);
+  hipLaunchKernelGGL((take_last_axis_broadcast_kernel<T>), dim3(static_cast<uint32_t>(grid)), dim3(256), 0, stream,
+                     static_cast<const T*>(src), idx, static_cast<T*>(out), total, src_seg, idx_seg, lead, oob_flag);
+  CPN_HIP_TRY(hipGetLastError());
+  return CPN_OK;
+}
+
 // ---- lexsort: several keys packed into one ------------------------------------------------
 //
 // A lexicographic order on keys (k_last, ..., k_0) is the order of the unsigned number whose
@@ -215,6 +280,54 @@ extern "C" int cpn_take_along_last_axis(int elem_bytes, const void* src, const i
     case 4: return cpn::launch_take<uint32_t>(src, indices, out, rows, src_seg, idx_seg, oob_flag, s);
     case 8: return cpn::launch_take<uint64_t>(src, indices, out, rows, src_seg, idx_seg, oob_flag, s);
     case 16: return cpn::launch_take<cpn::U128>(src, indices, out, rows, src_seg, idx_seg, oob_flag, s);
+    default: return CPN_ERR_DTYPE;
+  }
+}
+
+extern "C" int cpn_take_along_last_axis_broadcast(int elem_bytes, const void* src, const int64_t* indices, void* out,
+                                                  int lead_ndim, const uint64_t* out_lead_shape,
+                                                  const uint64_t* src_lead_strides, const uint64_t* idx_lead_strides,
+                                                  uint64_t src_seg, uint64_t idx_seg, uint32_t* oob_flag, void* stream)
+{
+  if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8 && elem_bytes != 16) {
+    return CPN_ERR_DTYPE;
+  }
+  if (lead_ndim < 0 || lead_ndim > cpn::TAKE_MAX_LEAD) {
+    return CPN_ERR_SHAPE;
+  }
+  if (lead_ndim > 0 && (out_lead_shape == nullptr || src_lead_strides == nullptr || idx_lead_strides == nullptr)) {
+    return CPN_ERR_NULL;
+  }
+  cpn::TakeLead lead{};
+  lead.ndim     = lead_ndim;
+  uint64_t rows = 1;
+  for (int d = 0; d < lead_ndim; ++d) {
+    lead.shape[d]      = out_lead_shape[d];
+    lead.src_stride[d] = src_lead_strides[d];
+    lead.idx_stride[d] = idx_lead_strides[d];
+    rows *= out_lead_shape[d];
+  }
+  if (rows == 0 || idx_seg == 0) {
+    return CPN_OK;
+  }
+  if (src == nullptr || indices == nullptr || out == nullptr) {
+    return CPN_ERR_NULL;
+  }
+  if (src_seg == 0) {
+    return CPN_ERR_SHAPE;  // nothing to take from
+  }
+  const uint64_t align = static_cast<uint64_t>(elem_bytes);
+  if ((reinterpret_cast<uintptr_t>(src) % align) != 0 || (reinterpret_cast<uintptr_t>(out) % align) != 0 ||
+      (reinterpret_cast<uintptr_t>(indices) % 8) != 0) {
+    return CPN_ERR_ALIGN;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (elem_bytes) {
+    case 1: return cpn::launch_take_broadcast<uint8_t>(src, indices, out, rows, src_seg, idx_seg, lead, oob_flag, s);
+    case 2: return cpn::launch_take_broadcast<uint16_t>(src, indices, out, rows, src_seg, idx_seg, lead, oob_flag, s);
+    case 4: return cpn::launch_take_broadcast<uint32_t>(src, indices, out, rows, src_seg, idx_seg, lead, oob_flag, s);
+    case 8: return cpn::launch_take_broadcast<uint64_t>(src, indices, out, rows, src_seg, idx_seg, lead, oob_flag, s);
+    case 16: return cpn::launch_take_broadcast<cpn::U128>(src, indices, out, rows, src_seg, idx_seg, lead, oob_flag, s);
     default: return CPN_ERR_DTYPE;
   }
 }

@@ -421,7 +421,7 @@ void lds_row_sort_kernel(const KeyT* keys_in,
       // The bin of a key: its place between the smallest and the largest key, in equal steps of the
       // value.  Float keys: subtraction of a constant, scaling and truncation never decrease with the
       // key, rounding included, so a key in a lower bin is a smaller key, which is all the split
-      // needs.  (An infinite extreme or span makes the scale 0 or the product NaN, which converts to
+      // needs.  (An infinite extreme or span makes the scale 0 or the product NaN, which is clamped to
       // bin 0: the row then crowds one bin and takes the radix passes.)  Integer keys: the distance
       // from the smallest key, shifted down until the largest distance fits the bins.
       using FT = typename std::conditional<sizeof(KeyT) == 4, float, double>::type;
@@ -439,8 +439,15 @@ void lds_row_sort_kernel(const KeyT* keys_in,
       }
       auto bin_of = [&](KeyT k) -> uint32_t {
         if constexpr (CODEC == CODEC_FLOAT) {
-          const uint32_t b = static_cast<uint32_t>((native(k) - origin) * scale);
-          return b < static_cast<uint32_t>(BINS) ? b : static_cast<uint32_t>(BINS - 1);
+          // (clamped as a floating-point value before the conversion, which is undefined for NaN and
+          // out-of-range values; fmax returns its other operand for a NaN)
+          FT t = (native(k) - origin) * scale;
+          if constexpr (sizeof(FT) == 4) {
+            t = __builtin_fminf(__builtin_fmaxf(t, 0.0f), static_cast<float>(BINS - 1));
+          } else {
+            t = __builtin_fmin(__builtin_fmax(t, 0.0), static_cast<double>(BINS - 1));
+          }
+          return static_cast<uint32_t>(t);
         } else {
           return static_cast<uint32_t>(static_cast<KeyT>(ordered_bits<CODEC, KeyT>(k) - img_lo) >> shift);
         }

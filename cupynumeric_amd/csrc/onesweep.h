@@ -449,6 +449,10 @@ struct SweepArgs {
   const VirtPlan* vplan;   // virtual digits (virtual_digits.h), nullptr when the request cannot use them
   const DistinctTable* dtable;  // with vplan: the row's different keys when there are at most 256
   int free_rank;                // from the plan: this pass need not be stable
+  // Index-only requests that may run on the ranks of the row's different keys: that one pass, when it
+  // is to run, has been done by a launch of its own in a shape that stages one byte per key (DONLY
+  // below), and the launch of the pass itself has nothing left to do.
+  uint32_t distinct_pass_done;
 };
 
 // ---- which tile a workgroup takes ----
@@ -510,6 +514,15 @@ __device__ __forceinline__ uint32_t claim_tile(uint32_t* xcd_tickets, uint32_t n
 #define CPN_ONESWEEP_WAVES_PER_EU 4
 #endif
 
+// Bytes per key of the LDS staging area: the wider of key and row position; DONLY kernels stage one
+// byte per key (its digit) and the row positions.
+template <typename KeyT, typename OffT, bool HAS_IDX, bool DONLY>
+__host__ __device__ constexpr int sweep_stage_elem()
+{
+  return DONLY ? static_cast<int>(sizeof(OffT))
+               : ((HAS_IDX && sizeof(OffT) > sizeof(KeyT)) ? static_cast<int>(sizeof(OffT)) : static_cast<int>(sizeof(KeyT)));
+}
+
 // Shared-memory view of one onesweep workgroup.
 template <typename KeyT, typename OffT, int WAVES, int TILE, int STAGE_ELEM>
 struct SweepShared {
@@ -528,15 +541,19 @@ struct SweepShared {
 // unsigned image as soon as they are loaded and writes them out that way; every pass extracts
 // digits with the identity codec, so the key transform is paid once per key instead of twice
 // per pass.  The values themselves are never returned in that case.
-template <typename KeyT, int CODEC, bool XFORM, bool BIG, bool HAS_IDX, int BLOCK, int ITEMS, bool FULL, bool VIRT>
+//
+// DONLY (with VIRT and HAS_IDX): the pass stores no keys (the one pass of an index-only sort on the
+// ranks of the row's different keys); the keys are turned into digits as they arrive and only
+// the digits, one byte each, go through LDS.
+template <typename KeyT, int CODEC, bool XFORM, bool BIG, bool HAS_IDX, int BLOCK, int ITEMS, bool FULL, bool VIRT,
+          bool DONLY = false>
 __device__ __forceinline__ void onesweep_tile(
   const SweepArgs<BIG>& a,
   const uint32_t vcount,    // VIRT: positions in this pass's group, their bit offsets (8 bits each)
   const uint64_t voffsets,  //       and their shifted lookup tables in LDS (virtual_digits.h)
   const uint8_t* vlut,
   SweepShared<KeyT, typename RowWidth<BIG>::off_t, BLOCK / WAVE, BLOCK * ITEMS,
-              ((HAS_IDX && sizeof(typename RowWidth<BIG>::off_t) > sizeof(KeyT)) ? sizeof(typename RowWidth<BIG>::off_t)
-                                                                                : sizeof(KeyT))>& sh,
+              sweep_stage_elem<KeyT, typename RowWidth<BIG>::off_t, HAS_IDX, DONLY>()>& sh,
   const uint32_t tile,
   const uint64_t row,
   const uint32_t trow,
@@ -561,11 +578,17 @@ __device__ __forceinline__ void onesweep_tile(
 
   // ---- load: item i of lane l is element  wave*WTILE + i*64 + l  of the tile ----
   const KeyT* kin = static_cast<const KeyT*>(a.keys_in) + row_base + tile_off;
-  KeyT key[ITEMS];
-#pragma unroll
-  for (int i = 0; i < ITEMS; ++i) {
+  // (DONLY: the keys are not kept; they arrive in groups of KEY_GROUP rounds, one group ahead of the
+  // ranking, see below)
+  constexpr int KEY_GROUP = 8;
+  KeyT key[DONLY ? KEY_GROUP : ITEMS];
+  auto load_key = [&](int i) -> KeyT {
     const uint32_t o = woff + i * WAVE;
-    key[i]           = (FULL || o < count) ? kin[o] : KeyT{};
+    return (FULL || o < count) ? kin[o] : KeyT{};
+  };
+#pragma unroll
+  for (int i = 0; i < (DONLY ? KEY_GROUP : ITEMS); ++i) {
+    key[i] = load_key(i);
   }
   if constexpr (XFORM) {
     if (a.first) {  // one uniform branch around all items, so that the loads above stay batched
@@ -587,16 +610,19 @@ __device__ __forceinline__ void onesweep_tile(
   const uint32_t* rank_base    = free_first ? sh.ctr : wctr;
   uint32_t dpk[ITEMS / 4];   // the digits, four per register
   uint32_t rnk2[ITEMS / 2];  // rank among the wave's keys of the same digit, two per register
-#pragma unroll
-  for (int i = 0; i < ITEMS; ++i) {
+  auto rank_item = [&](const int i, const KeyT k) {
     const bool valid = FULL || (woff + i * WAVE < count);
     uint32_t d;
-    if constexpr (VIRT) {
+    if constexpr (DONLY) {
       uint64_t ow[KeyTraits<DCODEC, KeyT>::NWORDS];
-      KeyTraits<DCODEC, KeyT>::words(key[i], ow);
+      KeyTraits<DCODEC, KeyT>::words(k, ow);
+      d = distinct_rank(ow[0], reinterpret_cast<const uint64_t*>(vlut), vlut + DISTINCT_LOOKUP * 8);
+    } else if constexpr (VIRT) {
+      uint64_t ow[KeyTraits<DCODEC, KeyT>::NWORDS];
+      KeyTraits<DCODEC, KeyT>::words(k, ow);
       d = virtual_digit(ow[0], vcount, voffsets, vlut);
     } else {
-      d = KeyTraits<DCODEC, KeyT>::digit(key[i], a.pass);
+      d = KeyTraits<DCODEC, KeyT>::digit(k, a.pass);
     }
     dpk[i / 4]       = (i % 4 == 0) ? d : (dpk[i / 4] | (d << (8 * (i % 4))));
     uint32_t r;
@@ -609,6 +635,32 @@ __device__ __forceinline__ void onesweep_tile(
     // the packed registers are opaque to the optimiser, which would otherwise keep every
     // digit and rank alive in a register of its own until the scatter phase
     asm volatile("" : "+v"(dpk[i / 4]), "+v"(rnk2[i / 2]));
+  };
+  if constexpr (DONLY) {
+    // 32 eight-byte keys would take 64 registers: the loads of the next KEY_GROUP rounds are issued
+    // before the current group is ranked, and a key is dropped as soon as its digit is known
+    static_assert(ITEMS % KEY_GROUP == 0, "whole groups of rounds");
+#pragma unroll
+    for (int g = 0; g < ITEMS / KEY_GROUP; ++g) {
+      KeyT ahead[KEY_GROUP];
+#pragma unroll
+      for (int j = 0; j < KEY_GROUP; ++j) {
+        ahead[j] = (g + 1 < ITEMS / KEY_GROUP) ? load_key((g + 1) * KEY_GROUP + j) : KeyT{};
+      }
+#pragma unroll
+      for (int j = 0; j < KEY_GROUP; ++j) {
+        rank_item(g * KEY_GROUP + j, key[j]);
+      }
+#pragma unroll
+      for (int j = 0; j < KEY_GROUP; ++j) {
+        key[j] = ahead[j];
+      }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      rank_item(i, key[i]);
+    }
   }
   __syncthreads();
 
@@ -658,7 +710,7 @@ __device__ __forceinline__ void onesweep_tile(
   // ---- scatter into LDS: counter = first position of this wave's keys with that digit ----
   // VIRT kernels, passes that store no keys (the last pass of an index-only sort): only the digits
   // travel, one byte each, and the table lookups for the second use of the digit fall away
-  const bool digits_only = VIRT && (a.keys_out == nullptr);
+  const bool digits_only = DONLY || (VIRT && (a.keys_out == nullptr));
   uint32_t pos2[ITEMS / 2];  // positions in the sorted tile, two per register
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
@@ -667,7 +719,7 @@ __device__ __forceinline__ void onesweep_tile(
     if (FULL || (woff + i * WAVE < count)) {
       if (VIRT && digits_only) {
         reinterpret_cast<uint8_t*>(s_keys)[pos] = static_cast<uint8_t>(d);
-      } else {
+      } else if constexpr (!DONLY) {
         s_keys[pos] = key[i];
       }
     }
@@ -752,7 +804,7 @@ __device__ __forceinline__ void onesweep_tile(
       const uint32_t d = (FULL || p < count) ? s_digits[p] : 0u;
       dq[k / 4]        = (k % 4 == 0) ? d : (dq[k / 4] | (d << (8 * (k % 4))));
     }
-  } else {
+  } else if constexpr (!DONLY) {
     KeyT kk[ITEMS];
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
@@ -828,11 +880,13 @@ __device__ __forceinline__ void onesweep_tile(
   }
 }
 
-template <typename KeyT, int CODEC, bool XFORM, bool BIG, bool HAS_IDX, int BLOCK, int ITEMS, bool VIRT = false>
+template <typename KeyT, int CODEC, bool XFORM, bool BIG, bool HAS_IDX, int BLOCK, int ITEMS, bool VIRT = false,
+          bool DONLY = false>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(CPN_ONESWEEP_WAVES_PER_EU)))
 void onesweep_kernel(const SweepArgs<BIG> a_in)
 {
   static_assert(!VIRT || (KeyTraits<CODEC, KeyT>::NWORDS == 1 && sizeof(KeyT) <= 8), "virtual digits: one ordered word");
+  static_assert(!DONLY || (VIRT && HAS_IDX && !XFORM), "digits-only kernels: the index-only pass on the ranks of the different keys");
   // VIRT kernels can do both: the device-side plan says whether this sort runs on virtual digits
   bool virt_on = false;
   if constexpr (VIRT) {
@@ -843,7 +897,7 @@ void onesweep_kernel(const SweepArgs<BIG> a_in)
   static_assert(ITEMS % 4 == 0, "digits are cached four to a register");
   constexpr int WAVES      = BLOCK / WAVE;
   constexpr int TILE       = BLOCK * ITEMS;
-  constexpr int STAGE_ELEM = (HAS_IDX && sizeof(OffT) > sizeof(KeyT)) ? sizeof(OffT) : sizeof(KeyT);
+  constexpr int STAGE_ELEM = sweep_stage_elem<KeyT, OffT, HAS_IDX, DONLY>();
   static_assert(TILE <= 65536, "positions inside a tile are kept in 16 bits");
 
   __shared__ SweepShared<KeyT, OffT, WAVES, TILE, STAGE_ELEM> sh;
@@ -854,6 +908,14 @@ void onesweep_kernel(const SweepArgs<BIG> a_in)
   const PassPlan pp = a_in.plan->pass[a_in.pass];
   if (pp.active == 0) {
     return;  // every key of every row has the same digit here
+  }
+  if constexpr (VIRT) {
+    // the index-only pass on the ranks of the row's different keys belongs to the DONLY launch,
+    // where the request has one (distinct_pass_done), and everything else does not
+    const bool its_pass = virt_on && a_in.vplan->enabled == VIRT_DISTINCT && pp.key_dst == BUF_NONE;
+    if (DONLY ? !its_pass : (its_pass && a_in.distinct_pass_done != 0)) {
+      return;
+    }
   }
   if (VIRT && virt_on && a_in.vplan->enabled == VIRT_DISTINCT) {
     // the one pass on the ranks of the row's different keys: their lookup table into LDS
@@ -921,19 +983,21 @@ void onesweep_kernel(const SweepArgs<BIG> a_in)
   const uint64_t remain = a.seg - static_cast<uint64_t>(trow) * TILE;
   if (VIRT && virt_on) {  // uniform for the launch
     if (remain >= static_cast<uint64_t>(TILE)) {
-      onesweep_tile<KeyT, CODEC, XFORM, BIG, HAS_IDX, BLOCK, ITEMS, true, VIRT>(a, vcount, voffsets, s_vlut, sh, tile, row,
-                                                                               trow, TILE);
+      onesweep_tile<KeyT, CODEC, XFORM, BIG, HAS_IDX, BLOCK, ITEMS, true, VIRT, DONLY>(a, vcount, voffsets, s_vlut, sh, tile,
+                                                                                      row, trow, TILE);
     } else {
-      onesweep_tile<KeyT, CODEC, XFORM, BIG, HAS_IDX, BLOCK, ITEMS, false, VIRT>(a, vcount, voffsets, s_vlut, sh, tile, row,
-                                                                                trow, static_cast<uint32_t>(remain));
+      onesweep_tile<KeyT, CODEC, XFORM, BIG, HAS_IDX, BLOCK, ITEMS, false, VIRT, DONLY>(a, vcount, voffsets, s_vlut, sh, tile,
+                                                                                       row, trow, static_cast<uint32_t>(remain));
     }
     return;
   }
-  if (remain >= static_cast<uint64_t>(TILE)) {
-    onesweep_tile<KeyT, CODEC, XFORM, BIG, HAS_IDX, BLOCK, ITEMS, true, false>(a, 0u, 0ull, nullptr, sh, tile, row, trow, TILE);
-  } else {
-    onesweep_tile<KeyT, CODEC, XFORM, BIG, HAS_IDX, BLOCK, ITEMS, false, false>(a, 0u, 0ull, nullptr, sh, tile, row, trow,
-                                                                                static_cast<uint32_t>(remain));
+  if constexpr (!DONLY) {  // (a DONLY launch has returned above unless the virtual plan is in force)
+    if (remain >= static_cast<uint64_t>(TILE)) {
+      onesweep_tile<KeyT, CODEC, XFORM, BIG, HAS_IDX, BLOCK, ITEMS, true, false>(a, 0u, 0ull, nullptr, sh, tile, row, trow, TILE);
+    } else {
+      onesweep_tile<KeyT, CODEC, XFORM, BIG, HAS_IDX, BLOCK, ITEMS, false, false>(a, 0u, 0ull, nullptr, sh, tile, row, trow,
+                                                                                  static_cast<uint32_t>(remain));
+    }
   }
 }
 

@@ -78,7 +78,7 @@ int merge_levels_limit(int key_bytes, bool want_indices)
   return key_bytes == 8 ? (want_indices ? 5 : 6) : 2;
 }
 
-// 1: rows of 2 ... 64 real keys go through the bitonic network; 0: through the ranking kernels
+// 1: rows of 2 ... 128 real keys go through the bitonic network; 0: through the ranking kernels
 static std::atomic<int> g_bitonic_rows{[] {
   const char* e = getenv("CPN_SORT_BITONIC_ROWS");
   return (e != nullptr && e[0] == '0') ? 0 : 1;
@@ -256,7 +256,18 @@ int cpn_local_sort(int dtype, const void* values_in, void* values_out, int64_t* 
                    uint64_t sort_dim_size, int64_t index_offset, int stable, void* temp, uint64_t temp_bytes,
                    void* stream)
 {
+  return cpn_local_sort_ex(dtype, values_in, values_out, indices_out, volume, sort_dim_size, index_offset, stable, 0u,
+                           temp, temp_bytes, stream);
+}
+
+int cpn_local_sort_ex(int dtype, const void* values_in, void* values_out, int64_t* indices_out, uint64_t volume,
+                      uint64_t sort_dim_size, int64_t index_offset, int stable, uint32_t options, void* temp,
+                      uint64_t temp_bytes, void* stream)
+{
   (void)stable;  // every path is stable
+  if ((options & ~static_cast<uint32_t>(CPN_SORT_SINGLE_TICKET)) != 0) {
+    return CPN_ERR_UNSUPPORTED;
+  }
   const cpn::KeyKind k = cpn::key_kind(dtype);
   if (k.bytes == 0) {
     return CPN_ERR_DTYPE;
@@ -288,6 +299,7 @@ int cpn_local_sort(int dtype, const void* values_in, void* values_out, int64_t* 
   r.temp         = temp;
   r.temp_bytes   = temp_bytes;
   r.stream       = static_cast<hipStream_t>(stream);
+  r.single_ticket = (options & CPN_SORT_SINGLE_TICKET) != 0;
   switch (k.bytes) {
     case 1: return cpn::sort_keys8(k.codec, r);
     case 2: return cpn::sort_keys16(k.codec, r);

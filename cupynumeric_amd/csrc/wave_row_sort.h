@@ -278,7 +278,7 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
         float top;
         __builtin_memcpy(&origin, &lo_bits, 4);
         __builtin_memcpy(&top, &hi_bits, 4);
-        scale = static_cast<float>(BINS) / (top - origin);  // (an infinite span gives 0: one crowded range)
+        scale = static_cast<float>(BINS) / (top - origin);  // (an infinite span gives 0: one crowded range, see bin_of)
       } else {
         const int bits = 32 - __builtin_clz((hi - lo) | 1u);
         shift          = bits > BINS_LOG2 ? bits - BINS_LOG2 : 0;
@@ -288,8 +288,11 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void wave_row_sort_kernel(con
           const uint32_t raw = sign_unflip(image);
           float v;
           __builtin_memcpy(&v, &raw, 4);
-          const uint32_t b = static_cast<uint32_t>((v - origin) * scale);
-          return b < static_cast<uint32_t>(BINS) ? b : static_cast<uint32_t>(BINS - 1);
+          // clamped as a float first: the product is NaN or infinite when the row holds an infinity or
+          // its span underflows (fmax returns its other operand for a NaN), and converting such a
+          // value to an integer is undefined
+          const float t = __builtin_fminf(__builtin_fmaxf((v - origin) * scale, 0.0f), static_cast<float>(BINS - 1));
+          return static_cast<uint32_t>(t);
         } else {
           return (image - lo) >> shift;
         }

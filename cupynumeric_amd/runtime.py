@@ -33,30 +33,48 @@ class Runtime:
         self.check_mode = {"0": "off", "off": "off", "1": "eager", "eager": "eager"}.get(mode, "lazy")
         self._torch = None
         self._status_slots = None
+        self._status_kinds: list[str] = []
         self._status_used = 0
 
     def defer_status(self, temp: "torch.Tensor") -> None:
         """Lazy mode: keep the status word of the sort that just used `temp` (stream-ordered copy)."""
+        self.defer_flag(temp[:4].view(self.torch.int32), "sort")
+
+    def defer_flag(self, word: "torch.Tensor", kind: str) -> None:
+        """Keep one 4-byte device word that a kernel raises on a condition the host has to report --
+        "sort": the status word of a global sort, "index": an index out of bounds -- until data next
+        reaches the host (`flush_status`).  The copy is ordered on the stream; nothing waits."""
         torch = self.torch
         if self._status_slots is None:
-            self._status_slots = torch.zeros(self.STATUS_SLOTS, dtype=torch.int32, device=temp.device)
+            self._status_slots = torch.zeros(self.STATUS_SLOTS, dtype=torch.int32, device=word.device)
+            self._status_kinds = []
         if self._status_used == self.STATUS_SLOTS:
             self.flush_status()
-        self._status_slots[self._status_used : self._status_used + 1].copy_(temp[:4].view(torch.int32))
+        self._status_slots[self._status_used : self._status_used + 1].copy_(word)
+        self._status_kinds.append(kind)
         self._status_used += 1
 
     def flush_status(self) -> None:
-        """Read back the deferred status words (synchronises); raises if a sort failed on the device."""
+        """Read back the deferred words (synchronises); raises if a sort failed on the device or an
+        index was out of bounds since the last host read."""
         used, self._status_used = self._status_used, 0
         if used == 0:
             return
+        kinds, self._status_kinds = self._status_kinds, []
         words = self._status_slots[:used].cpu()
-        if bool(words.any()):
+        if not bool(words.any()):
+            return
+        raised = {kinds[i] for i in range(used) if int(words[i]) != 0}
+        if "sort" in raised:
             raise RuntimeError(
                 "cpn_local_sort: a sort issued since the last host read failed on the device (a bounded wait "
                 "inside a kernel ran out, cpn_status -7); its result and everything computed from it are "
                 "invalid.  Repeat the work with CPN_SORT_TILE_ORDER=single or CUPYNUMERIC_AMD_CHECK_STATUS=eager"
             )
+        raise IndexError(
+            "index out of bounds in an indexed read (take / searchsorted sorter) issued since the last host read; "
+            "its result and everything computed from it are invalid"
+        )
 
     @property
     def torch(self):

@@ -70,93 +70,6 @@ const char* cpn_status_string(int status);
 /* hipError_t of the last HIP call that failed on the calling thread (0 if none). */
 int cpn_last_hip_error(void);
 
-/*
- * Process-wide tunable: rows of at most `limit` elements are sorted by the one-workgroup-
- * per-row LDS kernel, longer rows by the global radix sort.  Values above the kernel's
- * capacity are clamped to it, a negative value restores the default; the previous setting is
- * returned (-1 = default).  Also initialised from the environment variable
- * CPN_SORT_LDS_ROW_LIMIT.  Plays the role of the reference's compile-time
- * SEGMENT_THRESHOLD_RADIX_SORT (src/cupynumeric/sort/sort.cu:41).  Sizes returned by
- * cpn_local_sort_temp_bytes depend on it: do not change it between the size query and the sort.
- */
-int64_t cpn_set_lds_row_limit(int64_t limit);
-
-/*
- * Process-wide tunable: rows of at most `limit` elements (at most 1024) are sorted by one
- * wavefront each, longer rows that fit in LDS by one workgroup each.  A negative value
- * restores the default; the previous setting is returned.  Also initialised from the
- * environment variable CPN_SORT_WAVE_ROW_LIMIT.  Does not affect workspace sizes.
- */
-int64_t cpn_set_wave_row_limit(int64_t limit);
-
-/*
- * Process-wide switch: rows of 2 ... 64 real keys of up to 8 bytes are sorted by a bitonic network
- * between the lanes of a wavefront (enabled != 0, the default) or by the ranking kernels that take
- * the other key types of that length (0).  Returns the previous setting.  Also initialised from the
- * environment variable CPN_SORT_BITONIC_ROWS (0 switches it off).  Does not affect workspace sizes.
- * An A/B switch with no counterpart in the reference, which merge-sorts (segment id, value) tuples
- * for short rows (src/cupynumeric/sort/thrust_sort.cuh:68-122).
- */
-int cpn_set_bitonic_rows(int enabled);
-
-/*
- * Process-wide switch: rows longer than the per-row kernels take (real keys of 4 and 8 bytes) are cut
- * into 2, 4, ... pieces that the per-row kernel sorts and that are then merged pairwise, level by
- * level, as long as that is cheaper than the global path's one pass per key byte (mode 1, the default:
- * up to 6 levels for 8-byte keys, 5 with positions, i.e. rows of up to 1 048 576 and 458 752 keys;
- * 2 levels for 4-byte keys, rows of up to 65 536), or all go down the global path (mode 0).  A mode N >= 2 allows up to N - 1 levels for every key (A/B runs); a
- * negative mode restores the default.  Returns the previous mode.  Also initialised from the
- * environment variable CPN_SORT_MERGE_ROWS.  Changes the sizes returned by
- * cpn_local_sort_temp_bytes: do not change it between the size query and the sort.
- * An A/B switch with no counterpart in the reference, whose segmented radix sort takes every row
- * length (src/cupynumeric/sort/cub_sort.cuh:81-105).
- */
-int cpn_set_merge_rows(int mode);
-
-/*
- * Process-wide tunable: rows of at least `elements` elements on the global path keep their
- * per-row counts, tile descriptors and row positions in 64 bits.  The default and the maximum
- * is 2^30 (shorter rows use 32 bits); a negative value restores the default and the previous
- * setting is returned (-1 = default).  Lower values exist so that tests can run the 64-bit
- * kernels on small inputs; they change workspace sizes (cpn_local_sort_temp_bytes follows).
- * Also initialised from the environment variable CPN_SORT_WIDE_ROW_THRESHOLD.
- */
-int64_t cpn_set_wide_row_threshold(int64_t elements);
-
-/*
- * Process-wide tunable: how many times a tile of the global path polls the descriptor of a
- * predecessor before it gives up, sets the device status word (CPN_ERR_DEVICE from
- * cpn_local_sort_check) and lets every kernel run to its end with invalid output.  The default
- * (2^22 polls, restored by a value below 1) is far above any real wait; tests of the failure
- * path set 1.  The previous setting is returned.
- */
-int64_t cpn_set_lookback_spin_limit(int64_t polls);
-
-/*
- * Process-wide tunable: how the scatter passes of the global sort hand their tiles to workgroups.
- * 0 (default): per XCD, so that neighbouring tiles share an L2 (faster; assumes that every XCD of
- * the device keeps receiving workgroups of the launch: if foreign work held one XCD for seconds,
- * the bounded look-back would give up with CPN_ERR_DEVICE).  Non-zero: one ticket counter for the
- * whole launch, which has no such dependence; a caller that met CPN_ERR_DEVICE repeats the sort
- * this way.  Results do not depend on it.  Returns the previous setting.  Also initialised from the
- * environment variable CPN_SORT_TILE_ORDER ("single" selects the one counter).  The reference has no
- * counterpart (cub's onesweep takes tiles from one counter, behind src/cupynumeric/sort/cub_sort.cuh:120-143).
- */
-int cpn_set_tile_order(int single);
-
-/*
- * Process-wide tunable: a 1-D sort of real 8-byte keys with at least `elements` elements lets
- * the device replace its eight byte passes by one pass on the ranks of the keys when the row
- * holds at most 256 different keys, or by fewer passes on "virtual digits" when the
- * histograms show that the bytes of the keys take few distinct values (several bytes then
- * share one 8-bit digit; cupynumeric_amd/csrc/virtual_digits.h).  Results do not depend on
- * it.  The default is 2^26 (below that the extra launches outweigh the average gain); a
- * negative value restores it and the previous setting is returned.  It changes workspace
- * sizes by 24 KiB (cpn_local_sort_temp_bytes follows).  Also initialised from the
- * environment variable CPN_SORT_VIRTUAL_DIGIT_THRESHOLD.
- */
-int64_t cpn_set_virtual_digit_threshold(int64_t elements);
-
 /* Size in bytes of one element of `dtype`, or 0 for an unknown code. */
 uint64_t cpn_dtype_size(int dtype);
 
@@ -207,6 +120,23 @@ int cpn_local_sort(int dtype, const void* values_in, void* values_out, int64_t* 
                    void* temp, uint64_t temp_bytes, void* stream);
 
 /*
+ * cpn_local_sort with per-call options (a bit set of CPN_SORT_*; 0 = cpn_local_sort; unknown bits
+ * return CPN_ERR_UNSUPPORTED).  Same call site as cpn_local_sort (src/cupynumeric/sort/sort.cu:63-96);
+ * the options have no counterpart in the reference.
+ *
+ *   CPN_SORT_SINGLE_TICKET  the scatter passes of this call hand their tiles to workgroups through
+ *                           one counter for the whole launch instead of one per XCD.  Slower by a few
+ *                           per cent, and independent of every XCD of the device taking part in the
+ *                           launch: the way to repeat a sort that came back with CPN_ERR_DEVICE
+ *                           (cpn_local_sort_check), without touching process-wide state.  Results do
+ *                           not depend on it.
+ */
+#define CPN_SORT_SINGLE_TICKET 1u
+int cpn_local_sort_ex(int dtype, const void* values_in, void* values_out, int64_t* indices_out,
+                      uint64_t volume, uint64_t sort_dim_size, int64_t index_offset, int stable,
+                      uint32_t options, void* temp, uint64_t temp_bytes, void* stream);
+
+/*
  * cpn_local_sort for callers that cannot allocate device memory or pass a workspace: code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
  * counterpart in the reference, whose sort always draws its temporaries from a Legate pool
@@ -225,8 +155,10 @@ int cpn_local_sort(int dtype, const void* values_in, void* values_out, int64_t* 
  *     and the output is invalid (what cpn_local_sort_check reports for cpn_local_sort);
  *   - every call on one GPU uses that GPU's one array, whatever its stream: calls that overlap in
  *     time on one GPU race.  Order them on one stream, or with events;
- *   - the first call on a device looks up the array's address on that device
- *     (hipGetSymbolAddress); make that call outside graph capture.
+ *   - the first call on a device is the set-up: it looks up the array's address on that device
+ *     (hipGetSymbolAddress), and the HIP runtime brings the array into device memory with the
+ *     library's code then; make that call outside graph capture and before the part of the
+ *     program that must not allocate.
  */
 #define CPN_STATIC_SCRATCH_BYTES (64ull << 20)
 int cpn_local_sort_static(int dtype, const void* values_in, void* values_out, int64_t* indices_out,
@@ -365,6 +297,19 @@ int cpn_take_along_last_axis(int elem_bytes, const void* src, const int64_t* ind
                              void* stream);
 
 /*
+ * cpn_take_along_last_axis when the leading dimensions of `src` and `indices` broadcast against each
+ * other (every dimension but the axis may be 1 on either side, cupynumeric/_module/indexing.py:700-760,
+ * where the reference falls back to a gather over coordinate arrays).  The output has lead_ndim (0..7)
+ * leading dimensions out_lead_shape[] and rows of idx_seg elements; src_lead_strides[d] and
+ * idx_lead_strides[d] say how many rows of `src` / `indices` one step in leading dimension d is worth:
+ * the dense stride of that side, or 0 where its extent is 1.  Everything else as above.
+ */
+int cpn_take_along_last_axis_broadcast(int elem_bytes, const void* src, const int64_t* indices, void* out,
+                                       int lead_ndim, const uint64_t* out_lead_shape,
+                                       const uint64_t* src_lead_strides, const uint64_t* idx_lead_strides,
+                                       uint64_t src_seg, uint64_t idx_seg, uint32_t* oob_flag, void* stream);
+
+/*
  * Packs num_keys (1..8) real keys of `rows` dense rows of `seg` elements into one unsigned
  * word per element (packed_bytes = 4 or 8, at least the summed width of the keys):
  * keys[0] is the least significant key, as in lexsort; each key enters as the
@@ -377,6 +322,106 @@ int cpn_take_along_last_axis(int elem_bytes, const void* src, const int64_t* ind
  */
 int cpn_lexsort_pack(int num_keys, const int* dtypes, const void* const* keys, const int64_t* indices,
                      int packed_bytes, void* packed_out, uint64_t rows, uint64_t seg, void* stream);
+
+/* =============================================================================================
+ * Test, A/B and benchmark hooks.  A binding of the reference's call site needs nothing below this
+ * line: the entry points above are the product.  The cpn_set_* functions change process-wide
+ * state; they exist so that tests can reach kernels that small inputs would not (64-bit row
+ * positions, virtual digits, the bounded wait that gives up) and so that benchmarks can compare
+ * one kernel with another on the same input.  Call them at start-up or from one thread while no
+ * other thread sorts; never from code that serves requests.  Two of them (cpn_set_lds_row_limit,
+ * cpn_set_merge_rows) and the two thresholds change what cpn_local_sort_temp_bytes returns:
+ * cpn_local_sort works the size out again from the settings in force when it is called and
+ * returns CPN_ERR_TEMP, before it launches anything, when the workspace it was given is smaller
+ * than that.  Per-call choices go through cpn_local_sort_ex instead.
+ * ============================================================================================= */
+
+/*
+ * Process-wide tunable: rows of at most `limit` elements are sorted by the one-workgroup-
+ * per-row LDS kernel, longer rows by the global radix sort.  Values above the kernel's
+ * capacity are clamped to it, a negative value restores the default; the previous setting is
+ * returned (-1 = default).  Also initialised from the environment variable
+ * CPN_SORT_LDS_ROW_LIMIT.  Plays the role of the reference's compile-time
+ * SEGMENT_THRESHOLD_RADIX_SORT (src/cupynumeric/sort/sort.cu:41).  Sizes returned by
+ * cpn_local_sort_temp_bytes depend on it: do not change it between the size query and the sort.
+ */
+int64_t cpn_set_lds_row_limit(int64_t limit);
+
+/*
+ * Process-wide tunable: rows of at most `limit` elements (at most 1024) are sorted by one
+ * wavefront each, longer rows that fit in LDS by one workgroup each.  A negative value
+ * restores the default; the previous setting is returned.  Also initialised from the
+ * environment variable CPN_SORT_WAVE_ROW_LIMIT.  Does not affect workspace sizes.
+ */
+int64_t cpn_set_wave_row_limit(int64_t limit);
+
+/*
+ * Process-wide switch: rows of 2 ... 128 real keys of up to 8 bytes are sorted by a bitonic network
+ * between the lanes of a wavefront, one key per lane, two per lane above 64 keys (enabled != 0, the default) or by the ranking kernels that take
+ * the other key types of that length (0).  Returns the previous setting.  Also initialised from the
+ * environment variable CPN_SORT_BITONIC_ROWS (0 switches it off).  Does not affect workspace sizes.
+ * An A/B switch with no counterpart in the reference, which merge-sorts (segment id, value) tuples
+ * for short rows (src/cupynumeric/sort/thrust_sort.cuh:68-122).
+ */
+int cpn_set_bitonic_rows(int enabled);
+
+/*
+ * Process-wide switch: rows longer than the per-row kernels take (real keys of 4 and 8 bytes) are cut
+ * into 2, 4, ... pieces that the per-row kernel sorts and that are then merged pairwise, level by
+ * level, as long as that is cheaper than the global path's one pass per key byte (mode 1, the default:
+ * up to 6 levels for 8-byte keys, 5 with positions, i.e. rows of up to 1 048 576 and 458 752 keys;
+ * 2 levels for 4-byte keys, rows of up to 65 536), or all go down the global path (mode 0).  A mode N >= 2 allows up to N - 1 levels for every key (A/B runs); a
+ * negative mode restores the default.  Returns the previous mode.  Also initialised from the
+ * environment variable CPN_SORT_MERGE_ROWS.  Changes the sizes returned by
+ * cpn_local_sort_temp_bytes: do not change it between the size query and the sort.
+ * An A/B switch with no counterpart in the reference, whose segmented radix sort takes every row
+ * length (src/cupynumeric/sort/cub_sort.cuh:81-105).
+ */
+int cpn_set_merge_rows(int mode);
+
+/*
+ * Process-wide tunable: rows of at least `elements` elements on the global path keep their
+ * per-row counts, tile descriptors and row positions in 64 bits.  The default and the maximum
+ * is 2^30 (shorter rows use 32 bits); a negative value restores the default and the previous
+ * setting is returned (-1 = default).  Lower values exist so that tests can run the 64-bit
+ * kernels on small inputs; they change workspace sizes (cpn_local_sort_temp_bytes follows).
+ * Also initialised from the environment variable CPN_SORT_WIDE_ROW_THRESHOLD.
+ */
+int64_t cpn_set_wide_row_threshold(int64_t elements);
+
+/*
+ * Process-wide tunable: how many times a tile of the global path polls the descriptor of a
+ * predecessor before it gives up, sets the device status word (CPN_ERR_DEVICE from
+ * cpn_local_sort_check) and lets every kernel run to its end with invalid output.  The default
+ * (2^22 polls, restored by a value below 1) is far above any real wait; tests of the failure
+ * path set 1.  The previous setting is returned.
+ */
+int64_t cpn_set_lookback_spin_limit(int64_t polls);
+
+/*
+ * Process-wide tunable: how the scatter passes of the global sort hand their tiles to workgroups.
+ * 0 (default): per XCD, so that neighbouring tiles share an L2 (faster; assumes that every XCD of
+ * the device keeps receiving workgroups of the launch: if foreign work held one XCD for seconds,
+ * the bounded look-back would give up with CPN_ERR_DEVICE).  Non-zero: one ticket counter for the
+ * whole launch, which has no such dependence (one call at a time: CPN_SORT_SINGLE_TICKET of
+ * cpn_local_sort_ex).  Results do not depend on it.  Returns the previous setting.  Also initialised from the
+ * environment variable CPN_SORT_TILE_ORDER ("single" selects the one counter).  The reference has no
+ * counterpart (cub's onesweep takes tiles from one counter, behind src/cupynumeric/sort/cub_sort.cuh:120-143).
+ */
+int cpn_set_tile_order(int single);
+
+/*
+ * Process-wide tunable: a 1-D sort of real 8-byte keys with at least `elements` elements lets
+ * the device replace its eight byte passes by one pass on the ranks of the keys when the row
+ * holds at most 256 different keys, or by fewer passes on "virtual digits" when the
+ * histograms show that the bytes of the keys take few distinct values (several bytes then
+ * share one 8-bit digit; cupynumeric_amd/csrc/virtual_digits.h).  Results do not depend on
+ * it.  The default is 2^26 (below that the extra launches outweigh the average gain); a
+ * negative value restores it and the previous setting is returned.  It changes workspace
+ * sizes by 24 KiB (cpn_local_sort_temp_bytes follows).  Also initialised from the
+ * environment variable CPN_SORT_VIRTUAL_DIGIT_THRESHOLD.
+ */
+int64_t cpn_set_virtual_digit_threshold(int64_t elements);
 
 /*
  * Per-launch timing.  cpn_profile_enable(1) makes every kernel launch of the library record

@@ -289,3 +289,77 @@ def test_built_row_kernels_do_not_spill():
                     seen_row_kernels += pattern != "onesweep_kernel"
                     assert use.get("scratch_bytes_per_lane", 0) <= limit, (report.name, kernel, use)
     assert seen_row_kernels > 100  # the row kernels of five key widths were all looked at
+
+
+def test_setter_between_size_query_and_sort_is_refused(lib):
+    """A test hook that enlarges the workspace a request needs, called between the size query and the
+    sort: the sort works the size out again and returns CPN_ERR_TEMP before it launches anything (the
+    pointers below are not device memory)."""
+    code = _lib.DTYPE_CODES[np.dtype(np.float32)]
+    volume, seg = 1 << 20, 1 << 10  # rows the per-row kernel takes: the header only
+    small = lib.cpn_local_sort_temp_bytes(code, volume, seg, 1, 0, 0)
+    prev = lib.cpn_set_lds_row_limit(0)  # every row down the global path: histograms, descriptors, key buffers
+    try:
+        assert lib.cpn_local_sort_temp_bytes(code, volume, seg, 1, 0, 0) > small
+        assert lib.cpn_local_sort(code, 4096, 8192, None, volume, seg, 0, 1, 256, small, None) == _lib.CPN_ERR_TEMP
+        assert lib.cpn_local_sort_ex(code, 4096, 8192, None, volume, seg, 0, 1, 0, 256, small, None) == _lib.CPN_ERR_TEMP
+    finally:
+        lib.cpn_set_lds_row_limit(prev)
+    # the same for the switch of the merged rows: a row just past the per-row kernels
+    seg = 20_000
+    merged = lib.cpn_local_sort_temp_bytes(code, seg, seg, 1, 0, 0)
+    prev = lib.cpn_set_merge_rows(0)
+    try:
+        need = lib.cpn_local_sort_temp_bytes(code, seg, seg, 1, 0, 0)
+        if need > merged:
+            assert lib.cpn_local_sort(code, 4096, 1 << 20, None, seg, seg, 0, 1, 256, merged, None) == _lib.CPN_ERR_TEMP
+    finally:
+        lib.cpn_set_merge_rows(prev)
+    # unknown option bits of cpn_local_sort_ex are refused before anything else happens
+    assert lib.cpn_local_sort_ex(code, 4096, 8192, None, 16, 16, 0, 1, 0x80, 256, 4096, None) == _lib.CPN_ERR_UNSUPPORTED
+
+
+def test_merged_row_levels_and_workspace_over_the_limits(lib):
+    """Rows longer than the per-row kernels take: the number of pieces doubles at every multiple of the
+    per-row capacity up to the limit of levels, after which the global path takes over; the workspace
+    follows (one copy of the rows for one level, two from two levels on, plus the table of chunk starts)."""
+    f64, f32 = _lib.DTYPE_CODES[np.dtype(np.float64)], _lib.DTYPE_CODES[np.dtype(np.float32)]
+
+    def temp(code, seg, idx):
+        return lib.cpn_local_sort_temp_bytes(code, seg, seg, int(not idx), int(idx), 0)
+
+    # float64, values only: capacity 16384 keys, up to 6 levels -> rows of up to 1 048 576 keys
+    cap, prev_bytes = 16384, 0
+    for level in range(1, 7):
+        seg = cap << level
+        b = temp(f64, seg, False)
+        copies = 1 if level == 1 else 2
+        assert copies * seg * 8 <= b < copies * seg * 8 + (1 << 20), (level, b)
+        assert b > prev_bytes
+        prev_bytes = b
+    # one key past the limit: the global path (one key buffer beside the caller's output, histograms, descriptors)
+    over = (cap << 6) + 1
+    assert over * 8 < temp(f64, over, False) < over * 12
+    # with positions: capacity 14336, 5 levels -> 458 752 keys in two copies of (key, int64 position);
+    # one key more: the global path with the keys twice and 4-byte positions
+    seg = 14336 << 5
+    assert 2 * seg * 16 <= temp(f64, seg, True) < 2 * seg * 16 + (1 << 20)
+    assert (seg + 1) * 20 < temp(f64, seg + 1, True) < (seg + 1) * 24
+    # 4-byte keys: 2 levels -> 65 536 keys in two copies; one key more: the global path
+    assert 2 * 65536 * 4 <= temp(f32, 65536, False) < 2 * 65536 * 4 + (1 << 16)
+    assert 65537 * 4 < temp(f32, 65537, False) < 2 * 65536 * 4
+
+
+def test_no_allocation_calls_in_the_native_sources():
+    """cpn_local_sort_static promises that nothing on its path allocates: no translation unit of the
+    library calls hipMalloc, hipFree or creates events outside the profiling helper, which is off
+    unless a benchmark switches it on."""
+    csrc = ROOT / "cupynumeric_amd" / "csrc"
+    pattern = re.compile(r"\bhip(Malloc\w*|Free\w*|HostMalloc|EventCreate\w*|StreamCreate\w*|MemPool\w*)\s*\(")
+    for path in sorted(csrc.glob("*.h")) + sorted(csrc.glob("*.hip")):
+        text = re.sub(r"//[^\n]*", "", path.read_text())
+        hits = sorted({m.group(0) for m in pattern.finditer(text)})
+        if path.name == "profile.hip":
+            assert all(h.startswith("hipEventCreate") for h in hits), hits  # events, only while profiling is on
+        else:
+            assert hits == [], f"{path.name} calls {hits}"

@@ -720,6 +720,38 @@ def test_rows_sorted_as_merged_halves(lib, torch_cuda, dtype):
     assert lib.cpn_local_sort_temp_bytes(code, rows * seg, seg, 1, 0, 0) == merged_bytes
 
 
+@pytest.mark.parametrize("dtype", [np.float64, np.int64])
+def test_rows_merged_over_five_and_six_levels(lib, torch_cuda, dtype):
+    """8-byte keys: 32 pieces (five levels of merging; with positions the most there is) and 64 pieces (six
+    levels, values only), and rows one key past each limit, which take the global path and must give the
+    same bits."""
+    dt = np.dtype(dtype)
+    code = _lib.DTYPE_CODES[dt]
+    x = make_input(dtype, (2, 300_001), seed=41)  # 32 pieces, values and positions
+    x[1, ::3] = x[1, 0]                            # ties across every piece
+    check_rows(lib, torch_cuda, x, f"{dt} 2 x 300001, five levels")
+    v, i = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=True, offset=3)
+    assert_same_bits(v, oracle.local_sort(x, argsort=False), f"{dt} five levels, values+positions")
+    assert_same_bits(i, oracle.local_sort(x, argsort=True) + 3, f"{dt} five levels, positions")
+    y = make_input(dtype, (1, 600_001), seed=42)  # 64 pieces, values only
+    v, _ = abi_sort(lib, torch_cuda, y, want_values=True, want_indices=False)
+    assert_same_bits(v, oracle.local_sort(y, argsort=False), f"{dt} 1 x 600001, six levels")
+    v, _ = abi_sort(lib, torch_cuda, y, want_values=True, want_indices=False, in_place=True)
+    assert_same_bits(v, oracle.local_sort(y, argsort=False), f"{dt} six levels, in place")
+    # the limits themselves and one key past them (the global path)
+    for seg, idx in [(1_048_576, False), (1_048_577, False), (458_752, True), (458_753, True)]:
+        z = make_input(dtype, (1, seg), seed=seg)
+        per_key = lib.cpn_local_sort_temp_bytes(code, seg, seg, int(not idx), int(idx), 0) / seg
+        # merged rows hold two copies of the keys (and of int64 positions); the global path one key buffer
+        # beside the caller's output, or the keys twice and 4-byte positions
+        assert per_key >= (32 if idx else 16) if seg in (1_048_576, 458_752) else per_key < (24 if idx else 12)
+        v, i = abi_sort(lib, torch_cuda, z, want_values=not idx, want_indices=idx)
+        if idx:
+            assert_same_bits(i, oracle.local_sort(z, argsort=True), f"{dt} seg={seg} argsort")
+        else:
+            assert_same_bits(v, oracle.local_sort(z, argsort=False), f"{dt} seg={seg} sort")
+
+
 def test_merged_rows_many_rows_and_narrow_keys_stay_out(lib, torch_cuda):
     # many rows: every workgroup of the merge finds its own part of its own row
     x = make_input(np.float32, (300, 17000), seed=3)
@@ -1056,6 +1088,29 @@ def test_single_ticket_tile_order(lib, torch_cuda, global_path):
         assert lib.cpn_set_tile_order(prev) == 1
 
 
+def test_single_ticket_per_call(lib, torch_cuda, global_path):
+    """cpn_local_sort_ex with CPN_SORT_SINGLE_TICKET: the same bits as the default order, the process-wide
+    setting untouched; unknown option bits are refused."""
+    for dtype, shape, argsort in [(np.float32, (300_001,), True), (np.int64, (70_000,), False), (np.uint16, (5, 40_000), True)]:
+        x = make_input(dtype, shape, seed=6)
+        code, seg = _lib.DTYPE_CODES[x.dtype], x.shape[-1]
+        d_in = torch_cuda.from_numpy(x.reshape(-1).view(np.uint8).copy()).cuda()
+        d_val = torch_cuda.zeros_like(d_in)
+        d_idx = torch_cuda.zeros(x.size, dtype=torch_cuda.int64, device="cuda")
+        tb = lib.cpn_local_sort_temp_bytes(code, x.size, seg, 1, int(argsort), 0)
+        temp = torch_cuda.full((tb,), 0xFF, dtype=torch_cuda.uint8, device="cuda")
+        stream = ctypes.c_void_p(torch_cuda.cuda.current_stream().cuda_stream)
+        rc = lib.cpn_local_sort_ex(code, d_in.data_ptr(), d_val.data_ptr(), d_idx.data_ptr() if argsort else None, x.size, seg,
+                                   0, 1, _lib.CPN_SORT_SINGLE_TICKET, temp.data_ptr(), tb, stream)
+        assert rc == 0 and lib.cpn_local_sort_check(temp.data_ptr(), stream) == 0
+        assert_same_bits(d_val.cpu().numpy().view(x.dtype).reshape(x.shape), oracle.local_sort(x, argsort=False), f"{shape}")
+        if argsort:
+            assert np.array_equal(d_idx.cpu().numpy().reshape(x.shape), oracle.local_sort(x, argsort=True))
+        assert lib.cpn_local_sort_ex(code, d_in.data_ptr(), d_val.data_ptr(), None, x.size, seg, 0, 1, 2, temp.data_ptr(), tb,
+                                     stream) == _lib.CPN_ERR_UNSUPPORTED
+    assert lib.cpn_set_tile_order(0) == 0
+
+
 def test_python_layer_status_modes(lib, torch_cuda, monkeypatch):
     """The Python layer's handling of the device status word: lazy (default: read when data next
     reaches the host), eager with one repeat in single-ticket order, off.  The failure is forced from
@@ -1092,23 +1147,28 @@ def test_python_layer_status_modes(lib, torch_cuda, monkeypatch):
     assert np.array_equal(np.asarray(num.argsort(a)), want)
     # eager: a reported failure is answered by one repeat with the single tile counter
     monkeypatch.setattr(runtime, "check_mode", "eager")
-    real_check = lib.cpn_local_sort_check
-    calls = {"n": 0, "order_at_repeat": None}
+    real_check, real_sort = lib.cpn_local_sort_check, lib.cpn_local_sort_ex
+    calls = {"n": 0, "options": [], "order_at_repeat": None}
 
     def failing_once(temp, stream):
         calls["n"] += 1
         if calls["n"] == 1:
             real_check(temp, stream)
             return _lib.CPN_ERR_DEVICE
-        calls["order_at_repeat"] = lib.cpn_set_tile_order(1)  # returns the order in force
-        lib.cpn_set_tile_order(calls["order_at_repeat"])
+        calls["order_at_repeat"] = lib.cpn_set_tile_order(0)  # returns the order in force
         return real_check(temp, stream)
 
+    def recording_sort(*args):
+        calls["options"].append(args[8])
+        return real_sort(*args)
+
     monkeypatch.setattr(lib, "cpn_local_sort_check", failing_once)
+    monkeypatch.setattr(lib, "cpn_local_sort_ex", recording_sort)
     got = num.argsort(a)
     monkeypatch.setattr(lib, "cpn_local_sort_check", real_check)
-    assert calls == {"n": 2, "order_at_repeat": 1}
-    assert lib.cpn_set_tile_order(0) == 0, "the tile order was not restored"
+    monkeypatch.setattr(lib, "cpn_local_sort_ex", real_sort)
+    # the repeat asks for the single counter per call; the process-wide order is never touched
+    assert calls == {"n": 2, "options": [0, _lib.CPN_SORT_SINGLE_TICKET], "order_at_repeat": 0}
     assert np.array_equal(np.asarray(got), want)
     # an in-place sort cannot be repeated (its input is gone): the failure is raised
     calls["n"] = 0

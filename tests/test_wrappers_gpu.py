@@ -201,6 +201,81 @@ def test_take_along_axis_public():
         num.take_along_axis(x, np.zeros((4, 5), dtype=int), 2)
 
 
+def test_take_along_axis_broadcasts_like_numpy():
+    """Every dimension but the axis may be 1 on either side (`cupynumeric/_module/indexing.py:700-760`,
+    where the reference gathers through coordinate arrays): against numpy.take_along_axis."""
+    rng = np.random.default_rng(12)
+    cases = [((4, 7), (1, 3), 1), ((1, 7), (5, 3), 1), ((4, 7), (2, 1), 0), ((4, 1), (3, 6), 0),
+             ((3, 1, 5), (1, 4, 2), 2), ((3, 4, 5), (3, 1, 5), 1), ((1, 4, 1, 6), (2, 3, 5, 1), 1),
+             ((2, 1, 3, 1, 2), (1, 3, 2, 4, 1), 2), ((6,), (9,), 0), ((3, 5), (3, 0), 1), ((1, 5), (0, 2), 1)]
+    for a_shape, i_shape, axis in cases:
+        for dtype in (np.float32, np.int16, np.complex128):
+            x = (rng.standard_normal(a_shape) * 100).astype(dtype)
+            k = rng.integers(-a_shape[axis], a_shape[axis], i_shape)
+            want = np.take_along_axis(x, k, axis)
+            got = np.asarray(num.take_along_axis(num.array(x), num.array(k), axis))
+            assert got.shape == want.shape and np.array_equal(got, want), (a_shape, i_shape, axis, dtype)
+    # shapes that do not broadcast: IndexError, as in NumPy (`tests/integration/test_take_along_axis.py:378-384`)
+    with pytest.raises(IndexError, match="shape mismatch: indexing arrays could not be broadcast"):
+        num.take_along_axis(num.array(np.ones((3, 3))), num.array(np.ones((3, 2), dtype=int)), 0)
+    # out of bounds in the broadcast form is reported from the call too
+    with pytest.raises(IndexError, match="out of bounds"):
+        num.take_along_axis(num.array(np.ones((3, 3))), num.array(np.full((1, 3), 3)), 0)
+
+
+def test_getitem_with_an_integer_array():
+    """`arr.flatten()[argsort result]`, as `tests/integration/test_argsort.py:229-245` writes it, over that
+    file's shapes; NumPy indices, lists and negative positions; an index out of range surfaces as
+    IndexError with the next host read."""
+    rng = np.random.default_rng(13)
+    dim = 5
+    sizes = [(0,), (1,), (dim,), (0, 1), (1, 0), (1, 1), (1, dim), (dim, 1), (dim, dim), (1, 0, 0), (1, 1, 0), (1, 0, 1),
+             (1, 1, 1), (dim, 1, 1), (1, dim, 1), (1, 1, dim), (dim, dim, dim)]
+    for size in sizes:
+        arr_np = rng.integers(-100, 100, size)
+        arr_num = num.array(arr_np)
+        res_np = np.argsort(arr_np, axis=None)
+        res_num = num.argsort(arr_num, axis=None)
+        assert res_num.shape == (int(np.prod(size)),)
+        sorted_np = arr_np.flatten()[res_np]
+        sorted_num = arr_num.flatten()[res_num]
+        assert np.array_equal(np.asarray(sorted_num), sorted_np), size
+    x = rng.standard_normal(1000).astype(np.float32)
+    a = num.array(x)
+    k = rng.integers(-1000, 1000, 300)
+    assert np.array_equal(np.asarray(a[k]), x[k])
+    assert np.array_equal(np.asarray(a[k.astype(np.int32)]), x[k])
+    assert np.array_equal(np.asarray(a[[5, -1, 0]]), x[[5, -1, 0]])
+    assert np.asarray(a[[]]).shape == (0,)
+    with pytest.raises(NotImplementedError):
+        a[3]
+    with pytest.raises(NotImplementedError):
+        num.array(np.ones((2, 2)))[np.array([0])]
+    bad = a[np.array([0, 1000])]  # issued without a host read ...
+    with pytest.raises(IndexError, match="out of bounds"):
+        np.asarray(bad)  # ... and reported with the first one
+    assert np.array_equal(np.asarray(a[k]), x[k])  # the layer has recovered
+
+
+def test_searchsorted_sorter_does_not_synchronise(monkeypatch):
+    """The out-of-bounds flag of the gather behind `sorter` travels with the deferred status words: no
+    host read happens inside the call."""
+    from cupynumeric_amd.runtime import runtime
+
+    rng = np.random.default_rng(14)
+    x = rng.standard_normal(5000).astype(np.float32)
+    order = np.argsort(x, kind="stable")
+    v = rng.standard_normal(100).astype(np.float32)
+    a, s = num.array(x), num.array(order)
+    np.asarray(a), np.asarray(s)
+    monkeypatch.setattr(runtime, "check_mode", "lazy")
+    before = runtime._status_used
+    got = num.searchsorted(a, v, sorter=s)
+    assert runtime._status_used == before + 1 and runtime._status_kinds[-1] == "index"
+    assert np.array_equal(np.asarray(got), np.searchsorted(x, v, sorter=order))
+    assert runtime._status_used == 0
+
+
 def test_astype_float16_rounds_once():
     """Casts to float16 from wider types must round to nearest even once, as NumPy does: values on and
     around the midpoints between neighbouring float16 numbers, where rounding to float32 first and to

@@ -55,13 +55,16 @@ def run_both(lib, torch, x: np.ndarray, want_values: bool, want_indices: bool, i
     b_in, b_val, b_idx = buffers()
     status = torch.full((1,), 77, dtype=torch.int32, device=dev)
     torch.cuda.synchronize()
+    assert lib.cpn_profile_enable(0) == 0, "launch timing (which creates events) must be off"
     before = torch.cuda.memory_stats()["allocation.all.allocated"]
+    free_before = torch.cuda.mem_get_info()[0]  # the device's own count: sees allocations torch does not make
     rc = lib.cpn_local_sort_static(code, b_in.data_ptr(), b_val.data_ptr() if want_values else None,
                                    b_idx.data_ptr() if want_indices else None, volume, seg, offset, 1,
                                    status.data_ptr(), stream)
     assert rc == 0, _lib.status_string(rc)
     torch.cuda.synchronize()
     assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
+    assert torch.cuda.mem_get_info()[0] == free_before, "device memory was allocated or freed during the call"
     assert int(status.item()) == 0
     if want_values:
         assert torch.equal(a_val, b_val), "values differ"
@@ -69,6 +72,22 @@ def run_both(lib, torch, x: np.ndarray, want_values: bool, want_indices: bool, i
         assert torch.equal(a_idx, b_idx), "indices differ"
     if not in_place:
         assert np.array_equal(b_in.cpu().numpy(), raw), "input was modified"
+
+
+@pytest.fixture(scope="module", autouse=True)
+def static_scratch_set_up(lib, torch_cuda):
+    """The first call on a device is the set-up: it looks up the address of the static array, and the HIP
+    runtime loads the array with the library's code object then.  Every later call must leave the
+    device's free memory as it found it (run_both checks that)."""
+    torch = torch_cuda
+    x = torch.arange(64, dtype=torch.int32, device="cuda").flip(0).contiguous()
+    out = torch.empty_like(x)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rc = lib.cpn_local_sort_static(_lib.DTYPE_CODES[np.dtype(np.int32)], x.data_ptr(), out.data_ptr(), None, 64, 64, 0, 1,
+                                   None, stream)
+    assert rc == 0, _lib.status_string(rc)
+    torch.cuda.synchronize()
+    assert bool((out == torch.arange(64, dtype=torch.int32, device="cuda")).all())
 
 
 def test_static_scratch_matches_workspace_sort(lib, torch_cuda):
