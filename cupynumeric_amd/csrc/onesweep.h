@@ -235,6 +235,11 @@ constexpr uint32_t PLAN_FREE_RANK = 2u;
 struct SortPlan {
   PassPlan pass[MAX_PASSES];
   uint32_t n_active;
+  // Keys-only sorts of float keys without a NaN or a -0.0 (the histogram sweep has looked): the order-
+  // preserving image is then a bijection of the bits, so the first running pass stores the images,
+  // every pass takes plain bytes of them as digits, and the last pass maps them back as it stores
+  // (saves the key transform twice per key and pass; see onesweep_tile, UNFLIP).
+  uint32_t flipped;
 };
 
 struct PlanRequest {
@@ -262,6 +267,10 @@ __device__ __forceinline__ void make_plan(const uint32_t* varying, SortPlan* __r
     }
   }
   plan->n_active = k;
+  plan->flipped  = (rq.free_rank != 0 && rq.specials != nullptr && rq.want_indices == 0 &&
+                   __hip_atomic_load(rq.specials, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
+                     ? 1u
+                     : 0u;
   // scratch partner of T1: the caller's value array when it is free to be overwritten early
   const uint32_t key_x = (rq.want_values && !rq.in_place) ? KEY_OUT : KEY_T2;
   uint32_t j = 0, key_prev = KEY_IN, idx_prev = BUF_NONE;
@@ -545,8 +554,12 @@ struct SweepShared {
 // DONLY (with VIRT and HAS_IDX): the pass stores no keys (the one pass of an index-only sort on the
 // ranks of the row's different keys); the keys are turned into digits as they arrive and only
 // the digits, one byte each, go through LDS.
+//
+// UNFLIP (with XFORM, keys-only sorts of float keys that hold no NaN and no -0.0, SortPlan::flipped):
+// the images that the first pass stored are mapped back to the keys' bits by the last pass as it
+// stores them.
 template <typename KeyT, int CODEC, bool XFORM, bool BIG, bool HAS_IDX, int BLOCK, int ITEMS, bool FULL, bool VIRT,
-          bool DONLY = false>
+          bool DONLY = false, bool UNFLIP = false>
 __device__ __forceinline__ void onesweep_tile(
   const SweepArgs<BIG>& a,
   const uint32_t vcount,    // VIRT: positions in this pass's group, their bit offsets (8 bits each)
@@ -591,10 +604,12 @@ __device__ __forceinline__ void onesweep_tile(
     key[i] = load_key(i);
   }
   if constexpr (XFORM) {
+    static_assert(!UNFLIP || (CODEC == CODEC_FLOAT && !HAS_IDX), "images are mapped back for keys-only float sorts");
     if (a.first) {  // one uniform branch around all items, so that the loads above stay batched
 #pragma unroll
       for (int i = 0; i < ITEMS; ++i) {
-        key[i] = ordered_bits<CODEC, KeyT>(key[i]);
+        // (UNFLIP: no key is a NaN or a -0.0, for which alone the two images differ)
+        key[i] = UNFLIP ? sign_flip<KeyT>(key[i]) : ordered_bits<CODEC, KeyT>(key[i]);
       }
     }
   }
@@ -824,6 +839,14 @@ __device__ __forceinline__ void onesweep_tile(
       dq[k / 4]        = (k % 4 == 0) ? d : (dq[k / 4] | (d << (8 * (k % 4))));
     }
     if (a.keys_out != nullptr) {
+      if constexpr (UNFLIP) {
+        if (a.idx_final) {  // the last pass: the caller gets the keys' own bits back
+#pragma unroll
+          for (int k = 0; k < ITEMS; ++k) {
+            kk[k] = sign_unflip<KeyT>(kk[k]);
+          }
+        }
+      }
       KeyT* kout = static_cast<KeyT*>(a.keys_out) + row_base;
 #pragma unroll
       for (int k = 0; k < ITEMS; ++k) {
@@ -990,6 +1013,23 @@ void onesweep_kernel(const SweepArgs<BIG> a_in)
                                                                                        row, trow, static_cast<uint32_t>(remain));
     }
     return;
+  }
+  // keys-only sorts of float keys: the device-side plan says whether the passes run on stored images
+  // (keys of 4 and 8 bytes: the transform of a 2-byte key is cheap, and the second code path costs its
+  // kernel a workgroup per CU)
+  constexpr bool CAN_FLIP = !HAS_IDX && !XFORM && !DONLY && CODEC == CODEC_FLOAT && KeyTraits<CODEC, KeyT>::NWORDS == 1 &&
+                            sizeof(KeyT) >= 4;
+  if constexpr (CAN_FLIP) {
+    if (a_in.plan->flipped != 0) {  // uniform for the sort
+      if (remain >= static_cast<uint64_t>(TILE)) {
+        onesweep_tile<KeyT, CODEC, true, BIG, HAS_IDX, BLOCK, ITEMS, true, false, false, true>(a, 0u, 0ull, nullptr, sh, tile,
+                                                                                                row, trow, TILE);
+      } else {
+        onesweep_tile<KeyT, CODEC, true, BIG, HAS_IDX, BLOCK, ITEMS, false, false, false, true>(
+          a, 0u, 0ull, nullptr, sh, tile, row, trow, static_cast<uint32_t>(remain));
+      }
+      return;
+    }
   }
   if constexpr (!DONLY) {  // (a DONLY launch has returned above unless the virtual plan is in force)
     if (remain >= static_cast<uint64_t>(TILE)) {

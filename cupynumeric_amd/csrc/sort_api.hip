@@ -104,6 +104,19 @@ static const long long g_count16_min_row = [] {
 
 uint64_t count16_min_row() { return g_count16_min_row < 0 ? 0 : static_cast<uint64_t>(g_count16_min_row); }
 
+
+static const long long g_rank_row_min = [] {
+  const char* e = getenv("CPN_SORT_RANK_ROW_MIN");
+  return (e != nullptr && *e != 0) ? atoll(e) : static_cast<long long>(RANK_ROW_MIN);
+}();
+static const long long g_rank_row_max = [] {
+  const char* e = getenv("CPN_SORT_RANK_ROW_MAX");
+  return (e != nullptr && *e != 0) ? atoll(e) : static_cast<long long>(RANK_ROW_MAX);
+}();
+
+uint64_t rank_row_min() { return g_rank_row_min < 2 ? 2 : static_cast<uint64_t>(g_rank_row_min); }
+uint64_t rank_row_max() { return g_rank_row_max < 0 ? 0 : static_cast<uint64_t>(g_rank_row_max); }
+
 uint64_t wave_row_limit()
 {
   const long long limit = g_wave_row_limit.load(std::memory_order_relaxed);

@@ -334,7 +334,7 @@ from cupynumeric_amd import _lib
 lib = _lib.load()
 rng = np.random.default_rng(5)
 for dtype in (np.float16, np.int16, np.uint16):
-    for seg in (4097, 6000, 8191, 8192):
+    for seg in (4097, 6000, 8191, 8192, 9001, 16384):
         if dtype == np.float16:
             x = rng.standard_normal((5, seg)).astype(dtype)
             x[1, ::5] = np.nan
