@@ -1,14 +1,24 @@
-// Rows of up to 64 elements of real keys of up to 8 bytes, one element per lane and 64/S rows per
-// wavefront (S = slots per row, the next power of two), and rows of 65 ... 128 such keys, two
-// elements per lane and one row per wavefront, sorted by a bitonic network of
-// compare-exchanges between lanes.  What is compared is (order-preserving image of the key,
-// position in the row) as one unsigned word (an image and a position word for 8-byte keys), so
-// that no two are equal: the network, which is not stable by itself, then yields exactly the
-// stable order (NaNs tie with each other and +0.0 with -0.0 in the image, and the position
-// decides), and slots past the end of a row, which hold the largest image, sort behind every real
-// element.  The raw keys do not travel: every lane fetches the key of the position that ended up
-// in its slot once, at the end.  log2(S) (log2(S) + 1) / 2 exchanges of about eight vector
-// instructions (twelve for 8-byte keys), no LDS memory, no passes.
+// Rows of up to 128 real keys of up to 8 bytes (up to 256 keys of 1 and 2 bytes), sorted by a bitonic
+// network of compare-exchanges on words held in registers, eight elements per lane: element i of a
+// row sits in register i % 8 of the row's lane i / 8, a row of N slots (N = the next power of two
+// from 8 on) takes N / 8 lanes and a wavefront holds 512 / N rows.  The exchanges at distance 1, 2
+// and 4 happen between the registers of a lane (a compare and the selects), only those at distance 8
+// and more cross lanes, at lane distance 1, 2, ... through DPP and swizzle moves: of the 28 steps of
+// a row of 128 keys, 18 are inside the lanes and 10 cross them.  (One element per lane, the layout
+// this kernel started with, crosses lanes in all 28 steps: 2^26 float32 keys in rows of 128 took
+// 0.28 ms, now 0.22; rows of 32 0.25, now 0.13; rows of 8 0.20, now 0.09.)
+//
+// What is compared is (order-preserving image of the key, position in the row) as one unsigned word
+// (an image and a position word for 8-byte keys), so that no two are equal: the network, which is
+// not stable by itself, then yields exactly the stable order (NaNs tie with each other and +0.0 with
+// -0.0 in the image, and the position decides), and slots past the end of a row, which hold the
+// largest image, sort behind every real element.  The raw keys do not travel: they wait in LDS, and
+// every lane fetches the keys of the positions that ended up in its slots once, at the end.
+//
+// Memory is read and written in whole contiguous stretches: a lane of a full row moves its eight
+// neighbouring elements as 16-byte vectors; rows that are not full go through LDS, where the rows of
+// a wavefront lie as they do in memory, copied in and out with neighbouring lanes on neighbouring
+// elements.
 //
 // Stands, for such rows, where the reference sorts (segment id, value) tuples with a merge sort
 // (src/cupynumeric/sort/thrust_sort.cuh:68-122).
@@ -77,138 +87,261 @@ __device__ __forceinline__ uint32_t word_pos(uint32_t w) { return w; }
 __device__ __forceinline__ uint32_t word_pos(uint64_t w) { return static_cast<uint32_t>(w); }
 __device__ __forceinline__ uint32_t word_pos(const ImagePos& w) { return static_cast<uint32_t>(w.pos); }
 
-// One step of the network on rows of N = 64 E elements, element i of a row in register i / 64 of
-// lane i % 64 (E == 1: S <= 64 slots per row and 64 / S rows per wavefront): element i meets
-// element i ^ J, and the one of the two that is to hold the smaller word is the lower one where
-// the run of K elements it belongs to ascends.  J < 64 exchanges between lanes, J >= 64 between
-// the registers of a lane.
-template <int K, int J, int N, int E, typename W>
-__device__ __forceinline__ void bitonic_exchange(W (&w)[E], uint32_t lane)
+// Elements per lane.
+constexpr int BLOCKED_E = 8;
+
+// One compare-exchange between two registers of a lane; `ascending`: the smaller word goes to `lo`.
+template <typename W>
+__device__ __forceinline__ void blocked_exchange_in_lane(W& lo, W& hi, bool ascending)
 {
-  if constexpr (J < WAVE) {
-    const bool lower = (lane & J) == 0;
+  const W a = lo, b = hi;
+  const bool swap = (b < a) == ascending;
+  lo              = word_select(swap, b, a);
+  hi              = word_select(swap, a, b);
+}
+
+// Step (K, J) of the network on rows of N slots; `sub` is the lane's number inside its row.
+template <int K, int J, int N, typename W>
+__device__ __forceinline__ void blocked_step(W (&w)[BLOCKED_E], uint32_t sub)
+{
+  constexpr int E = BLOCKED_E;
+  if constexpr (J < E) {
 #pragma unroll
-    for (int e = 0; e < E; ++e) {
-      const W other = lane_xor<J>(w[e]);
-      // (the last merge of a row ascends in every row of the wave)
-      const bool ascending = (K == N) || (K < WAVE ? (lane & K) == 0 : ((e * WAVE) & K) == 0);
-      const bool keep_min  = lower == ascending;
-      w[e]                 = word_select((w[e] < other) == keep_min, w[e], other);
-    }
-  } else {
-    constexpr int D = J / WAVE;
-#pragma unroll
-    for (int e = 0; e < E; ++e) {
-      if ((e & D) == 0) {
-        const bool ascending = (K == N) || (((e * WAVE) & K) == 0);
-        const W a = w[e], b = w[e + D];
-        const bool swap = (b < a) == ascending;
-        w[e]            = word_select(swap, b, a);
-        w[e + D]        = word_select(swap, a, b);
+    for (int r = 0; r < E; ++r) {
+      if ((r & J) == 0) {
+        // the run of K elements this pair belongs to ascends where bit K of the element number is clear
+        const bool ascending = (K == N) || (K < E ? (r & K) == 0 : (sub & (K / E)) == 0);
+        blocked_exchange_in_lane(w[r], w[r | J], ascending);
       }
     }
-  }
-}
-template <int K, int J, int N, int E, typename W>
-__device__ __forceinline__ void bitonic_merge(W (&w)[E], uint32_t lane)
-{
-  if constexpr (J >= 1) {
-    bitonic_exchange<K, J, N>(w, lane);
-    if constexpr (J > 1) {
-      bitonic_merge<K, J / 2, N>(w, lane);
+  } else {
+    constexpr int D      = J / E;  // lane distance
+    const bool lower     = (sub & D) == 0;
+    const bool ascending = (K == N) || ((sub & (K / E)) == 0);
+    const bool keep_min  = lower == ascending;
+#pragma unroll
+    for (int r = 0; r < E; ++r) {
+      const W other = lane_xor<D>(w[r]);
+      w[r]          = word_select((w[r] < other) == keep_min, w[r], other);
     }
   }
 }
-template <int K, int N, int E, typename W>
-__device__ __forceinline__ void bitonic_sort(W (&w)[E], uint32_t lane)
+template <int K, int J, int N, typename W>
+__device__ __forceinline__ void blocked_merge(W (&w)[BLOCKED_E], uint32_t sub)
+{
+  if constexpr (J >= 1) {
+    blocked_step<K, J, N>(w, sub);
+    if constexpr (J > 1) {
+      blocked_merge<K, J / 2, N>(w, sub);
+    }
+  }
+}
+template <int K, int N, typename W>
+__device__ __forceinline__ void blocked_sort(W (&w)[BLOCKED_E], uint32_t sub)
 {
   if constexpr (K <= N) {
-    bitonic_merge<K, K / 2, N>(w, lane);
+    blocked_merge<K, K / 2, N>(w, sub);
     if constexpr (K < N) {
-      bitonic_sort<2 * K, N>(w, lane);
+      blocked_sort<2 * K, N>(w, sub);
     }
   }
 }
 
-// S = slots per row (power of two, 2 ... 128, >= row length); 64/S rows per wavefront up to 64
-// slots, one row per wavefront and two elements per lane for 128.
-template <typename KeyT, int CODEC, bool HAS_IDX, int S>
+// N = slots per row (8 ... 512, a power of two, >= row length); N / 8 lanes per row, 512 / N rows per
+// wavefront, four wavefronts per workgroup.
+template <typename KeyT, int CODEC, bool HAS_IDX, int N>
 __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __restrict__ keys_in,
-                                                                KeyT* keys_out,
-                                                                int64_t* __restrict__ idx_out,
-                                                                uint32_t seg,
-                                                                uint64_t rows,
-                                                                int64_t index_offset,
-                                                                uint32_t* status)
+                                                                        KeyT* keys_out,
+                                                                        int64_t* __restrict__ idx_out,
+                                                                        uint32_t seg,
+                                                                        uint64_t rows,
+                                                                        int64_t index_offset,
+                                                                        uint32_t* status)
 {
   static_assert(sizeof(KeyT) <= 8 && (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT),
                 "real keys of up to 8 bytes");
-  static_assert(S >= 2 && S <= 2 * WAVE && (S & (S - 1)) == 0, "slots per row: a power of two up to 128");
-
+  constexpr int E = BLOCKED_E;
+  static_assert(N >= E && N <= E * WAVE && (N & (N - 1)) == 0, "slots per row: a power of two from 8 to 512");
   if (blockIdx.x == 0 && threadIdx.x == 0) {
     *status = 0;  // the workspace's status word: a per-row sort cannot fail on the device
   }
-  // 4-byte keys: image in the high word, position in the low one; shorter keys: image << 8 | position;
+  // 4-byte keys: image in the high word, position in the low one; shorter keys: image << 16 | position;
   // 8-byte keys: two registers for the image, one for the position
   using W = std::conditional_t<sizeof(KeyT) == 8, ImagePos, std::conditional_t<sizeof(KeyT) == 4, uint64_t, uint32_t>>;
-  constexpr int E         = S > WAVE ? S / WAVE : 1;  // elements per lane
-  constexpr int LANES     = S > WAVE ? WAVE : S;      // lanes per row
+  constexpr int LANES     = N / E;  // lanes per row
   constexpr int ROWS_WAVE = WAVE / LANES;
+  constexpr int WAVES     = 256 / WAVE;
+  __shared__ KeyT s_raw[256 * E];
+  __shared__ uint16_t s_from[HAS_IDX ? 256 * E : 1];
 
-  const uint32_t lane = threadIdx.x & (WAVE - 1);
-  const uint64_t wave = static_cast<uint64_t>(blockIdx.x) * (256 / WAVE) + threadIdx.x / WAVE;
-  const uint32_t slot = lane & (LANES - 1);  // position of this lane's first element in its row
-  const uint64_t row  = wave * ROWS_WAVE + lane / LANES;
-  const uint64_t base = row * seg;
+  const uint32_t lane   = threadIdx.x & (WAVE - 1);
+  const uint32_t wslot  = threadIdx.x / WAVE;
+  const uint64_t wave   = static_cast<uint64_t>(blockIdx.x) * WAVES + wslot;
+  const uint32_t sub    = lane & (LANES - 1);
+  const uint32_t wrow   = lane / LANES;  // row of this lane inside its wavefront
+  const uint64_t row    = wave * ROWS_WAVE + wrow;
+  const uint64_t base   = row * seg;
+  const uint32_t first  = sub * E;  // position of this lane's first element in its row
+  const bool row_exists = row < rows;
+
+  // Full rows whose lanes' eight elements can be moved as 16-byte (single bytes: 8-byte) vectors: a wavefront
+  // then reads and writes whole contiguous kilobytes per instruction.  Other rows go through LDS: the rows of
+  // a wavefront are one contiguous stretch of memory, which its lanes copy in and out element by element,
+  // neighbouring lanes on neighbouring elements, and from which every lane takes the eight elements it owns.
+  constexpr int LANE_BYTES = E * static_cast<int>(sizeof(KeyT));
+  using VecT               = std::conditional_t<(LANE_BYTES >= 16), uint4, uint2>;
+  constexpr int VECS       = LANE_BYTES / static_cast<int>(sizeof(VecT));
+  const bool vec_keys = (seg == N) && ((reinterpret_cast<uintptr_t>(keys_in) | reinterpret_cast<uintptr_t>(keys_out)) &
+                                       (sizeof(VecT) - 1)) == 0;  // uniform
+  const bool vec_idx  = (seg == N) && (reinterpret_cast<uintptr_t>(idx_out) & 15u) == 0;
+  // the stretch of this wavefront: its rows, densely, as in memory
+  const uint64_t wave_row0 = wave * ROWS_WAVE;
+  const uint32_t wave_rows =
+    wave_row0 >= rows ? 0u : static_cast<uint32_t>(rows - wave_row0 < ROWS_WAVE ? rows - wave_row0 : ROWS_WAVE);
+  const uint32_t stretch_len  = wave_rows * seg;  // at most 512 elements
+  const uint64_t stretch_base = wave_row0 * seg;
+  KeyT* const s_wave          = s_raw + wslot * (WAVE * E);
+  KeyT* const s_row           = s_wave + wrow * seg;  // this lane's row inside the stretch
 
   KeyT raw[E];
+  if (vec_keys) {
+    VecT q[VECS];
+#pragma unroll
+    for (int v = 0; v < VECS; ++v) {
+      q[v] = VecT{};
+      if (row_exists) {
+        q[v] = reinterpret_cast<const VecT*>(keys_in + base + first)[v];
+      }
+    }
+    __builtin_memcpy(raw, q, LANE_BYTES);
+  } else {
+    KeyT got[E];
+#pragma unroll
+    for (int k = 0; k < E; ++k) {  // (all loads first)
+      const uint32_t e = lane + k * WAVE;
+      got[k]           = KeyT{};
+      if (e < stretch_len) {
+        got[k] = keys_in[stretch_base + e];
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < E; ++k) {
+      const uint32_t e = lane + k * WAVE;
+      if (e < stretch_len) {
+        s_wave[e] = got[k];
+      }
+    }
+    __builtin_amdgcn_wave_barrier();  // (a stretch belongs to one wavefront, whose LDS operations execute in order)
+#pragma unroll
+    for (int r = 0; r < E; ++r) {
+      const uint32_t pos = first + r;
+      raw[r]             = KeyT{};
+      if (row_exists && pos < seg) {
+        raw[r] = s_row[pos];
+      }
+    }
+  }
   W w[E];
 #pragma unroll
-  for (int e = 0; e < E; ++e) {  // (all loads first)
-    const uint32_t pos = slot + e * WAVE;
-    const bool valid   = (row < rows) && (pos < seg);
-    raw[e]             = KeyT{};
-    if (valid) {
-      raw[e] = keys_in[base + pos];
-    }
-  }
-#pragma unroll
-  for (int e = 0; e < E; ++e) {
-    const uint32_t pos = slot + e * WAVE;
-    const bool valid   = (row < rows) && (pos < seg);
-    const KeyT image   = valid ? ordered_bits<CODEC, KeyT>(raw[e]) : static_cast<KeyT>(~KeyT{0});
+  for (int r = 0; r < E; ++r) {
+    const uint32_t pos = first + r;
+    const bool valid   = row_exists && pos < seg;
+    // (slots past the end of a row: the largest image, and a position behind every element's)
+    const KeyT image = valid ? ordered_bits<CODEC, KeyT>(raw[r]) : static_cast<KeyT>(~KeyT{0});
     if constexpr (sizeof(KeyT) == 8) {
-      w[e] = ImagePos{image, pos};
+      w[r] = ImagePos{image, pos};
     } else {
-      w[e] = (static_cast<W>(image) << (sizeof(KeyT) == 4 ? 32 : 8)) | pos;
+      w[r] = (static_cast<W>(image) << (sizeof(KeyT) == 4 ? 32 : 16)) | pos;
     }
   }
-  bitonic_sort<2, S>(w, lane);
+  blocked_sort<2, N>(w, sub);
 
+  // ---- slot p of the sorted row holds the element that came from position `from` ----
+  uint32_t from[E];
 #pragma unroll
-  for (int e = 0; e < E; ++e) {
-    const uint32_t pos  = slot + e * WAVE;
-    const uint32_t from = word_pos(w[e]) & (S - 1);  // the position whose element belongs here
-    const int src_lane  = static_cast<int>((lane & ~(LANES - 1)) | (from & (LANES - 1)));
-    KeyT bits           = KeyT{};
+  for (int r = 0; r < E; ++r) {
+    from[r] = word_pos(w[r]) & (N - 1);
+  }
+  if (keys_out != nullptr) {
+    if (vec_keys) {
+      // every lane parks its raw keys and takes those of the positions that ended up in its slots
+      KeyT* mine = s_wave + wrow * N;
 #pragma unroll
-    for (int f = 0; f < E; ++f) {  // the register of that lane that holds it
-      KeyT got;
-      if constexpr (sizeof(KeyT) == 8) {
-        const uint32_t lo = static_cast<uint32_t>(__shfl(static_cast<int>(static_cast<uint32_t>(raw[f])), src_lane, WAVE));
-        const uint32_t hi = static_cast<uint32_t>(__shfl(static_cast<int>(static_cast<uint32_t>(raw[f] >> 32)), src_lane, WAVE));
-        got               = (static_cast<uint64_t>(hi) << 32) | lo;
-      } else {
-        got = static_cast<KeyT>(__shfl(static_cast<int>(static_cast<uint32_t>(raw[f])), src_lane, WAVE));
+      for (int r = 0; r < E; ++r) {
+        mine[first + r] = raw[r];
       }
-      bits = (E == 1 || from / WAVE == static_cast<uint32_t>(f)) ? got : bits;
+      __builtin_amdgcn_wave_barrier();
+      KeyT bits[E];
+#pragma unroll
+      for (int r = 0; r < E; ++r) {
+        bits[r] = mine[from[r]];
+      }
+      if (row_exists) {
+        VecT q[VECS];
+        __builtin_memcpy(q, bits, LANE_BYTES);
+#pragma unroll
+        for (int v = 0; v < VECS; ++v) {
+          reinterpret_cast<VecT*>(keys_out + base + first)[v] = q[v];
+        }
+      }
+    } else {
+      // the stretch still holds the raw keys: permute it in place (all reads, then all writes), copy it out
+      KeyT bits[E];
+#pragma unroll
+      for (int r = 0; r < E; ++r) {
+        const uint32_t pos = first + r;
+        bits[r]            = (row_exists && pos < seg) ? s_row[from[r]] : KeyT{};
+      }
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int r = 0; r < E; ++r) {
+        const uint32_t pos = first + r;
+        if (row_exists && pos < seg) {
+          s_row[pos] = bits[r];
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int k = 0; k < E; ++k) {
+        const uint32_t e = lane + k * WAVE;
+        if (e < stretch_len) {
+          keys_out[stretch_base + e] = s_wave[e];
+        }
+      }
     }
-    if ((row < rows) && (pos < seg)) {  // (the first seg positions of a row hold its seg elements)
-      if (keys_out != nullptr) {
-        keys_out[base + pos] = bits;
+  }
+  if constexpr (HAS_IDX) {
+    if (vec_idx) {
+      if (row_exists) {
+        int64_t out[E];
+#pragma unroll
+        for (int r = 0; r < E; ++r) {
+          out[r] = static_cast<int64_t>(from[r]) + index_offset;
+        }
+        uint4 q[E / 2];
+        __builtin_memcpy(q, out, sizeof(out));
+#pragma unroll
+        for (int v = 0; v < E / 2; ++v) {
+          reinterpret_cast<uint4*>(idx_out + base + first)[v] = q[v];
+        }
       }
-      if constexpr (HAS_IDX) {
-        idx_out[base + pos] = static_cast<int64_t>(from) + index_offset;
+    } else {
+      // positions through LDS as well, so that neighbouring lanes store neighbouring int64 words
+      uint16_t* const s_fwave = s_from + wslot * (WAVE * E);
+#pragma unroll
+      for (int r = 0; r < E; ++r) {
+        const uint32_t pos = first + r;
+        if (row_exists && pos < seg) {
+          s_fwave[wrow * seg + pos] = static_cast<uint16_t>(from[r]);
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int k = 0; k < E; ++k) {
+        const uint32_t e = lane + k * WAVE;
+        if (e < stretch_len) {
+          idx_out[stretch_base + e] = static_cast<int64_t>(s_fwave[e]) + index_offset;
+        }
       }
     }
   }

@@ -353,10 +353,12 @@ __global__ __launch_bounds__(COUNT16_BLOCK) void count16_rows_kernel(const uint1
   }
 }
 
-// Rows of 8193 to 16 384 keys.  grid = rows, block = 1024, thread t owns elements [16t, 16t+16).
+// Rows of 8193 to 16 384 keys (ITEMS = 16) and of up to 32 768 (ITEMS = 32).  grid = rows, block = 1024,
+// thread t owns elements [ITEMS t, ITEMS (t + 1)).
 // No LDS is left for a marker row here: every key takes its offset from an atomic on the scanned
-// histogram and is staged in the histogram's memory once that is no longer needed.
-template <int CODEC>
+// histogram and is staged in the histogram's memory once that is no longer needed (65 536 bins of 16
+// bits are room for 65 536 keys; a bin counts up to 65 535, more than the longest row).
+template <int CODEC, int ITEMS>
 __global__ __launch_bounds__(COUNT16_BLOCK) void count16_long_rows_kernel(const uint16_t* keys_in,
                                                                            uint16_t* keys_out,
                                                                            uint32_t seg,
@@ -366,7 +368,7 @@ __global__ __launch_bounds__(COUNT16_BLOCK) void count16_long_rows_kernel(const 
   if (blockIdx.x == 0 && threadIdx.x == 0) {
     *status = 0;  // the workspace's status word: a per-row sort cannot fail on the device
   }
-  constexpr int ITEMS = 16;
+  static_assert(ITEMS % 8 == 0 && COUNT16_BLOCK * ITEMS < 65536, "whole 16-byte loads; counts and offsets fit 16 bits");
   constexpr int WAVES = COUNT16_BLOCK / WAVE;
   __shared__ __align__(16) uint32_t s_hist[COUNT16_WORDS];
   __shared__ uint32_t s_wsum[WAVES];

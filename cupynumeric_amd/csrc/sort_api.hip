@@ -105,18 +105,6 @@ static const long long g_count16_min_row = [] {
 uint64_t count16_min_row() { return g_count16_min_row < 0 ? 0 : static_cast<uint64_t>(g_count16_min_row); }
 
 
-static const long long g_rank_row_min = [] {
-  const char* e = getenv("CPN_SORT_RANK_ROW_MIN");
-  return (e != nullptr && *e != 0) ? atoll(e) : static_cast<long long>(RANK_ROW_MIN);
-}();
-static const long long g_rank_row_max = [] {
-  const char* e = getenv("CPN_SORT_RANK_ROW_MAX");
-  return (e != nullptr && *e != 0) ? atoll(e) : static_cast<long long>(RANK_ROW_MAX);
-}();
-
-uint64_t rank_row_min() { return g_rank_row_min < 2 ? 2 : static_cast<uint64_t>(g_rank_row_min); }
-uint64_t rank_row_max() { return g_rank_row_max < 0 ? 0 : static_cast<uint64_t>(g_rank_row_max); }
-
 uint64_t wave_row_limit()
 {
   const long long limit = g_wave_row_limit.load(std::memory_order_relaxed);
@@ -126,7 +114,10 @@ uint64_t wave_row_limit()
 uint64_t lds_row_limit(int key_bytes, bool with_positions)
 {
   const long long limit = g_lds_row_limit.load(std::memory_order_relaxed);
-  const uint64_t cap    = lds_row_capacity(key_bytes, with_positions);
+  uint64_t cap          = lds_row_capacity(key_bytes, with_positions);
+  if (key_bytes == 2 && !with_positions && count16_min_row() <= cap + 1) {
+    cap = COUNT16_ROW_CAPACITY;  // the counting kernel takes over where the radix shapes end
+  }
   if (limit >= 0 && static_cast<uint64_t>(limit) < cap) {
     return static_cast<uint64_t>(limit);
   }

@@ -98,6 +98,9 @@ __host__ __device__ constexpr uint64_t lds_row_capacity(int key_bytes, bool with
 {
   return key_bytes == 16 ? 4096 : (key_bytes == 8 ? (with_positions ? 14336 : 16384) : 16384);
 }
+// Values-only sorts of 2-byte keys: the counting kernel (count_row_sort.h) needs no room for the row beside
+// its 65 536 bins and takes rows of up to 32 768 keys (lds_row_limit says whether it is in use).
+constexpr uint64_t COUNT16_ROW_CAPACITY = 32768;
 // Radix passes of a key: one per byte, plus the NaN-class pass of complex keys.
 __host__ __device__ constexpr int key_passes(int key_bytes, int codec)
 {
@@ -116,12 +119,6 @@ uint64_t wave_row_limit();
 // (count_row_sort.h): COUNT16_MIN_ROW unless CPN_SORT_COUNT16_MIN_ROW in the environment says
 // otherwise (A/B runs; a value above the LDS row capacity switches the kernel off).
 uint64_t count16_min_row();
-// Row lengths given to the counting-rank kernel (rank_row_sort.h): 33 ... 48 and 65 ... 72 (68 for 4-byte
-// keys), as far as they lie in RANK_ROW_MIN ... RANK_ROW_MAX, which CPN_SORT_RANK_ROW_MIN /
-// CPN_SORT_RANK_ROW_MAX in the environment can narrow (A/B runs; min above max switches the kernel off).
-uint64_t rank_row_min();
-uint64_t rank_row_max();
-constexpr uint64_t RANK_ROW_MIN = 33, RANK_ROW_MAX = 72;
 
 // Row length up to which the LDS kernel is used.  Equals lds_row_capacity unless the
 // environment variable CPN_SORT_LDS_ROW_LIMIT or cpn_set_lds_row_limit lowers it, e.g. to 0
@@ -434,8 +431,13 @@ inline int launch_count16_rows(const SortRequest& r)
       hipLaunchKernelGGL((count16_rows_kernel<CODEC>), dim3(static_cast<uint32_t>(grid)), dim3(COUNT16_BLOCK), 0, r.stream,
                          static_cast<const uint16_t*>(r.values_in), static_cast<uint16_t*>(r.values_out),
                          static_cast<uint32_t>(r.seg), static_cast<uint32_t>(rows), static_cast<uint32_t*>(r.temp));
+    } else if (r.seg <= 16384) {
+      hipLaunchKernelGGL((count16_long_rows_kernel<CODEC, 16>), dim3(static_cast<uint32_t>(rows)), dim3(COUNT16_BLOCK), 0,
+                         r.stream, static_cast<const uint16_t*>(r.values_in), static_cast<uint16_t*>(r.values_out),
+                         static_cast<uint32_t>(r.seg), static_cast<uint32_t*>(r.temp));
     } else {
-      hipLaunchKernelGGL((count16_long_rows_kernel<CODEC>), dim3(static_cast<uint32_t>(rows)), dim3(COUNT16_BLOCK), 0,
+      // 16 385 ... 32 768 keys: 32 keys per thread
+      hipLaunchKernelGGL((count16_long_rows_kernel<CODEC, 32>), dim3(static_cast<uint32_t>(rows)), dim3(COUNT16_BLOCK), 0,
                          r.stream, static_cast<const uint16_t*>(r.values_in), static_cast<uint16_t*>(r.values_out),
                          static_cast<uint32_t>(r.seg), static_cast<uint32_t*>(r.temp));
     }
@@ -462,16 +464,16 @@ inline int launch_wave_rows(const SortRequest& r)
   return CPN_OK;
 }
 
-template <typename KeyT, int CODEC, bool HAS_IDX, int S>
+template <typename KeyT, int CODEC, bool HAS_IDX, int N>
 inline int launch_bitonic_rows(const SortRequest& r)
 {
   const uint64_t rows           = r.volume / r.seg;
-  const uint64_t rows_per_block = (256 / WAVE) * (S >= WAVE ? 1 : WAVE / S);
+  const uint64_t rows_per_block = (256 / WAVE) * (BLOCKED_E * WAVE / N);
   const uint64_t blocks         = (rows + rows_per_block - 1) / rows_per_block;
   {
     ProfileScope prof("bitonic_row_sort", r.stream);
-    hipLaunchKernelGGL((bitonic_row_sort_kernel<KeyT, CODEC, HAS_IDX, S>), dim3(static_cast<uint32_t>(blocks)), dim3(256),
-                       0, r.stream, static_cast<const KeyT*>(r.values_in), static_cast<KeyT*>(r.values_out),
+    hipLaunchKernelGGL((bitonic_row_sort_kernel<KeyT, CODEC, HAS_IDX, N>), dim3(static_cast<uint32_t>(blocks)),
+                       dim3(256), 0, r.stream, static_cast<const KeyT*>(r.values_in), static_cast<KeyT*>(r.values_out),
                        r.indices_out, static_cast<uint32_t>(r.seg), rows, r.index_offset, static_cast<uint32_t*>(r.temp));
   }
   CPN_HIP_TRY(hipGetLastError());
@@ -523,27 +525,16 @@ inline int sort_rows_in_lds(const SortRequest& r)
     return CPN_ERR_UNSUPPORTED;
   }
   if constexpr (sizeof(KeyT) <= 8 && (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT)) {
-    // real keys, row lengths just past a power of two, where the network below would run half empty:
-    // every element counts the elements of its row that come before it
-    // (measured on 2^26 keys, this kernel / the network: rows of 33 float32 keys 0.30 / 0.52 ms, of 40 0.33 / 0.44,
-    // of 48 0.37 / 0.37, of 65 0.49 / 0.51, of 72 0.48 / 0.46; float64 rows of 33 0.39 / 0.73, of 48 0.49 / 0.54,
-    // of 65 0.63 / 0.79, of 72 0.63 / 0.74, of 80 0.72 / 0.68; float16 rows of 33 0.19 / 0.40, of 48 0.25 / 0.28,
-    // of 65 0.33 / 0.38, of 72 0.32 / 0.35, of 80 0.36 / 0.32)
-    if (r.seg >= rank_row_min() && r.seg <= rank_row_max() && r.seg <= 2 * RANK_ROW_BLOCK && r.seg <= wave_row_limit() &&
-        bitonic_rows_enabled()) {
-      const bool first  = r.seg >= 33 && r.seg <= 48;
-      const bool second = r.seg >= 65 && r.seg <= (sizeof(KeyT) == 4 ? 68u : 72u);
-      if (first || second) {
-        return launch_rank_rows<KeyT, CODEC, HAS_IDX>(r);
-      }
+    // Rows just past 32 keys, where the network below would run in 64 slots: every element counts the
+    // elements of its row that come before it (measured on 2^26 keys, counting / network: rows of 33 float32
+    // keys 0.29 / 0.31 ms, of 40 0.33 / 0.28; float64 rows of 33 0.39 / 0.49, of 40 0.43 / 0.44; float16
+    // rows of 33 0.20 / 0.23, of 40 0.22 / 0.20)
+    if (r.seg >= 33 && r.seg <= (sizeof(KeyT) == 8 ? 40u : 36u) && r.seg <= wave_row_limit() && bitonic_rows_enabled()) {
+      return launch_rank_rows<KeyT, CODEC, HAS_IDX>(r);
     }
-    // real keys, rows of 2 ... 128: a bitonic network between the lanes of a wavefront
-    if (r.seg >= 2 && r.seg <= 128 && r.seg <= wave_row_limit() && bitonic_rows_enabled()) {
-      if (r.seg <= 2) {
-        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 2>(r);
-      } else if (r.seg <= 4) {
-        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 4>(r);
-      } else if (r.seg <= 8) {
+    // rows of 2 ... 128 keys (256 for keys of 1 and 2 bytes): a bitonic network on eight elements per lane
+    if (r.seg >= 2 && r.seg <= (sizeof(KeyT) <= 2 ? 256u : 128u) && r.seg <= wave_row_limit() && bitonic_rows_enabled()) {
+      if (r.seg <= 8) {
         return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 8>(r);
       } else if (r.seg <= 16) {
         return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 16>(r);
@@ -551,8 +542,10 @@ inline int sort_rows_in_lds(const SortRequest& r)
         return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 32>(r);
       } else if (r.seg <= 64) {
         return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 64>(r);
-      } else {
+      } else if (r.seg <= 128) {
         return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 128>(r);
+      } else {
+        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 256>(r);
       }
     }
   }
@@ -689,6 +682,10 @@ inline int sort_rows_in_lds(const SortRequest& r)
           return launch_lds_rows<KeyT, CODEC, HAS_IDX, 512, 24>(r);  // two workgroups per CU, as above
         }
       }
+      // (2-byte keys, values only, come here when the counting kernel is switched off or starts later.  A
+      // 512 x 32 shape for them, two workgroups per CU and rows dealt in equal shares, measured 0.35 ms for
+      // 2^26 float16 keys in rows of 8193 and 0.27 in rows of 16 384 against the counting kernel's 0.38 and
+      // 0.19: not kept)
       return launch_lds_rows<KeyT, CODEC, HAS_IDX, 1024, 16>(r);  // up to 16 384 keys
     }
   }

@@ -356,9 +356,10 @@ int64_t cpn_set_lds_row_limit(int64_t limit);
 int64_t cpn_set_wave_row_limit(int64_t limit);
 
 /*
- * Process-wide switch: rows of 2 ... 128 real keys of up to 8 bytes are sorted by a bitonic network
- * between the lanes of a wavefront, one key per lane, two per lane above 64 keys (enabled != 0, the default) or by the ranking kernels that take
- * the other key types of that length (0).  Returns the previous setting.  Also initialised from the
+ * Process-wide switch: rows of 2 ... 128 real keys of up to 8 bytes (256 keys of 1 and 2 bytes) are sorted
+ * by a bitonic network on eight keys per lane of a wavefront -- rows of 33 ... 36 keys (40 of 8 bytes) by
+ * counting, for every key, the keys of its row that come before it -- (enabled != 0, the default) or by
+ * the ranking kernels that take the other key types of that length (0).  Returns the previous setting.  Also initialised from the
  * environment variable CPN_SORT_BITONIC_ROWS (0 switches it off).  Does not affect workspace sizes.
  * An A/B switch with no counterpart in the reference, which merge-sorts (segment id, value) tuples
  * for short rows (src/cupynumeric/sort/thrust_sort.cuh:68-122).

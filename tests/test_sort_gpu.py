@@ -376,6 +376,76 @@ def test_counting_kernel_for_rows_of_up_to_8192_keys_behind_its_switch(torch_cud
     assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stdout[-1000:] + out.stderr[-3000:]
 
 
+TWO_BYTE_LONG_ROWS_CHILD = r"""
+import numpy as np
+import cupynumeric_amd as num
+from cupynumeric_amd import _lib
+lib = _lib.load()
+rng = np.random.default_rng(6)
+u = np.uint16
+for dtype in (np.float16, np.int16, np.uint16):
+    for seg in (8193, 9001, 12000, 16383, 16384, 16385, 20001, 32768):
+        if dtype == np.float16:
+            x = rng.standard_normal((4, seg)).astype(dtype)
+            x[1, ::5] = np.nan
+            x[1, 1::5] = -0.0
+            x[1, 2::5] = 0.0
+            x[2] = x[2, 0]
+            b = x[3].view(u)
+            b[::7] = 0xFE01  # negative NaN with a payload
+        else:
+            info = np.iinfo(dtype)
+            x = rng.integers(info.min, info.max, (4, seg), dtype=dtype, endpoint=True)
+            x[2] = x[2, 0]
+        lib.cpn_profile_enable(1)
+        _lib.profile_collect()
+        got = np.asarray(num.sort(num.array(x)))
+        labels = {k for k, _ in _lib.profile_collect()}
+        lib.cpn_profile_enable(0)
+        assert labels == ({"lds_row_sort"} if seg <= 16384 else {"count16_row_sort"}), (dtype, seg, labels)
+        order = np.argsort(x.astype(np.float32), axis=-1, kind="stable") if dtype == np.float16 else np.argsort(x, axis=-1, kind="stable")
+        want = np.take_along_axis(x, order, axis=-1)
+        assert np.array_equal(got.view(u), want.view(u)), (dtype, seg)
+print("ok")
+"""
+
+
+def test_two_byte_rows_of_8193_to_16384_keys_through_the_radix_shape(torch_cuda):
+    """With the counting kernel starting at 16 385 keys (CPN_SORT_COUNT16_MIN_ROW, read when the library is
+    loaded), plain sorts of 8193 ... 16 384 two-byte keys take the radix kernel in its 1024 x 16 shape, rows
+    shorter than the tile dealt in equal shares, and longer rows still the counting kernel: a child process
+    checks bits and which kernel ran, with NaNs of both signs, payloads, zeros of both signs and constant rows."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, CPN_SORT_COUNT16_MIN_ROW="16385", PYTHONPATH=root + os.pathsep + os.environ.get("PYTHONPATH", ""))
+    out = subprocess.run([sys.executable, "-c", TWO_BYTE_LONG_ROWS_CHILD], env=env, cwd=root, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stdout[-1000:] + out.stderr[-3000:]
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.int16, np.uint16])
+def test_two_byte_rows_of_up_to_32768_keys_are_counted(lib, torch_cuda, dtype):
+    """Plain sorts of rows of 16 385 ... 32 768 two-byte keys: the counting kernel with 32 keys per thread
+    (zeros and NaNs in input order); one key more, and the same rows with positions, take the global path."""
+    u = np.uint16
+    for seg in (16385, 16392, 20001, 32767, 32768, 32769):
+        x = make_input(dtype, (5, seg), seed=seg)
+        x[2] = x[2, 0]
+        x[3] = np.sort(x[3])[::-1]
+        lib.cpn_profile_enable(1)
+        _lib.profile_collect()
+        v, _ = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=False)
+        labels = {k for k, _ in _lib.profile_collect()}
+        lib.cpn_profile_enable(0)
+        assert ("count16_row_sort" in labels) == (seg <= 32768), (seg, labels)
+        assert_same_bits(v, oracle.local_sort(x, argsort=False), f"{np.dtype(dtype)} seg={seg}")
+        v, _ = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=False, in_place=True)
+        assert_same_bits(v, oracle.local_sort(x, argsort=False), f"{np.dtype(dtype)} seg={seg} in place")
+        check_rows(lib, torch_cuda, x, f"{np.dtype(dtype)} seg={seg}")  # (also the argsort of the same rows)
+
+
 def test_lds_many_short_rows(lib, torch_cuda):
     for dtype, shape in [(np.float64, (3000, 37)), (np.int8, (5000, 5)), (np.float16, (700, 401)), (np.uint32, (129, 1024))]:
         check_rows(lib, torch_cuda, make_input(dtype, shape, seed=11), f"{np.dtype(dtype)} {shape}")
