@@ -7,13 +7,15 @@ ctypes.  There is no fallback: if the shared library is missing, loading raises.
 from __future__ import annotations
 
 import ctypes
+import os
 from ctypes import c_char_p, c_int, c_int64, c_uint64, c_void_p
 from pathlib import Path
 
 import numpy as np
 
 LIB_NAME = "libcpnsort.so"
-LIB_PATH = Path(__file__).resolve().parent / LIB_NAME
+# (CUPYNUMERIC_AMD_LIBRARY names another build of the same library, for A/B runs of kernel variants)
+LIB_PATH = Path(os.environ.get("CUPYNUMERIC_AMD_LIBRARY") or (Path(__file__).resolve().parent / LIB_NAME))
 
 # element type codes of include/cpn_sort.h (enum cpn_dtype)
 DTYPE_CODES: dict[np.dtype, int] = {

@@ -83,7 +83,7 @@ __host__ __device__ constexpr int global_block(int key_bytes) { return key_bytes
 // 64 KiB for 512 threads, two workgroups per CU, and is 128 KiB for the 1024 threads of 8-byte keys)
 __host__ __device__ constexpr int global_items(int key_bytes, bool big)
 {
-  return key_bytes == 16 ? CPN_GLOBAL_ITEMS / 4 : ((key_bytes == 8 || big) ? CPN_GLOBAL_ITEMS / 2 : CPN_GLOBAL_ITEMS);
+  return key_bytes == 16 ? 8 : ((key_bytes == 8 || big) ? 16 : CPN_GLOBAL_ITEMS);
 }
 __host__ __device__ constexpr int global_tile(int key_bytes, bool big)
 {
