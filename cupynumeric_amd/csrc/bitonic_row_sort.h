@@ -1,19 +1,22 @@
-// Rows of up to 128 real keys of up to 8 bytes (up to 256 keys of 1 and 2 bytes), sorted by a bitonic
-// network of compare-exchanges on words held in registers, eight elements per lane: element i of a
-// row sits in register i % 8 of the row's lane i / 8, a row of N slots (N = the next power of two
-// from 8 on) takes N / 8 lanes and a wavefront holds 512 / N rows.  The exchanges at distance 1, 2
-// and 4 happen between the registers of a lane (a compare and the selects), only those at distance 8
-// and more cross lanes, at lane distance 1, 2, ... through DPP and swizzle moves: of the 28 steps of
-// a row of 128 keys, 18 are inside the lanes and 10 cross them.  (One element per lane, the layout
-// this kernel started with, crosses lanes in all 28 steps: 2^26 float32 keys in rows of 128 took
-// 0.28 ms, now 0.22; rows of 32 0.25, now 0.13; rows of 8 0.20, now 0.09.)
+// Short rows of real keys of up to 8 bytes (how long: bitonic_row_limit, 128 ... 512 keys), sorted by a
+// bitonic network of compare-exchanges on words held in registers, eight elements per lane: element i of
+// a row sits in register i % 8 of the row's lane i / 8, a row of N slots (N = the next power of two from 8
+// on) takes N / 8 lanes and a wavefront holds 512 / N rows.  The exchanges between elements less than 8
+// apart happen between the registers of a lane, only the others cross lanes, through DPP and swizzle
+// moves: of the 28 steps of a row of 128 keys, 18 are inside the lanes and 10 cross them.  (One element
+// per lane, the layout this kernel started with, crosses lanes in all 28 steps: 2^26 float32 keys in rows
+// of 128 took 0.28 ms, rows of 32 0.25, rows of 8 0.20.)
 //
-// What is compared is (order-preserving image of the key, position in the row) as one unsigned word
-// (an image and a position word for 8-byte keys), so that no two are equal: the network, which is
-// not stable by itself, then yields exactly the stable order (NaNs tie with each other and +0.0 with
-// -0.0 in the image, and the position decides), and slots past the end of a row, which hold the
-// largest image, sort behind every real element.  The raw keys do not travel: they wait in LDS, and
-// every lane fetches the keys of the positions that ended up in its slots once, at the end.
+// What is compared: a sort that returns values only, on keys whose image is a bijection of their bits
+// (integers; floats when no row of the wavefront holds a NaN or a -0.0), sorts the bare images and maps
+// them back (2^26 float32 keys in rows of 128 0.11 ms, of 32 0.09: the speed of the memory).  Otherwise
+// the words are (order-preserving image of the key, position in the row) as one unsigned word (an image
+// and a position word for 8-byte keys), so that no two are equal: the network, which is not stable by
+// itself, then yields exactly the stable order (NaNs tie with each other and +0.0 with -0.0 in the image,
+// and the position decides); the raw keys do not travel: they wait in LDS, and every lane fetches the
+// keys of the positions that ended up in its slots once, at the end (rows of 128 float32 keys 0.22 ms,
+// with positions out 0.25).  Slots past the end of a row hold the largest image and sort behind, or
+// beside, every real element.
 //
 // Memory is read and written in whole contiguous stretches: a lane of a full row moves its eight
 // neighbouring elements as 16-byte vectors; rows that are not full go through LDS, where the rows of
@@ -90,18 +93,85 @@ __device__ __forceinline__ uint32_t word_pos(const ImagePos& w) { return static_
 // Elements per lane.
 constexpr int BLOCKED_E = 8;
 
-// One compare-exchange between two registers of a lane; `ascending`: the smaller word goes to `lo`.
-template <typename W>
-__device__ __forceinline__ void blocked_exchange_in_lane(W& lo, W& hi, bool ascending)
+// The value of lane (lane ^ M) for M = 2^k - 1: the lane's mirror image inside its group of M + 1 lanes.
+template <int M>
+__device__ __forceinline__ uint32_t lane_mirror(uint32_t v)
 {
-  const W a = lo, b = hi;
-  const bool swap = (b < a) == ascending;
-  lo              = word_select(swap, b, a);
-  hi              = word_select(swap, a, b);
+  static_assert(M == 1 || M == 3 || M == 7 || M == 15 || M == 31 || M == 63, "all bits below a power of two");
+  if constexpr (M == 1) {
+    return static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(v), 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
+  } else if constexpr (M == 3) {
+    return static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(v), 0x1B, 0xF, 0xF, true));  // quad_perm [3,2,1,0]
+  } else if constexpr (M == 7) {
+    return static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(v), 0x141, 0xF, 0xF, true));  // row_half_mirror
+  } else if constexpr (M == 15) {
+    return static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(v), 0x140, 0xF, 0xF, true));  // row_mirror
+  } else if constexpr (M == 31) {
+    return static_cast<uint32_t>(__builtin_amdgcn_ds_swizzle(static_cast<int>(v), (0x1F << 10) | 0x1F));  // xor mask within 32 lanes
+  } else {
+    return static_cast<uint32_t>(__shfl_xor(static_cast<int>(v), 63, WAVE));
+  }
+}
+template <int M>
+__device__ __forceinline__ uint64_t lane_mirror(uint64_t v)
+{
+  const uint32_t lo = lane_mirror<M>(static_cast<uint32_t>(v));
+  const uint32_t hi = lane_mirror<M>(static_cast<uint32_t>(v >> 32));
+  return (static_cast<uint64_t>(hi) << 32) | lo;
+}
+template <int M>
+__device__ __forceinline__ ImagePos lane_mirror(ImagePos v)
+{
+  return ImagePos{lane_mirror<M>(v.image), lane_mirror<M>(static_cast<uint32_t>(v.pos))};
 }
 
-// Step (K, J) of the network on rows of N slots; `sub` is the lane's number inside its row.
-template <int K, int J, int N, typename W>
+// One compare-exchange between two registers of a lane: the smaller word goes to `lo`.
+template <typename W>
+__device__ __forceinline__ void blocked_exchange_in_lane(W& lo, W& hi)
+{
+  const W a = lo, b = hi;
+  if constexpr (std::is_same_v<W, uint32_t>) {
+    lo = a < b ? a : b;  // (one min and one max instruction)
+    hi = a < b ? b : a;
+  } else {
+    const bool swap = b < a;
+    lo              = word_select(swap, b, a);
+    hi              = word_select(swap, a, b);
+  }
+}
+
+// The network is the bitonic sorter in the form whose comparators all point the same way: the merge of two
+// sorted runs of K / 2 elements starts by comparing element i with its mirror image i ^ (K - 1) in the run
+// of K, and goes on with the partners i ^ J for J = K / 4 ... 1; the smaller word always goes to the
+// smaller element number, so no step has to know which way its run points.  Element i of a row is register
+// i % 8 of lane i / 8: partners closer than 8 elements are registers of one lane, and a mirror image across
+// lanes is register 7 - r of the mirrored lane.  `sub` is the lane's number inside its row.
+template <int K, typename W>
+__device__ __forceinline__ void blocked_mirror_step(W (&w)[BLOCKED_E], uint32_t sub)
+{
+  constexpr int E = BLOCKED_E;
+  if constexpr (K <= E) {
+#pragma unroll
+    for (int r = 0; r < E; ++r) {
+      if ((r & (K / 2)) == 0) {
+        blocked_exchange_in_lane(w[r], w[r ^ (K - 1)]);
+      }
+    }
+  } else {
+    constexpr int M     = K / E - 1;                  // lane ^ M: the mirrored lane
+    const bool keep_min = (sub & ((M + 1) / 2)) == 0;  // the lower half of the run keeps the smaller words
+    W other[E];
+#pragma unroll
+    for (int r = 0; r < E; ++r) {
+      other[r] = lane_mirror<M>(w[E - 1 - r]);
+    }
+#pragma unroll
+    for (int r = 0; r < E; ++r) {
+      w[r] = word_select((w[r] < other[r]) == keep_min, w[r], other[r]);
+    }
+  }
+}
+template <int J, typename W>
 __device__ __forceinline__ void blocked_step(W (&w)[BLOCKED_E], uint32_t sub)
 {
   constexpr int E = BLOCKED_E;
@@ -109,16 +179,12 @@ __device__ __forceinline__ void blocked_step(W (&w)[BLOCKED_E], uint32_t sub)
 #pragma unroll
     for (int r = 0; r < E; ++r) {
       if ((r & J) == 0) {
-        // the run of K elements this pair belongs to ascends where bit K of the element number is clear
-        const bool ascending = (K == N) || (K < E ? (r & K) == 0 : (sub & (K / E)) == 0);
-        blocked_exchange_in_lane(w[r], w[r | J], ascending);
+        blocked_exchange_in_lane(w[r], w[r | J]);
       }
     }
   } else {
-    constexpr int D      = J / E;  // lane distance
-    const bool lower     = (sub & D) == 0;
-    const bool ascending = (K == N) || ((sub & (K / E)) == 0);
-    const bool keep_min  = lower == ascending;
+    constexpr int D     = J / E;  // lane distance
+    const bool keep_min = (sub & D) == 0;
 #pragma unroll
     for (int r = 0; r < E; ++r) {
       const W other = lane_xor<D>(w[r]);
@@ -126,24 +192,21 @@ __device__ __forceinline__ void blocked_step(W (&w)[BLOCKED_E], uint32_t sub)
     }
   }
 }
-template <int K, int J, int N, typename W>
+template <int J, typename W>
 __device__ __forceinline__ void blocked_merge(W (&w)[BLOCKED_E], uint32_t sub)
 {
   if constexpr (J >= 1) {
-    blocked_step<K, J, N>(w, sub);
-    if constexpr (J > 1) {
-      blocked_merge<K, J / 2, N>(w, sub);
-    }
+    blocked_step<J>(w, sub);
+    blocked_merge<J / 2>(w, sub);
   }
 }
 template <int K, int N, typename W>
 __device__ __forceinline__ void blocked_sort(W (&w)[BLOCKED_E], uint32_t sub)
 {
   if constexpr (K <= N) {
-    blocked_merge<K, K / 2, N>(w, sub);
-    if constexpr (K < N) {
-      blocked_sort<2 * K, N>(w, sub);
-    }
+    blocked_mirror_step<K>(w, sub);
+    blocked_merge<K / 4>(w, sub);
+    blocked_sort<2 * K, N>(w, sub);
   }
 }
 
@@ -239,6 +302,76 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
       if (row_exists && pos < seg) {
         raw[r] = s_row[pos];
       }
+    }
+  }
+  // A sort that returns values only, on keys whose image is a bijection of their bits (integers; floats when
+  // no row of the wavefront holds a NaN or a -0.0), sorts the bare images, one word per element, and maps
+  // them back: equal images are equal keys, so nothing has to tell them apart.
+  if constexpr (!HAS_IDX) {
+    bool bare = true;  // uniform over the wavefront
+    if constexpr (CODEC == CODEC_FLOAT) {
+      bool special = false;
+#pragma unroll
+      for (int r = 0; r < E; ++r) {
+        special |= row_exists && first + r < seg && is_nan_or_negative_zero(raw[r]);
+      }
+      bare = __ballot(special) == 0;
+    }
+    if (bare) {
+      using B = std::conditional_t<sizeof(KeyT) == 8, uint64_t, uint32_t>;
+      B b[E];
+#pragma unroll
+      for (int r = 0; r < E; ++r) {
+        const bool valid = row_exists && first + r < seg;
+        KeyT image;
+        if constexpr (CODEC == CODEC_FLOAT) {
+          image = sign_flip<KeyT>(raw[r]);
+        } else {
+          image = ordered_bits<CODEC, KeyT>(raw[r]);
+        }
+        b[r] = valid ? static_cast<B>(image) : static_cast<B>(~B{0});  // (slots past the end: behind or beside the largest key)
+      }
+      blocked_sort<2, N>(b, sub);
+      KeyT bits[E];
+#pragma unroll
+      for (int r = 0; r < E; ++r) {
+        const KeyT image = static_cast<KeyT>(b[r]);
+        if constexpr (CODEC == CODEC_FLOAT) {
+          bits[r] = sign_unflip<KeyT>(image);
+        } else {
+          bits[r] = ordered_bits<CODEC, KeyT>(image);  // (the identity, or the sign bit flipped back)
+        }
+      }
+      if (keys_out == nullptr) {
+        return;
+      }
+      if (vec_keys) {
+        if (row_exists) {
+          VecT q[VECS];
+          __builtin_memcpy(q, bits, LANE_BYTES);
+#pragma unroll
+          for (int v = 0; v < VECS; ++v) {
+            reinterpret_cast<VecT*>(keys_out + base + first)[v] = q[v];
+          }
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < E; ++r) {
+          const uint32_t pos = first + r;
+          if (row_exists && pos < seg) {
+            s_row[pos] = bits[r];  // (every lane has read its elements of the stretch; LDS operations of a wavefront execute in order)
+          }
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int k = 0; k < E; ++k) {
+          const uint32_t e = lane + k * WAVE;
+          if (e < stretch_len) {
+            keys_out[stretch_base + e] = s_wave[e];
+          }
+        }
+      }
+      return;
     }
   }
   W w[E];

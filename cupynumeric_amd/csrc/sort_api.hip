@@ -85,6 +85,27 @@ static std::atomic<int> g_bitonic_rows{[] {
 }()};
 
 bool bitonic_rows_enabled() { return g_bitonic_rows.load(std::memory_order_relaxed) != 0; }
+uint64_t bitonic_row_limit(int key_bytes, bool with_positions)
+{
+  static const uint64_t cap = [] {
+    const char* e = getenv("CPN_SORT_BITONIC_ROW_LIMIT");
+    return e != nullptr && *e != '\0' ? strtoull(e, nullptr, 10) : ~0ull;
+  }();
+  // Measured on 2^26 keys against the kernels that take over (network / other, ms).  Values only, where
+  // the network sorts bare images: float32 rows of 129 0.30 / 0.38, of 256 0.17 / 0.24, of 257 0.34 / 0.35,
+  // of 512 0.20 / 0.23; float16 rows of 129 0.32 / 0.38, of 256 0.14 / 0.21, of 257 0.36 / 0.30; float64
+  // rows of 129 0.53 / 0.50, of 256 0.31 / 0.32, of 257 0.63 / 0.40; int8 rows of 129 0.29 / 0.18, of 256
+  // 0.11 / 0.11.
+  uint64_t limit = 128;
+  if (with_positions) {
+    limit = key_bytes <= 2 ? 256 : 128;
+  } else if (key_bytes == 2) {
+    limit = 256;
+  } else if (key_bytes == 4) {
+    limit = 512;
+  }
+  return limit < cap ? limit : cap;
+}
 
 static std::atomic<long long> g_spin_limit{static_cast<long long>(LOOKBACK_SPIN_LIMIT)};
 

@@ -110,6 +110,9 @@ __host__ __device__ constexpr int key_passes(int key_bytes, int codec)
 // Rows of 2 ... 128 real keys go through the bitonic network (bitonic_row_sort.h)
 // unless CPN_SORT_BITONIC_ROWS=0 in the environment sends them to the ranking kernels (A/B runs).
 bool bitonic_rows_enabled();
+// Longest row that goes through the network, per key width and with or without positions; the environment
+// variable CPN_SORT_BITONIC_ROW_LIMIT lowers it (A/B runs).
+uint64_t bitonic_row_limit(int key_bytes, bool with_positions);
 
 // Row length up to which one wavefront (instead of one workgroup) sorts a row; at most 1024.
 // Changed by cpn_set_wave_row_limit / CPN_SORT_WAVE_ROW_LIMIT for A/B runs.
@@ -529,11 +532,15 @@ inline int sort_rows_in_lds(const SortRequest& r)
     // elements of its row that come before it (measured on 2^26 keys, counting / network: rows of 33 float32
     // keys 0.29 / 0.31 ms, of 40 0.33 / 0.28; float64 rows of 33 0.39 / 0.49, of 40 0.43 / 0.44; float16
     // rows of 33 0.20 / 0.23, of 40 0.22 / 0.20)
-    if (r.seg >= 33 && r.seg <= (sizeof(KeyT) == 8 ? 40u : 36u) && r.seg <= wave_row_limit() && bitonic_rows_enabled()) {
-      return launch_rank_rows<KeyT, CODEC, HAS_IDX>(r);
+    // (Values only, the network sorts bare images of 4- and 8-byte keys and is ahead there as well: float32
+    // rows of 36 keys 0.31 ms counted, rows of 37 0.19 through the network; float64 rows of 40 / 41 0.45 / 0.36.)
+    if constexpr (HAS_IDX || sizeof(KeyT) <= 2) {
+      if (r.seg >= 33 && r.seg <= (sizeof(KeyT) == 8 ? 40u : 36u) && r.seg <= wave_row_limit() && bitonic_rows_enabled()) {
+        return launch_rank_rows<KeyT, CODEC, HAS_IDX>(r);
+      }
     }
-    // rows of 2 ... 128 keys (256 for keys of 1 and 2 bytes): a bitonic network on eight elements per lane
-    if (r.seg >= 2 && r.seg <= (sizeof(KeyT) <= 2 ? 256u : 128u) && r.seg <= wave_row_limit() && bitonic_rows_enabled()) {
+    // rows of 2 ... 128 keys and more (bitonic_row_limit): a bitonic network on eight elements per lane
+    if (r.seg >= 2 && r.seg <= bitonic_row_limit(sizeof(KeyT), HAS_IDX) && r.seg <= wave_row_limit() && bitonic_rows_enabled()) {
       if (r.seg <= 8) {
         return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 8>(r);
       } else if (r.seg <= 16) {
@@ -544,8 +551,11 @@ inline int sort_rows_in_lds(const SortRequest& r)
         return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 64>(r);
       } else if (r.seg <= 128) {
         return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 128>(r);
-      } else {
+      } else if (r.seg <= 256) {
         return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 256>(r);
+      }
+      if constexpr (!HAS_IDX && sizeof(KeyT) == 4) {
+        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 512>(r);  // (a row per wavefront)
       }
     }
   }

@@ -274,6 +274,39 @@ def test_wave_rows_split_into_ranges(lib, torch_cuda, dtype):
     assert_same_bits(got_i, np.argsort(big, axis=-1, kind="stable"), f"{dt} many rows of 128, argsort")
 
 
+@pytest.mark.parametrize("dtype", [np.float16, np.float32, np.float64])
+def test_short_float_rows_without_nans_or_negative_zeros(lib, torch_cuda, dtype):
+    """Values-only sorts of short rows sort bare images of the keys when no row of a wavefront holds a NaN
+    or a -0.0: inputs with none of them at every row length, with infinities, the largest finite values
+    and +0.0 (the images next to the one that padding slots hold), in place and out of place; then many rows
+    of which a few hold a NaN or a -0.0, so that wavefronts of both kinds run in one launch."""
+    dt = np.dtype(dtype)
+    rng = np.random.default_rng(dt.num * 17 + 3)
+    for seg in list(range(2, 70)) + [95, 96, 100, 127, 128, 129, 200, 255, 256]:
+        rows = 1 + (seg * 5) % 19 if seg % 3 else 150 + seg
+        x = rng.standard_normal((rows, seg)).astype(dtype)
+        x[0] = x[0, 0]
+        if rows > 3:
+            x[1, ::2] = np.inf
+            x[1, 1::4] = -np.inf
+            x[2, ::3] = np.finfo(dtype).max
+            x[2, 1::3] = 0.0
+            x[3] = np.sort(x[3])[::-1]
+        want = np.sort(x, axis=-1, kind="stable")
+        got, _ = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=False)
+        assert_same_bits(got, want, f"{dt} seg={seg} clean rows")
+        if seg in (2, 7, 8, 33, 64, 100, 128, 256):
+            got, _ = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=False, in_place=True)
+            assert_same_bits(got, want, f"{dt} seg={seg} clean rows, in place")
+    for seg in (8, 24, 64, 128):
+        x = rng.standard_normal((30000, seg)).astype(dtype)
+        x[::97, 1] = np.nan
+        x[5::211, 0] = -0.0
+        x[7::211, seg - 1] = 0.0
+        got, _ = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=False)
+        assert_same_bits(got, np.sort(x, axis=-1, kind="stable"), f"{dt} seg={seg} rows with and without special values")
+
+
 REAL_DTYPES = [np.bool_, np.int8, np.uint8, np.int16, np.uint16, np.float16, np.int32, np.uint32, np.float32,
                np.int64, np.uint64, np.float64]
 
