@@ -99,7 +99,7 @@ uint64_t bitonic_row_limit(int key_bytes, bool with_positions)
   uint64_t limit = 128;
   if (with_positions) {
     limit = key_bytes <= 2 ? 256 : 128;
-  } else if (key_bytes == 2) {
+  } else if (key_bytes == 2 || key_bytes == 8) {
     limit = 256;
   } else if (key_bytes == 4) {
     limit = 512;

@@ -470,12 +470,13 @@ inline int launch_wave_rows(const SortRequest& r)
 template <typename KeyT, int CODEC, bool HAS_IDX, int N>
 inline int launch_bitonic_rows(const SortRequest& r)
 {
+  constexpr int E               = blocked_elements(sizeof(KeyT), HAS_IDX, N);
   const uint64_t rows           = r.volume / r.seg;
-  const uint64_t rows_per_block = (256 / WAVE) * (BLOCKED_E * WAVE / N);
+  const uint64_t rows_per_block = (256 / WAVE) * (E * WAVE / N);
   const uint64_t blocks         = (rows + rows_per_block - 1) / rows_per_block;
   {
     ProfileScope prof("bitonic_row_sort", r.stream);
-    hipLaunchKernelGGL((bitonic_row_sort_kernel<KeyT, CODEC, HAS_IDX, N>), dim3(static_cast<uint32_t>(blocks)),
+    hipLaunchKernelGGL((bitonic_row_sort_kernel<KeyT, CODEC, HAS_IDX, N, E>), dim3(static_cast<uint32_t>(blocks)),
                        dim3(256), 0, r.stream, static_cast<const KeyT*>(r.values_in), static_cast<KeyT*>(r.values_out),
                        r.indices_out, static_cast<uint32_t>(r.seg), rows, r.index_offset, static_cast<uint32_t*>(r.temp));
   }
