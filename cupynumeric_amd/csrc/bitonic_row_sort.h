@@ -10,8 +10,9 @@
 // What is compared: a sort that returns values only, on keys whose image is a bijection of their bits
 // (integers; floats when no row of the wavefront holds a NaN or a -0.0), sorts the bare images and maps
 // them back (2^26 float32 keys in rows of 128 0.11 ms, of 32 0.09: the speed of the memory).  Otherwise
-// the words are (order-preserving image of the key, position in the row) as one unsigned word (an image
-// and a position word for 8-byte keys), so that no two are equal: the network, which is not stable by
+// the words are (order-preserving image of the key, position in the row) as one word (32 bits for 1- and
+// 2-byte keys; for 4-byte keys a double whose mantissa holds both; an image and a position word for 8-byte
+// keys), so that no two are equal: the network, which is not stable by
 // itself, then yields exactly the stable order (NaNs tie with each other and +0.0 with -0.0 in the image,
 // and the position decides); the raw keys do not travel: they wait in LDS, and every lane fetches the
 // keys of the positions that ended up in its slots once, at the end (rows of 128 float32 keys 0.22 ms,
@@ -102,6 +103,14 @@ __device__ __forceinline__ F64Word lane_xor(F64Word w)
   return F64Word{__longlong_as_double(static_cast<long long>(lane_xor<J>(static_cast<uint64_t>(__double_as_longlong(w.v)))))};
 }
 __device__ __forceinline__ F64Word word_select(bool first, const F64Word& a, const F64Word& b) { return F64Word{first ? a.v : b.v}; }
+// (image of a 4-byte key, position in the row) as a number: the 52 bits image << 20 | position are the
+// mantissa of a double of the fixed exponent 2^52, so the numbers order as the pairs do and are all finite.
+__device__ __forceinline__ F64Word pack_image_pos(uint32_t image, uint32_t pos)
+{
+  const uint64_t bits = 0x4330000000000000ull | (static_cast<uint64_t>(image) << 20) | pos;
+  return F64Word{__longlong_as_double(static_cast<long long>(bits))};
+}
+__device__ __forceinline__ uint32_t word_pos(const F64Word& w) { return static_cast<uint32_t>(__double_as_longlong(w.v)) & 0xFFFFFu; }
 
 // Elements per lane: eight, or sixteen where a sort returns values only of 8-byte keys (fewer of the steps
 // cross lanes: 6 instead of 10 of the 28 steps of a row of 128 keys.  2^26 float64 keys in rows of 32 0.29 ->
@@ -266,12 +275,12 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
   }
   // 4-byte keys: image in the high word, position in the low one; shorter keys: image << 16 | position;
   // 8-byte keys: two registers for the image, one for the position
-  using W = std::conditional_t<sizeof(KeyT) == 8, ImagePos, std::conditional_t<sizeof(KeyT) == 4, uint64_t, uint32_t>>;
+  using W = std::conditional_t<sizeof(KeyT) == 8, ImagePos, std::conditional_t<sizeof(KeyT) == 4, F64Word, uint32_t>>;
   constexpr int LANES     = N / E;  // lanes per row
   constexpr int ROWS_WAVE = WAVE / LANES;
   constexpr int WAVES     = 256 / WAVE;
   __shared__ __align__(16) KeyT s_raw[256 * E];
-  __shared__ uint16_t s_from[HAS_IDX ? 256 * E : 1];
+  __shared__ __align__(16) uint16_t s_from[HAS_IDX ? 256 * E : 8];
 
   const uint32_t lane   = threadIdx.x & (WAVE - 1);
   const uint32_t wslot  = threadIdx.x / WAVE;
@@ -302,12 +311,13 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
   KeyT* const s_wave          = s_raw + wslot * (WAVE * E);
   KeyT* const s_row           = s_wave + wrow * seg;  // this lane's row inside the stretch
 
-  // Sixteen elements per lane are 64 or 128 bytes: lanes that fetched their own elements straight from memory
-  // would touch twice the cache lines per instruction that lanes with 32 bytes do (measured: rows of 32
-  // float32 keys 0.135 ms against 0.09).  So the wavefront moves its stretch in 16-byte pieces, neighbouring
-  // lanes on neighbouring pieces, and the pieces change hands in LDS: piece q lies at q ^ ((q >> 3) & 7), which
-  // keeps eight neighbouring pieces, and the pieces that eight neighbouring lanes own, in different banks.
-  constexpr bool VIA_LDS      = E == 16;
+  // Lanes that own 64 bytes or more (8-byte keys; sixteen elements) and fetched them straight from memory would
+  // touch a cache line of their own with every instruction (measured with 64 bytes of float32 keys per lane:
+  // rows of 32 keys 0.135 ms against 0.09 with 32 bytes).  So the wavefront moves its stretch in 16-byte
+  // pieces, neighbouring lanes on neighbouring pieces, and the pieces change hands in LDS: piece q lies at
+  // q ^ ((q >> 3) & 7), which keeps eight neighbouring pieces, and the pieces that eight neighbouring lanes
+  // own, in different banks.
+  constexpr bool VIA_LDS      = LANE_BYTES >= 64;
   constexpr int PIECE_KEYS    = 16 / static_cast<int>(sizeof(KeyT));
   constexpr int PIECES        = VIA_LDS ? LANE_BYTES / 16 : 1;  // per lane
   uint4* const s_pieces       = reinterpret_cast<uint4*>(s_wave);
@@ -490,7 +500,11 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
     if constexpr (sizeof(KeyT) == 8) {
       w[r] = ImagePos{image, pos};
     } else {
-      w[r] = (static_cast<W>(image) << (sizeof(KeyT) == 4 ? 32 : 16)) | pos;
+      if constexpr (sizeof(KeyT) == 4) {
+        w[r] = pack_image_pos(image, pos);
+      } else {
+        w[r] = (static_cast<W>(image) << 16) | pos;
+      }
     }
   }
   blocked_sort<2, N>(w, sub);
@@ -545,17 +559,33 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
   }
   if constexpr (HAS_IDX) {
     if (vec_idx) {
-      if (row_exists) {
-        int64_t out[E];
+      // The positions change hands in LDS as 16-bit words, so that a lane stores two neighbouring int64 words
+      // and its neighbours the next ones: a lane that stored the 64 bytes of its own eight slots would touch
+      // a cache line of its own with every instruction (2^21 rows of 128 float32 keys: 0.79 ms that way).
+      uint16_t* const s_fwave = s_from + wslot * (WAVE * E);
+      uint16_t mine[E];
 #pragma unroll
-        for (int r = 0; r < E; ++r) {
-          out[r] = static_cast<int64_t>(from[r]) + index_offset;
-        }
-        uint4 q[E / 2];
-        __builtin_memcpy(q, out, sizeof(out));
+      for (int r = 0; r < E; ++r) {
+        mine[r] = static_cast<uint16_t>(from[r]);
+      }
+      uint4 packed[E / 8];
+      __builtin_memcpy(packed, mine, sizeof(mine));
 #pragma unroll
-        for (int v = 0; v < E / 2; ++v) {
-          reinterpret_cast<uint4*>(idx_out + base + first)[v] = q[v];
+      for (int v = 0; v < E / 8; ++v) {
+        reinterpret_cast<uint4*>(s_fwave)[lane * (E / 8) + v] = packed[v];
+      }
+      __builtin_amdgcn_wave_barrier();
+      uint4* const dst = reinterpret_cast<uint4*>(idx_out + stretch_base);
+#pragma unroll
+      for (int k = 0; k < E / 2; ++k) {
+        const uint32_t q = k * WAVE + lane;  // slots 2 q and 2 q + 1 of the stretch
+        if (2 * q < stretch_len) {
+          const uint32_t pair = reinterpret_cast<const uint32_t*>(s_fwave)[q];
+          const int64_t out[2] = {static_cast<int64_t>(pair & 0xFFFFu) + index_offset,
+                                  static_cast<int64_t>(pair >> 16) + index_offset};
+          uint4 word;
+          __builtin_memcpy(&word, out, sizeof(word));
+          dst[q] = word;
         }
       }
     } else {
