@@ -95,10 +95,11 @@ uint64_t bitonic_row_limit(int key_bytes, bool with_positions)
   // the network sorts bare images: float32 rows of 129 0.30 / 0.38, of 256 0.17 / 0.24, of 257 0.34 / 0.35,
   // of 512 0.20 / 0.23; float16 rows of 129 0.32 / 0.38, of 256 0.14 / 0.21, of 257 0.36 / 0.30; float64
   // rows of 129 0.53 / 0.50, of 256 0.31 / 0.32, of 257 0.63 / 0.40; int8 rows of 129 0.29 / 0.18, of 256
-  // 0.11 / 0.11.
+  // 0.11 / 0.11.  With positions: float32 rows of 129 0.39 / 0.46, of 256 0.23 / 0.31; int32 0.37 / 0.42 and
+  // 0.21 / 0.27.
   uint64_t limit = 128;
   if (with_positions) {
-    limit = key_bytes <= 2 ? 256 : 128;
+    limit = key_bytes <= 4 ? 256 : 128;
   } else if (key_bytes == 2 || key_bytes == 8) {
     limit = 256;
   } else if (key_bytes == 4) {
