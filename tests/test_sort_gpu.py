@@ -307,6 +307,49 @@ def test_short_float_rows_without_nans_or_negative_zeros(lib, torch_cuda, dtype)
         assert_same_bits(got, np.sort(x, axis=-1, kind="stable"), f"{dt} seg={seg} rows with and without special values")
 
 
+@pytest.mark.parametrize("dtype", [np.uint8, np.float16, np.int32, np.float32, np.int64, np.float64])
+def test_short_rows_at_pointers_that_are_not_16_byte_aligned(lib, torch_cuda, dtype):
+    """Full rows are moved as 16-byte vectors only when the buffers allow it: the same sorts with input,
+    output and index buffers that start 1 ... 3 elements into an allocation, with a guard word on either
+    side of the index buffer."""
+    torch = torch_cuda
+    dt = np.dtype(dtype)
+    rng = np.random.default_rng(dt.num + 77)
+    word = {1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}[dt.itemsize]
+    np_word = {1: np.uint8, 2: np.int16, 4: np.int32, 8: np.int64}[dt.itemsize]
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for seg, rows, offs in ((8, 1000, (1, 2, 3)), (32, 777, (3, 0, 1)), (64, 300, (0, 1, 0)), (128, 513, (2, 2, 1)),
+                            (256, 100, (1, 3, 3)), (512, 65, (3, 1, 2)), (100, 400, (1, 1, 1))):
+        if dt.kind == "f":
+            x = rng.standard_normal((rows, seg)).astype(dtype)
+            x[::7, 0] = np.nan
+            x[3::11, seg - 1] = -0.0
+        else:
+            x = rng.integers(np.iinfo(dtype).min, np.iinfo(dtype).max, (rows, seg), endpoint=True, dtype=dtype)
+        n = x.size
+        order = np.argsort(x.astype(np.float32) if dt == np.float16 else x, axis=-1, kind="stable")
+        for want_values, want_indices in ((True, False), (False, True), (True, True)):
+            d_in = torch.zeros(n + 8, dtype=word, device="cuda")
+            d_in[offs[0]:offs[0] + n] = torch.from_numpy(x.reshape(-1).view(np_word).copy()).cuda()
+            d_out = torch.zeros(n + 8, dtype=word, device="cuda")
+            d_idx = torch.full((n + 8,), -7, dtype=torch.int64, device="cuda")
+            tb = lib.cpn_local_sort_temp_bytes(_lib.DTYPE_CODES[dt], n, seg, int(want_values), int(want_indices), 0)
+            temp = torch.full((tb,), 0xFF, dtype=torch.uint8, device="cuda")
+            rc = lib.cpn_local_sort(_lib.DTYPE_CODES[dt], d_in.data_ptr() + offs[0] * dt.itemsize,
+                                    d_out.data_ptr() + offs[1] * dt.itemsize if want_values else None,
+                                    d_idx.data_ptr() + offs[2] * 8 if want_indices else None, n, seg, 0, 1,
+                                    temp.data_ptr(), tb, stream)
+            assert rc == 0, _lib.status_string(rc)
+            where = f"{dt} rows of {seg}, offsets {offs}, values={want_values}, indices={want_indices}"
+            if want_values:
+                got = d_out[offs[1]:offs[1] + n].cpu().numpy().view(dtype).reshape(rows, seg)
+                assert_same_bits(got, np.take_along_axis(x, order, axis=-1), where)
+            if want_indices:
+                got = d_idx.cpu().numpy()
+                assert np.array_equal(got[offs[2]:offs[2] + n].reshape(rows, seg), order), where
+                assert (got[:offs[2]] == -7).all() and (got[offs[2] + n:] == -7).all(), where + ": wrote outside the index buffer"
+
+
 REAL_DTYPES = [np.bool_, np.int8, np.uint8, np.int16, np.uint16, np.float16, np.int32, np.uint32, np.float32,
                np.int64, np.uint64, np.float64]
 
