@@ -127,11 +127,11 @@ def make_config(name: str, log2n: int | None = None, rows: int | None = None) ->
 # Row lengths on either side of every length at which the library changes kernels (--edges): key type,
 # operation, lengths whose successor is timed too; 2^26 keys per run.
 EDGE_LENGTHS = (
-    ("float32", "sort", (32, 36, 64, 128, 256, 512, 768, 1024, 1536, 2048, 3072, 4096, 6144, 8192, 12288, 16384, 32768, 65536)),
-    ("float64", "sort", (32, 40, 64, 128, 256, 512, 768, 1024, 1536, 2048, 3072, 4096, 6144, 8192, 16384, 32768, 65536, 1048576)),
-    ("float16", "sort", (32, 36, 64, 128, 256, 4096, 8192, 16384, 32768)),
-    ("float32", "argsort", (32, 36, 64, 128, 256, 512, 2048, 4096, 6144, 8192, 16384, 32768, 65536)),
-    ("float64", "argsort", (32, 40, 64, 128, 256, 512, 2048, 4096, 6144, 8192, 14336, 28672, 57344, 458752)),
+    ("float32", "sort", (32, 40, 64, 96, 128, 256, 512, 768, 1024, 1536, 2048, 3072, 4096, 6144, 8192, 12288, 16384, 32768, 65536)),
+    ("float64", "sort", (32, 40, 64, 96, 128, 256, 512, 768, 1024, 1536, 2048, 3072, 4096, 6144, 8192, 16384, 32768, 65536, 1048576)),
+    ("float16", "sort", (32, 40, 64, 96, 128, 256, 4096, 8192, 16384, 32768)),
+    ("float32", "argsort", (32, 40, 64, 96, 128, 256, 512, 2048, 4096, 6144, 8192, 16384, 32768, 65536)),
+    ("float64", "argsort", (32, 40, 64, 96, 128, 256, 512, 2048, 4096, 6144, 8192, 14336, 28672, 57344, 458752)),
 )
 
 
@@ -722,7 +722,7 @@ def run_consumer(args) -> dict:
 
 
 # -------------------------------------------------------------------------------------------------
-ROW_KERNELS = ("bitonic_row_sort", "rank_row_sort", "tiny_row_sort", "wave_row_sort", "lds_row_sort", "count16_row_sort")
+ROW_KERNELS = ("bitonic_row_sort", "tiny_row_sort", "wave_row_sort", "lds_row_sort", "count16_row_sort")
 
 
 def verify_result(job: GpuJob, cfg: dict) -> str:

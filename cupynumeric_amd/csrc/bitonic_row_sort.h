@@ -112,16 +112,12 @@ __device__ __forceinline__ F64Word pack_image_pos(uint32_t image, uint32_t pos)
 }
 __device__ __forceinline__ uint32_t word_pos(const F64Word& w) { return static_cast<uint32_t>(__double_as_longlong(w.v)) & 0xFFFFFu; }
 
-// Elements per lane: eight, or sixteen where a sort returns values only of 8-byte keys (fewer of the steps
-// cross lanes: 6 instead of 10 of the 28 steps of a row of 128 keys.  2^26 float64 keys in rows of 32 0.29 ->
-// 0.19 ms, of 128 0.31 -> 0.23; int64 0.21 and 0.27.  Plain sorts of 4-byte keys, which already move at the
-// speed of the memory with eight, lose to the hand-over in LDS that sixteen need: rows of 128 float32 keys 0.11 ->
-// 0.14 ms.)
+// Elements per lane: eight for full rows (five to seven for rows in between, see the network below), or
+// sixteen where a sort returns values only of full rows of 8-byte keys (fewer of the steps cross lanes: 6
+// instead of 10 of the 28 steps of a row of 128 keys.  2^26 float64 keys in rows of 32 0.29 -> 0.19 ms, of 128
+// 0.31 -> 0.23; int64 0.21 and 0.27.  Plain sorts of 4-byte keys, which already move at the speed of the
+// memory with eight, lose to the hand-over in LDS that sixteen need: rows of 128 float32 keys 0.11 -> 0.14 ms.)
 constexpr int BLOCKED_E = 8;
-__host__ __device__ constexpr int blocked_elements(int key_bytes, bool with_positions, int slots)
-{
-  return (!with_positions && key_bytes == 8 && slots >= 32) ? 16 : BLOCKED_E;
-}
 
 // a < b on the words of the network.  (For 64-bit words the borrow of a subtraction and a compare of the
 // halves were measured against the plain compare: the same and 10 % slower on rows of 128 keys.)
@@ -187,14 +183,37 @@ __device__ __forceinline__ void blocked_exchange_in_lane(W& lo, W& hi)
   }
 }
 
-// The network is the bitonic sorter in the form whose comparators all point the same way: the merge of two
-// sorted runs of K / 2 elements starts by comparing element i with its mirror image i ^ (K - 1) in the run
-// of K, and goes on with the partners i ^ J for J = K / 4 ... 1; the smaller word always goes to the
-// smaller element number, so no step has to know which way its run points.  Element i of a row is register
-// i % 8 of lane i / 8: partners closer than 8 elements are registers of one lane, and a mirror image across
-// lanes is register 7 - r of the mirrored lane.  `sub` is the lane's number inside its row.
+// The network.  A lane first sorts its own E elements; then, level by level, the sorted runs of 1, 2, 4 ...
+// lanes are merged in pairs: a merge starts by comparing every element with its mirror image in the run of
+// both (register E - 1 - r of the mirrored lane), goes on with the same register of the lanes at distance
+// KL / 4 ... 1, and ends inside the lanes, whose elements are a bitonic sequence by then.  The smaller word
+// always goes to the smaller element number, so no step has to know which way its run points.  For E = 8 and
+// 16 this is the bitonic sorter (its comparators all pointing the same way); E = 5, 6, 7 use the smallest
+// known networks of 9, 12 and 16 exchanges inside a lane (a bitonic sequence of 6: a half-cleaner and two
+// networks of 3), which lets a row of n keys take 8, 16, 32 or 64 lanes of ceil(n / lanes) elements each
+// instead of the next power of two of slots.  `sub` is the lane's number inside its row.
+template <int A, int B, typename W, int E>
+__device__ __forceinline__ void lane_exchange(W (&w)[E])
+{
+  static_assert(A < B && B < E, "the smaller word goes to the smaller element number");
+  blocked_exchange_in_lane(w[A], w[B]);
+}
+// The steps (i, i | J) for J = J0, J0 / 2 ... 1: sorts a bitonic sequence of a power of two of elements.
+template <int J, typename W, int E>
+__device__ __forceinline__ void lane_half_cleaners(W (&w)[E])
+{
+  if constexpr (J >= 1) {
+#pragma unroll
+    for (int r = 0; r < E; ++r) {
+      if ((r & J) == 0) {
+        blocked_exchange_in_lane(w[r], w[r | J]);
+      }
+    }
+    lane_half_cleaners<J / 2>(w);
+  }
+}
 template <int K, typename W, int E>
-__device__ __forceinline__ void blocked_mirror_step(W (&w)[E], uint32_t sub)
+__device__ __forceinline__ void lane_bitonic_levels(W (&w)[E])
 {
   if constexpr (K <= E) {
 #pragma unroll
@@ -203,61 +222,103 @@ __device__ __forceinline__ void blocked_mirror_step(W (&w)[E], uint32_t sub)
         blocked_exchange_in_lane(w[r], w[r ^ (K - 1)]);
       }
     }
-  } else {
-    constexpr int M     = K / E - 1;                  // lane ^ M: the mirrored lane
-    const bool keep_min = (sub & ((M + 1) / 2)) == 0;  // the lower half of the run keeps the smaller words
-    W other[E];
-#pragma unroll
-    for (int r = 0; r < E; ++r) {
-      other[r] = lane_mirror<M>(w[E - 1 - r]);
-    }
-#pragma unroll
-    for (int r = 0; r < E; ++r) {
-      w[r] = word_select(word_less(w[r], other[r]) == keep_min, w[r], other[r]);
-    }
+    lane_half_cleaners<K / 4>(w);
+    lane_bitonic_levels<2 * K>(w);
   }
 }
-template <int J, typename W, int E>
-__device__ __forceinline__ void blocked_step(W (&w)[E], uint32_t sub)
+// Sorts the E elements of a lane, whatever their order.
+template <typename W, int E>
+__device__ __forceinline__ void lane_sort(W (&w)[E])
 {
-  if constexpr (J < E) {
-#pragma unroll
-    for (int r = 0; r < E; ++r) {
-      if ((r & J) == 0) {
-        blocked_exchange_in_lane(w[r], w[r | J]);
-      }
-    }
+  if constexpr (E == 3) {
+    lane_exchange<0, 2>(w), lane_exchange<0, 1>(w), lane_exchange<1, 2>(w);
+  } else if constexpr (E == 5) {
+    lane_exchange<0, 3>(w), lane_exchange<1, 4>(w);
+    lane_exchange<0, 2>(w), lane_exchange<1, 3>(w);
+    lane_exchange<0, 1>(w), lane_exchange<2, 4>(w);
+    lane_exchange<1, 2>(w), lane_exchange<3, 4>(w);
+    lane_exchange<2, 3>(w);
+  } else if constexpr (E == 6) {
+    lane_exchange<0, 5>(w), lane_exchange<1, 3>(w), lane_exchange<2, 4>(w);
+    lane_exchange<1, 2>(w), lane_exchange<3, 4>(w);
+    lane_exchange<0, 3>(w), lane_exchange<2, 5>(w);
+    lane_exchange<0, 1>(w), lane_exchange<2, 3>(w), lane_exchange<4, 5>(w);
+    lane_exchange<1, 2>(w), lane_exchange<3, 4>(w);
+  } else if constexpr (E == 7) {
+    lane_exchange<0, 6>(w), lane_exchange<2, 3>(w), lane_exchange<4, 5>(w);
+    lane_exchange<0, 2>(w), lane_exchange<1, 4>(w), lane_exchange<3, 6>(w);
+    lane_exchange<0, 1>(w), lane_exchange<2, 5>(w), lane_exchange<3, 4>(w);
+    lane_exchange<1, 2>(w), lane_exchange<4, 6>(w);
+    lane_exchange<2, 3>(w), lane_exchange<4, 5>(w);
+    lane_exchange<1, 2>(w), lane_exchange<3, 4>(w), lane_exchange<5, 6>(w);
   } else {
-    constexpr int D     = J / E;  // lane distance
+    static_assert((E & (E - 1)) == 0, "a power of two of elements: the bitonic sorter");
+    lane_bitonic_levels<2>(w);
+  }
+}
+// Sorts the E elements of a lane that form a bitonic sequence.
+template <typename W, int E>
+__device__ __forceinline__ void lane_sort_bitonic(W (&w)[E])
+{
+  if constexpr ((E & (E - 1)) == 0) {
+    lane_half_cleaners<E / 2>(w);
+  } else if constexpr (E == 6) {
+    lane_exchange<0, 3>(w), lane_exchange<1, 4>(w), lane_exchange<2, 5>(w);
+    lane_exchange<0, 2>(w), lane_exchange<0, 1>(w), lane_exchange<1, 2>(w);
+    lane_exchange<3, 5>(w), lane_exchange<3, 4>(w), lane_exchange<4, 5>(w);
+  } else {
+    lane_sort(w);
+  }
+}
+// The steps of a merge that cross lanes: the mirror image in the run of KL lanes, then the lanes at distance D.
+template <int KL, typename W, int E>
+__device__ __forceinline__ void cross_mirror(W (&w)[E], uint32_t sub)
+{
+  const bool keep_min = (sub & (KL / 2)) == 0;  // the lower half of the run keeps the smaller words
+  W other[E];
+#pragma unroll
+  for (int r = 0; r < E; ++r) {
+    other[r] = lane_mirror<KL - 1>(w[E - 1 - r]);
+  }
+#pragma unroll
+  for (int r = 0; r < E; ++r) {
+    w[r] = word_select(word_less(w[r], other[r]) == keep_min, w[r], other[r]);
+  }
+}
+template <int D, typename W, int E>
+__device__ __forceinline__ void cross_steps(W (&w)[E], uint32_t sub)
+{
+  if constexpr (D >= 1) {
     const bool keep_min = (sub & D) == 0;
 #pragma unroll
     for (int r = 0; r < E; ++r) {
       const W other = lane_xor<D>(w[r]);
       w[r]          = word_select(word_less(w[r], other) == keep_min, w[r], other);
     }
+    cross_steps<D / 2>(w, sub);
   }
 }
-template <int J, typename W, int E>
-__device__ __forceinline__ void blocked_merge(W (&w)[E], uint32_t sub)
+template <int KL, int LANES, typename W, int E>
+__device__ __forceinline__ void merge_levels(W (&w)[E], uint32_t sub)
 {
-  if constexpr (J >= 1) {
-    blocked_step<J>(w, sub);
-    blocked_merge<J / 2>(w, sub);
+  if constexpr (KL <= LANES) {
+    cross_mirror<KL>(w, sub);
+    cross_steps<KL / 4>(w, sub);
+    lane_sort_bitonic(w);
+    merge_levels<2 * KL, LANES>(w, sub);
   }
 }
-template <int K, int N, typename W, int E>
+// A row of LANES x E slots.
+template <int LANES, typename W, int E>
 __device__ __forceinline__ void blocked_sort(W (&w)[E], uint32_t sub)
 {
-  if constexpr (K <= N) {
-    blocked_mirror_step<K>(w, sub);
-    blocked_merge<K / 4>(w, sub);
-    blocked_sort<2 * K, N>(w, sub);
-  }
+  lane_sort(w);
+  merge_levels<2, LANES>(w, sub);
 }
 
-// N = slots per row (8 ... 512, a power of two, >= row length), E = elements per lane; N / E lanes per row,
-// 64 E / N rows per wavefront, four wavefronts per workgroup.
-template <typename KeyT, int CODEC, bool HAS_IDX, int N, int E>
+// LANES = lanes per row (a power of two), E = elements per lane: LANES x E slots per row (>= row length),
+// 64 / LANES rows per wavefront, four wavefronts per workgroup.
+template <typename KeyT, int CODEC, bool HAS_IDX, int LANES, int E>
 __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __restrict__ keys_in,
                                                                         KeyT* keys_out,
                                                                         int64_t* __restrict__ idx_out,
@@ -268,22 +329,29 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
 {
   static_assert(sizeof(KeyT) <= 8 && (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT),
                 "real keys of up to 8 bytes");
-  static_assert(E == 8 || E == 16, "elements per lane");
-  static_assert(N >= E && N <= E * WAVE && (N & (N - 1)) == 0, "slots per row: a power of two from E to 64 E");
+  static_assert((E >= 5 && E <= 8) || E == 16, "elements per lane");
+  static_assert(LANES >= 1 && LANES <= WAVE && (LANES & (LANES - 1)) == 0, "lanes per row: a power of two");
+  constexpr int N = LANES * E;  // slots per row
   if (blockIdx.x == 0 && threadIdx.x == 0) {
     *status = 0;  // the workspace's status word: a per-row sort cannot fail on the device
   }
   // 4-byte keys: image in the high word, position in the low one; shorter keys: image << 16 | position;
   // 8-byte keys: two registers for the image, one for the position
   using W = std::conditional_t<sizeof(KeyT) == 8, ImagePos, std::conditional_t<sizeof(KeyT) == 4, F64Word, uint32_t>>;
-  constexpr int LANES     = N / E;  // lanes per row
   constexpr int ROWS_WAVE = WAVE / LANES;
   constexpr int WAVES     = 256 / WAVE;
-  __shared__ __align__(16) KeyT s_raw[256 * E];
+  // The stretch of a wavefront in LDS, as it lies in memory.  (A word of padding after every 32, so that lanes
+  // whose elements start 8 elements apart do not meet in four banks, was measured and changed nothing: what the
+  // rows that go through here pay for is instructions, 94 per key against 68 for rows moved as vectors before
+  // the addresses below were made uniform.)
+  constexpr int WAVE_SLOTS = WAVE * E;
+  __shared__ __align__(16) KeyT s_raw[(256 / WAVE) * WAVE_SLOTS];
   __shared__ __align__(16) uint16_t s_from[HAS_IDX ? 256 * E : 8];
 
   const uint32_t lane   = threadIdx.x & (WAVE - 1);
-  const uint32_t wslot  = threadIdx.x / WAVE;
+  // (the number of the wavefront, read from its first lane so that the compiler knows that everything derived
+  // from it is the same in all lanes: the addresses of the stretch then need no vector arithmetic)
+  const uint32_t wslot  = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x / WAVE)));
   const uint64_t wave   = static_cast<uint64_t>(blockIdx.x) * WAVES + wslot;
   const uint32_t sub    = lane & (LANES - 1);
   const uint32_t wrow   = lane / LANES;  // row of this lane inside its wavefront
@@ -291,25 +359,28 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
   const uint64_t base   = row * seg;
   const uint32_t first  = sub * E;  // position of this lane's first element in its row
   const bool row_exists = row < rows;
+  const uint32_t row_len = row_exists ? seg : 0u;  // slots of this lane's row that hold keys
 
   // Full rows whose lanes' eight elements can be moved as 16-byte (single bytes: 8-byte) vectors: a wavefront
   // then reads and writes whole contiguous kilobytes per instruction.  Other rows go through LDS: the rows of
   // a wavefront are one contiguous stretch of memory, which its lanes copy in and out element by element,
   // neighbouring lanes on neighbouring elements, and from which every lane takes the eight elements it owns.
   constexpr int LANE_BYTES = E * static_cast<int>(sizeof(KeyT));
+  constexpr bool CAN_VEC   = E == 8 || E == 16;  // (other lanes own a number of bytes that is no whole vector)
   using VecT               = std::conditional_t<(LANE_BYTES >= 16), uint4, uint2>;
-  constexpr int VECS       = LANE_BYTES / static_cast<int>(sizeof(VecT));
-  const bool vec_keys = (seg == N) && ((reinterpret_cast<uintptr_t>(keys_in) | reinterpret_cast<uintptr_t>(keys_out)) &
+  constexpr int VECS       = CAN_VEC ? LANE_BYTES / static_cast<int>(sizeof(VecT)) : 1;
+  const bool vec_keys = CAN_VEC && (seg == N) && ((reinterpret_cast<uintptr_t>(keys_in) | reinterpret_cast<uintptr_t>(keys_out)) &
                                        (sizeof(VecT) - 1)) == 0;  // uniform
-  const bool vec_idx  = (seg == N) && (reinterpret_cast<uintptr_t>(idx_out) & 15u) == 0;
+  const bool vec_idx  = CAN_VEC && (seg == N) && (reinterpret_cast<uintptr_t>(idx_out) & 15u) == 0;
   // the stretch of this wavefront: its rows, densely, as in memory
   const uint64_t wave_row0 = wave * ROWS_WAVE;
   const uint32_t wave_rows =
     wave_row0 >= rows ? 0u : static_cast<uint32_t>(rows - wave_row0 < ROWS_WAVE ? rows - wave_row0 : ROWS_WAVE);
   const uint32_t stretch_len  = wave_rows * seg;  // at most 512 elements
   const uint64_t stretch_base = wave_row0 * seg;
-  KeyT* const s_wave          = s_raw + wslot * (WAVE * E);
-  KeyT* const s_row           = s_wave + wrow * seg;  // this lane's row inside the stretch
+  KeyT* const s_wave          = s_raw + wslot * WAVE_SLOTS;
+  KeyT* const dst_keys        = keys_out + stretch_base;  // (used where keys_out is not null)
+  const uint32_t row_at       = wrow * seg;  // this lane's row inside the stretch
 
   // Lanes that own 64 bytes or more (8-byte keys; sixteen elements) and fetched them straight from memory would
   // touch a cache line of their own with every instruction (measured with 64 bytes of float32 keys per lane:
@@ -317,14 +388,16 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
   // pieces, neighbouring lanes on neighbouring pieces, and the pieces change hands in LDS: piece q lies at
   // q ^ ((q >> 3) & 7), which keeps eight neighbouring pieces, and the pieces that eight neighbouring lanes
   // own, in different banks.
-  constexpr bool VIA_LDS      = LANE_BYTES >= 64;
+  constexpr bool VIA_LDS      = CAN_VEC && LANE_BYTES >= 64;
   constexpr int PIECE_KEYS    = 16 / static_cast<int>(sizeof(KeyT));
   constexpr int PIECES        = VIA_LDS ? LANE_BYTES / 16 : 1;  // per lane
   uint4* const s_pieces       = reinterpret_cast<uint4*>(s_wave);
   const uint32_t stretch_pieces = stretch_len / PIECE_KEYS;
   auto piece_slot = [](uint32_t q) { return q ^ ((q >> 3) & 7u); };
   auto load_full_rows = [&](KeyT (&dst)[E]) {
-    if constexpr (VIA_LDS) {
+    if constexpr (!CAN_VEC) {
+      (void)dst;
+    } else if constexpr (VIA_LDS) {
       const uint4* src = reinterpret_cast<const uint4*>(keys_in + stretch_base);
       uint4 got[PIECES];
 #pragma unroll
@@ -359,7 +432,9 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
     }
   };
   auto store_full_rows = [&](const KeyT (&src)[E]) {
-    if constexpr (VIA_LDS) {
+    if constexpr (!CAN_VEC) {
+      (void)src;
+    } else if constexpr (VIA_LDS) {
       uint4 own[PIECES];
       __builtin_memcpy(own, src, LANE_BYTES);
 #pragma unroll
@@ -392,29 +467,26 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
     load_full_rows(raw);
   } else {
     KeyT got[E];
+    const KeyT* const src = keys_in + stretch_base;
 #pragma unroll
     for (int k = 0; k < E; ++k) {  // (all loads first)
       const uint32_t e = lane + k * WAVE;
       got[k]           = KeyT{};
       if (e < stretch_len) {
-        got[k] = keys_in[stretch_base + e];
+        got[k] = src[e];
       }
     }
 #pragma unroll
     for (int k = 0; k < E; ++k) {
-      const uint32_t e = lane + k * WAVE;
-      if (e < stretch_len) {
-        s_wave[e] = got[k];
-      }
+      s_wave[lane + k * WAVE] = got[k];  // (past the end of the stretch: zeros, which nothing uses)
     }
     __builtin_amdgcn_wave_barrier();  // (a stretch belongs to one wavefront, whose LDS operations execute in order)
+    // (a lane reads its E slots whether its row fills them or not: they lie inside the wavefront's part of
+    // the array, and what lies past the end of a row is replaced below)
+    const KeyT* const own = s_wave + row_at + first;
 #pragma unroll
     for (int r = 0; r < E; ++r) {
-      const uint32_t pos = first + r;
-      raw[r]             = KeyT{};
-      if (row_exists && pos < seg) {
-        raw[r] = s_row[pos];
-      }
+      raw[r] = own[r];
     }
   }
   // A sort that returns values only, on keys whose image is a bijection of their bits (integers; floats when
@@ -426,7 +498,7 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
       bool special = false;
 #pragma unroll
       for (int r = 0; r < E; ++r) {
-        special |= row_exists && first + r < seg && is_nan_or_negative_zero(raw[r]);
+        special |= first + r < row_len && is_nan_or_negative_zero(raw[r]);
       }
       bare = __ballot(special) == 0;
     }
@@ -436,7 +508,7 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
       B b[E];
 #pragma unroll
       for (int r = 0; r < E; ++r) {
-        const bool valid = row_exists && first + r < seg;
+        const bool valid = first + r < row_len;
         // (slots past the end: behind or beside the largest key)
         if constexpr (NATIVE) {
           b[r] = F64Word{valid ? __longlong_as_double(static_cast<long long>(raw[r])) : __builtin_huge_val()};
@@ -450,7 +522,7 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
           b[r] = valid ? static_cast<B>(image) : static_cast<B>(~B{0});
         }
       }
-      blocked_sort<2, N>(b, sub);
+      blocked_sort<LANES>(b, sub);
       KeyT bits[E];
 #pragma unroll
       for (int r = 0; r < E; ++r) {
@@ -474,8 +546,8 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
 #pragma unroll
         for (int r = 0; r < E; ++r) {
           const uint32_t pos = first + r;
-          if (row_exists && pos < seg) {
-            s_row[pos] = bits[r];  // (every lane has read its elements of the stretch; LDS operations of a wavefront execute in order)
+          if (pos < row_len) {
+            s_wave[row_at + pos] = bits[r];  // (every lane has read its elements of the stretch; LDS operations of a wavefront execute in order)
           }
         }
         __builtin_amdgcn_wave_barrier();
@@ -483,7 +555,7 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
         for (int k = 0; k < E; ++k) {
           const uint32_t e = lane + k * WAVE;
           if (e < stretch_len) {
-            keys_out[stretch_base + e] = s_wave[e];
+            dst_keys[e] = s_wave[e];
           }
         }
       }
@@ -494,7 +566,7 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
 #pragma unroll
   for (int r = 0; r < E; ++r) {
     const uint32_t pos = first + r;
-    const bool valid   = row_exists && pos < seg;
+    const bool valid   = pos < row_len;
     // (slots past the end of a row: the largest image, and a position behind every element's)
     const KeyT image = valid ? ordered_bits<CODEC, KeyT>(raw[r]) : static_cast<KeyT>(~KeyT{0});
     if constexpr (sizeof(KeyT) == 8) {
@@ -507,27 +579,27 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
       }
     }
   }
-  blocked_sort<2, N>(w, sub);
+  blocked_sort<LANES>(w, sub);
 
   // ---- slot p of the sorted row holds the element that came from position `from` ----
   uint32_t from[E];
 #pragma unroll
   for (int r = 0; r < E; ++r) {
-    from[r] = word_pos(w[r]) & (N - 1);
+    from[r] = word_pos(w[r]) & 0xFFFFu;
   }
   if (keys_out != nullptr) {
     if (vec_keys) {
       // every lane parks its raw keys and takes those of the positions that ended up in its slots
-      KeyT* mine = s_wave + wrow * N;
+      const uint32_t mine = wrow * N;
 #pragma unroll
       for (int r = 0; r < E; ++r) {
-        mine[first + r] = raw[r];
+        s_wave[mine + first + r] = raw[r];
       }
       __builtin_amdgcn_wave_barrier();
       KeyT bits[E];
 #pragma unroll
       for (int r = 0; r < E; ++r) {
-        bits[r] = mine[from[r]];
+        bits[r] = s_wave[mine + from[r]];
       }
       __builtin_amdgcn_wave_barrier();  // (the parked keys have been read before the pieces of the result go to LDS)
       store_full_rows(bits);
@@ -537,14 +609,14 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
 #pragma unroll
       for (int r = 0; r < E; ++r) {
         const uint32_t pos = first + r;
-        bits[r]            = (row_exists && pos < seg) ? s_row[from[r]] : KeyT{};
+        bits[r]            = (pos < row_len) ? s_wave[row_at + from[r]] : KeyT{};
       }
       __builtin_amdgcn_wave_barrier();
 #pragma unroll
       for (int r = 0; r < E; ++r) {
         const uint32_t pos = first + r;
-        if (row_exists && pos < seg) {
-          s_row[pos] = bits[r];
+        if (pos < row_len) {
+          s_wave[row_at + pos] = bits[r];
         }
       }
       __builtin_amdgcn_wave_barrier();
@@ -552,13 +624,16 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
       for (int k = 0; k < E; ++k) {
         const uint32_t e = lane + k * WAVE;
         if (e < stretch_len) {
-          keys_out[stretch_base + e] = s_wave[e];
+          dst_keys[e] = s_wave[e];
         }
       }
     }
   }
   if constexpr (HAS_IDX) {
-    if (vec_idx) {
+    bool stored = false;
+    if constexpr (CAN_VEC) {
+     if (vec_idx) {
+      stored = true;
       // The positions change hands in LDS as 16-bit words, so that a lane stores two neighbouring int64 words
       // and its neighbours the next ones: a lane that stored the 64 bytes of its own eight slots would touch
       // a cache line of its own with every instruction (2^21 rows of 128 float32 keys: 0.79 ms that way).
@@ -588,13 +663,16 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
           dst[q] = word;
         }
       }
-    } else {
+     }
+    }
+    if (!stored) {
       // positions through LDS as well, so that neighbouring lanes store neighbouring int64 words
       uint16_t* const s_fwave = s_from + wslot * (WAVE * E);
+      int64_t* const dst_idx  = idx_out + stretch_base;
 #pragma unroll
       for (int r = 0; r < E; ++r) {
         const uint32_t pos = first + r;
-        if (row_exists && pos < seg) {
+        if (pos < row_len) {
           s_fwave[wrow * seg + pos] = static_cast<uint16_t>(from[r]);
         }
       }
@@ -603,7 +681,7 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
       for (int k = 0; k < E; ++k) {
         const uint32_t e = lane + k * WAVE;
         if (e < stretch_len) {
-          idx_out[stretch_base + e] = static_cast<int64_t>(s_fwave[e]) + index_offset;
+          dst_idx[e] = static_cast<int64_t>(s_fwave[e]) + index_offset;
         }
       }
     }

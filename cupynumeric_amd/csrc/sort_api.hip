@@ -91,19 +91,19 @@ uint64_t bitonic_row_limit(int key_bytes, bool with_positions)
     const char* e = getenv("CPN_SORT_BITONIC_ROW_LIMIT");
     return e != nullptr && *e != '\0' ? strtoull(e, nullptr, 10) : ~0ull;
   }();
-  // Measured on 2^26 keys against the kernels that take over (network / other, ms).  Values only, where
-  // the network sorts bare images: float32 rows of 129 0.30 / 0.38, of 256 0.17 / 0.24, of 257 0.34 / 0.35,
-  // of 512 0.20 / 0.23; float16 rows of 129 0.32 / 0.38, of 256 0.14 / 0.21, of 257 0.36 / 0.30; float64
-  // rows of 129 0.53 / 0.50, of 256 0.31 / 0.32, of 257 0.63 / 0.40; int8 rows of 129 0.29 / 0.18, of 256
-  // 0.11 / 0.11.  With positions: float32 rows of 129 0.39 / 0.46, of 256 0.23 / 0.31; int32 0.37 / 0.42 and
-  // 0.21 / 0.27.
+  // Measured on 2^26 keys against the kernels that take over (network / other, ms).  Values only: float16 rows of
+  // 257 0.23 / 0.30, of 512 0.16 / 0.19; int16 rows of 257 0.22 / 0.27; float32 rows of 257 0.26 / 0.35, of 512
+  // 0.18 / 0.23; float64 rows of 129 0.29 / 0.51, of 256 0.26 / 0.33, of 257 0.36 / 0.40, of 512 0.30 / 0.28; int64
+  // rows of 256 0.31 / 0.33, of 257 0.45 / 0.40; int8 rows of 129 0.29 / 0.18, of 256 0.11 / 0.11.  With
+  // positions: float16 rows of 257 0.29 / 0.43, of 512 0.19 / 0.27; float32 rows of 257 0.33 / 0.41, of 512 0.27 /
+  // 0.30; float64 rows of 129 0.50 / 0.49, of 256 0.42 / 0.36.
   uint64_t limit = 128;
-  if (with_positions) {
-    limit = key_bytes <= 4 ? 256 : 128;
-  } else if (key_bytes == 2 || key_bytes == 8) {
-    limit = 256;
-  } else if (key_bytes == 4) {
+  if (key_bytes == 2 || key_bytes == 4) {
     limit = 512;
+  } else if (key_bytes == 1) {
+    limit = with_positions ? 256 : 128;
+  } else if (!with_positions) {
+    limit = 256;
   }
   return limit < cap ? limit : cap;
 }

@@ -15,7 +15,6 @@
 #include "profile.h"
 #include "tiny_row_sort.h"
 #include "bitonic_row_sort.h"
-#include "rank_row_sort.h"
 #include "merge_rows.h"
 #include "wave_row_sort.h"
 
@@ -467,38 +466,34 @@ inline int launch_wave_rows(const SortRequest& r)
   return CPN_OK;
 }
 
-template <typename KeyT, int CODEC, bool HAS_IDX, int N>
+template <typename KeyT, int CODEC, bool HAS_IDX, int LANES, int E>
 inline int launch_bitonic_rows(const SortRequest& r)
 {
-  constexpr int E               = blocked_elements(sizeof(KeyT), HAS_IDX, N);
   const uint64_t rows           = r.volume / r.seg;
-  const uint64_t rows_per_block = (256 / WAVE) * (E * WAVE / N);
+  const uint64_t rows_per_block = (256 / WAVE) * (WAVE / LANES);
   const uint64_t blocks         = (rows + rows_per_block - 1) / rows_per_block;
   {
     ProfileScope prof("bitonic_row_sort", r.stream);
-    hipLaunchKernelGGL((bitonic_row_sort_kernel<KeyT, CODEC, HAS_IDX, N, E>), dim3(static_cast<uint32_t>(blocks)),
+    hipLaunchKernelGGL((bitonic_row_sort_kernel<KeyT, CODEC, HAS_IDX, LANES, E>), dim3(static_cast<uint32_t>(blocks)),
                        dim3(256), 0, r.stream, static_cast<const KeyT*>(r.values_in), static_cast<KeyT*>(r.values_out),
                        r.indices_out, static_cast<uint32_t>(r.seg), rows, r.index_offset, static_cast<uint32_t*>(r.temp));
   }
   CPN_HIP_TRY(hipGetLastError());
   return CPN_OK;
 }
-
-template <typename KeyT, int CODEC, bool HAS_IDX>
-inline int launch_rank_rows(const SortRequest& r)
+// A row of up to 8 LANES keys on LANES lanes: 5 ... 8 elements per lane, whichever covers the row.
+template <typename KeyT, int CODEC, bool HAS_IDX, int LANES>
+inline int launch_bitonic_lanes(const SortRequest& r)
 {
-  const uint64_t rows           = r.volume / r.seg;
-  const uint32_t rows_per_block = RANK_ROW_BLOCK / rank_row_threads(static_cast<uint32_t>(r.seg));
-  const uint64_t blocks         = (rows + rows_per_block - 1) / rows_per_block;
-  {
-    ProfileScope prof("rank_row_sort", r.stream);
-    hipLaunchKernelGGL((rank_row_sort_kernel<KeyT, CODEC, HAS_IDX>), dim3(static_cast<uint32_t>(blocks)),
-                       dim3(RANK_ROW_BLOCK), 0, r.stream, static_cast<const KeyT*>(r.values_in),
-                       static_cast<KeyT*>(r.values_out), r.indices_out, static_cast<uint32_t>(r.seg), rows, rows_per_block,
-                       r.index_offset, static_cast<uint32_t*>(r.temp));
+  const uint64_t e = (r.seg + LANES - 1) / LANES;
+  if (e <= 5) {
+    return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, LANES, 5>(r);
+  } else if (e == 6) {
+    return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, LANES, 6>(r);
+  } else if (e == 7) {
+    return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, LANES, 7>(r);
   }
-  CPN_HIP_TRY(hipGetLastError());
-  return CPN_OK;
+  return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, LANES, 8>(r);
 }
 
 template <typename KeyT, int CODEC, bool HAS_IDX, int S>
@@ -529,34 +524,38 @@ inline int sort_rows_in_lds(const SortRequest& r)
     return CPN_ERR_UNSUPPORTED;
   }
   if constexpr (sizeof(KeyT) <= 8 && (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT)) {
-    // Rows just past 32 keys, where the network below would run in 64 slots: every element counts the
-    // elements of its row that come before it (measured on 2^26 keys, counting / network: rows of 33 float32
-    // keys 0.29 / 0.31 ms, of 40 0.33 / 0.28; float64 rows of 33 0.39 / 0.49, of 40 0.43 / 0.44; float16
-    // rows of 33 0.20 / 0.23, of 40 0.22 / 0.20)
-    // (Values only, the network sorts bare images of 4- and 8-byte keys and is ahead there as well: float32
-    // rows of 36 keys 0.31 ms counted, rows of 37 0.19 through the network; float64 rows of 40 / 41 0.45 / 0.36.)
-    if constexpr (HAS_IDX || sizeof(KeyT) <= 2) {
-      if (r.seg >= 33 && r.seg <= (sizeof(KeyT) == 8 ? 40u : 36u) && r.seg <= wave_row_limit() && bitonic_rows_enabled()) {
-        return launch_rank_rows<KeyT, CODEC, HAS_IDX>(r);
-      }
-    }
-    // rows of 2 ... 128 keys and more (bitonic_row_limit): a bitonic network on eight elements per lane
+    // (Rows just past 32 and 64 keys used to be sorted by counting, for every key, the keys of its row that come
+    // before it, because the network ran in the next power of two of slots: 2^26 float32 keys in rows of 33 with
+    // positions 0.33 ms counted, 0.18 in the network since a row takes 8 lanes of 5 elements.)
+    // rows of 2 ... 128 keys and more (bitonic_row_limit): a sorting network on five to eight elements per lane
     if (r.seg >= 2 && r.seg <= bitonic_row_limit(sizeof(KeyT), HAS_IDX) && r.seg <= wave_row_limit() && bitonic_rows_enabled()) {
-      if (r.seg <= 8) {
-        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 8>(r);
-      } else if (r.seg <= 16) {
-        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 16>(r);
-      } else if (r.seg <= 32) {
-        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 32>(r);
-      } else if (r.seg <= 64) {
-        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 64>(r);
-      } else if (r.seg <= 128) {
-        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 128>(r);
-      } else if (r.seg <= 256) {
-        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 256>(r);
+      if constexpr (!HAS_IDX && sizeof(KeyT) == 8) {
+        // full rows of a power of two of 8-byte keys, values only: sixteen elements per lane
+        if (r.seg == 32) {
+          return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 2, 16>(r);
+        } else if (r.seg == 64) {
+          return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 4, 16>(r);
+        } else if (r.seg == 128) {
+          return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 8, 16>(r);
+        } else if (r.seg == 256) {
+          return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 16, 16>(r);
+        }
       }
-      if constexpr (!HAS_IDX && sizeof(KeyT) == 4) {
-        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 512>(r);  // (a row per wavefront)
+      if (r.seg <= 8) {
+        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 1, 8>(r);
+      } else if (r.seg <= 16) {
+        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 2, 8>(r);
+      } else if (r.seg <= 32) {
+        return launch_bitonic_lanes<KeyT, CODEC, HAS_IDX, 4>(r);
+      } else if (r.seg <= 64) {
+        return launch_bitonic_lanes<KeyT, CODEC, HAS_IDX, 8>(r);
+      } else if (r.seg <= 128) {
+        return launch_bitonic_lanes<KeyT, CODEC, HAS_IDX, 16>(r);
+      } else if (r.seg <= 256) {
+        return launch_bitonic_lanes<KeyT, CODEC, HAS_IDX, 32>(r);
+      }
+      if constexpr (sizeof(KeyT) == 2 || sizeof(KeyT) == 4) {
+        return launch_bitonic_lanes<KeyT, CODEC, HAS_IDX, 64>(r);  // (a row per wavefront)
       }
     }
   }
