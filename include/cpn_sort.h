@@ -356,13 +356,11 @@ int64_t cpn_set_lds_row_limit(int64_t limit);
 int64_t cpn_set_wave_row_limit(int64_t limit);
 
 /*
- * Process-wide switch: short rows of real keys of up to 8 bytes (2 ... 128 keys; up to 256 keys of 2 and 4 bytes, of
- * 1 byte when positions are returned and of 8 bytes when only values are; up to 512 keys of 4 bytes when only
- * values are) are sorted by a bitonic
- * network on eight keys per lane of a wavefront -- rows of 33 ... 36 keys (40 of 8 bytes) that return positions
- * or have 2-byte keys by counting, for every key, the keys of its row that come before it -- (enabled != 0, the
- * default) or by the ranking kernels that take the other key types of that length (0).  Returns the previous
- * setting.  Also initialised from the environment variable CPN_SORT_BITONIC_ROWS (0 switches it off);
+ * Process-wide switch: short rows of real keys of up to 8 bytes (2 ... 128 keys; up to 256 keys of 1 byte when
+ * positions are returned and of 8 bytes when only values are; up to 512 keys of 2 and 4 bytes) are sorted by a
+ * network of compare-exchanges on five to eight keys per lane of a wavefront (enabled != 0, the default) or by
+ * the ranking kernels that take the other key types of that length (0).  Returns the previous setting.  Also
+ * initialised from the environment variable CPN_SORT_BITONIC_ROWS (0 switches it off);
  * CPN_SORT_BITONIC_ROW_LIMIT lowers the longest row that the network takes.  Does not affect workspace sizes.
  * An A/B switch with no counterpart in the reference, which merge-sorts (segment id, value) tuples
  * for short rows (src/cupynumeric/sort/thrust_sort.cuh:68-122).
