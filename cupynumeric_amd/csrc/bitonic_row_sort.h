@@ -112,7 +112,7 @@ __device__ __forceinline__ F64Word pack_image_pos(uint32_t image, uint32_t pos)
 }
 __device__ __forceinline__ uint32_t word_pos(const F64Word& w) { return static_cast<uint32_t>(__double_as_longlong(w.v)) & 0xFFFFFu; }
 
-// Elements per lane: eight for full rows (five to seven for rows in between, see the network below), or
+// Elements per lane: eight for full rows (ten, twelve or fourteen for rows in between, see the network below), or
 // sixteen where a sort returns values only of full rows of 8-byte keys (fewer of the steps cross lanes: 6
 // instead of 10 of the 28 steps of a row of 128 keys.  2^26 float64 keys in rows of 32 0.29 -> 0.19 ms, of 128
 // 0.31 -> 0.23; int64 0.21 and 0.27.  Plain sorts of 4-byte keys, which already move at the speed of the
@@ -187,88 +187,97 @@ __device__ __forceinline__ void blocked_exchange_in_lane(W& lo, W& hi)
 // lanes are merged in pairs: a merge starts by comparing every element with its mirror image in the run of
 // both (register E - 1 - r of the mirrored lane), goes on with the same register of the lanes at distance
 // KL / 4 ... 1, and ends inside the lanes, whose elements are a bitonic sequence by then.  The smaller word
-// always goes to the smaller element number, so no step has to know which way its run points.  For E = 8 and
-// 16 this is the bitonic sorter (its comparators all pointing the same way); E = 5, 6, 7 use the smallest
-// known networks of 9, 12 and 16 exchanges inside a lane (a bitonic sequence of 6: a half-cleaner and two
-// networks of 3), which lets a row of n keys take 8, 16, 32 or 64 lanes of ceil(n / lanes) elements each
-// instead of the next power of two of slots.  `sub` is the lane's number inside its row.
+// always goes to the smaller element number, so no step has to know which way its run points.  E need not be
+// a power of two: a row of n keys takes 1, 2, 4 ... 32 lanes of 8, 10, 12, 14 or 16 elements each, whichever
+// covers it, instead of the next power of two of slots.  Inside a lane: Batcher's odd-even merge sort for 16
+// elements without the exchanges that touch elements past E (they would compare with padding that is never
+// smaller), 19, 32, 42, 53 and 63 exchanges for E = 8 ... 16; a bitonic sequence of an even number of elements
+// takes a half-cleaner and becomes two bitonic sequences of half the length, and one of 3, 5 or 7 elements is
+// sorted by the smallest known network (3, 9, 16 exchanges).  `sub` is the lane's number inside its row.
 template <int A, int B, typename W, int E>
 __device__ __forceinline__ void lane_exchange(W (&w)[E])
 {
   static_assert(A < B && B < E, "the smaller word goes to the smaller element number");
   blocked_exchange_in_lane(w[A], w[B]);
 }
-// The steps (i, i | J) for J = J0, J0 / 2 ... 1: sorts a bitonic sequence of a power of two of elements.
-template <int J, typename W, int E>
-__device__ __forceinline__ void lane_half_cleaners(W (&w)[E])
+template <int LO, int N, int R, typename W, int E>
+__device__ __forceinline__ void oddeven_merge(W (&w)[E])
 {
-  if constexpr (J >= 1) {
+  if constexpr (LO + R < E) {
+    constexpr int M = 2 * R;
+    if constexpr (M < N) {
+      oddeven_merge<LO, N, M>(w);
+      oddeven_merge<LO + R, N, M>(w);
 #pragma unroll
-    for (int r = 0; r < E; ++r) {
-      if ((r & J) == 0) {
-        blocked_exchange_in_lane(w[r], w[r | J]);
+      for (int i = LO + R; i + R < LO + N; i += M) {
+        if (i + R < E) {
+          blocked_exchange_in_lane(w[i], w[i + R]);
+        }
       }
+    } else {
+      blocked_exchange_in_lane(w[LO], w[LO + R]);
     }
-    lane_half_cleaners<J / 2>(w);
   }
 }
-template <int K, typename W, int E>
-__device__ __forceinline__ void lane_bitonic_levels(W (&w)[E])
+template <int LO, int N, typename W, int E>
+__device__ __forceinline__ void oddeven_merge_sort(W (&w)[E])
 {
-  if constexpr (K <= E) {
-#pragma unroll
-    for (int r = 0; r < E; ++r) {
-      if ((r & (K / 2)) == 0) {
-        blocked_exchange_in_lane(w[r], w[r ^ (K - 1)]);
-      }
-    }
-    lane_half_cleaners<K / 4>(w);
-    lane_bitonic_levels<2 * K>(w);
+  if constexpr (N > 1 && LO + 1 < E) {
+    oddeven_merge_sort<LO, N / 2>(w);
+    oddeven_merge_sort<LO + N / 2, N / 2>(w);
+    oddeven_merge<LO, N, 1>(w);
   }
 }
 // Sorts the E elements of a lane, whatever their order.
 template <typename W, int E>
 __device__ __forceinline__ void lane_sort(W (&w)[E])
 {
-  if constexpr (E == 3) {
-    lane_exchange<0, 2>(w), lane_exchange<0, 1>(w), lane_exchange<1, 2>(w);
-  } else if constexpr (E == 5) {
-    lane_exchange<0, 3>(w), lane_exchange<1, 4>(w);
-    lane_exchange<0, 2>(w), lane_exchange<1, 3>(w);
-    lane_exchange<0, 1>(w), lane_exchange<2, 4>(w);
-    lane_exchange<1, 2>(w), lane_exchange<3, 4>(w);
-    lane_exchange<2, 3>(w);
-  } else if constexpr (E == 6) {
-    lane_exchange<0, 5>(w), lane_exchange<1, 3>(w), lane_exchange<2, 4>(w);
-    lane_exchange<1, 2>(w), lane_exchange<3, 4>(w);
-    lane_exchange<0, 3>(w), lane_exchange<2, 5>(w);
-    lane_exchange<0, 1>(w), lane_exchange<2, 3>(w), lane_exchange<4, 5>(w);
-    lane_exchange<1, 2>(w), lane_exchange<3, 4>(w);
-  } else if constexpr (E == 7) {
-    lane_exchange<0, 6>(w), lane_exchange<2, 3>(w), lane_exchange<4, 5>(w);
-    lane_exchange<0, 2>(w), lane_exchange<1, 4>(w), lane_exchange<3, 6>(w);
-    lane_exchange<0, 1>(w), lane_exchange<2, 5>(w), lane_exchange<3, 4>(w);
-    lane_exchange<1, 2>(w), lane_exchange<4, 6>(w);
-    lane_exchange<2, 3>(w), lane_exchange<4, 5>(w);
-    lane_exchange<1, 2>(w), lane_exchange<3, 4>(w), lane_exchange<5, 6>(w);
+  static_assert(E > 4 && E <= 16, "elements per lane");
+  oddeven_merge_sort<0, (E <= 8 ? 8 : 16)>(w);
+}
+// Sorts elements OFF ... OFF + M - 1 of a lane, M = 3, 5, 7.
+template <int OFF, int M, typename W, int E>
+__device__ __forceinline__ void lane_sort_part(W (&w)[E])
+{
+  if constexpr (M == 3) {
+    lane_exchange<OFF + 0, OFF + 2>(w), lane_exchange<OFF + 0, OFF + 1>(w), lane_exchange<OFF + 1, OFF + 2>(w);
+  } else if constexpr (M == 5) {
+    lane_exchange<OFF + 0, OFF + 3>(w), lane_exchange<OFF + 1, OFF + 4>(w);
+    lane_exchange<OFF + 0, OFF + 2>(w), lane_exchange<OFF + 1, OFF + 3>(w);
+    lane_exchange<OFF + 0, OFF + 1>(w), lane_exchange<OFF + 2, OFF + 4>(w);
+    lane_exchange<OFF + 1, OFF + 2>(w), lane_exchange<OFF + 3, OFF + 4>(w);
+    lane_exchange<OFF + 2, OFF + 3>(w);
   } else {
-    static_assert((E & (E - 1)) == 0, "a power of two of elements: the bitonic sorter");
-    lane_bitonic_levels<2>(w);
+    static_assert(M == 7, "networks for 3, 5 and 7 elements");
+    lane_exchange<OFF + 0, OFF + 6>(w), lane_exchange<OFF + 2, OFF + 3>(w), lane_exchange<OFF + 4, OFF + 5>(w);
+    lane_exchange<OFF + 0, OFF + 2>(w), lane_exchange<OFF + 1, OFF + 4>(w), lane_exchange<OFF + 3, OFF + 6>(w);
+    lane_exchange<OFF + 0, OFF + 1>(w), lane_exchange<OFF + 2, OFF + 5>(w), lane_exchange<OFF + 3, OFF + 4>(w);
+    lane_exchange<OFF + 1, OFF + 2>(w), lane_exchange<OFF + 4, OFF + 6>(w);
+    lane_exchange<OFF + 2, OFF + 3>(w), lane_exchange<OFF + 4, OFF + 5>(w);
+    lane_exchange<OFF + 1, OFF + 2>(w), lane_exchange<OFF + 3, OFF + 4>(w), lane_exchange<OFF + 5, OFF + 6>(w);
   }
 }
-// Sorts the E elements of a lane that form a bitonic sequence.
+// Sorts elements OFF ... OFF + M - 1 of a lane, which form a bitonic sequence.
+template <int OFF, int M, typename W, int E>
+__device__ __forceinline__ void lane_sort_bitonic_part(W (&w)[E])
+{
+  if constexpr (M > 1) {
+    if constexpr (M % 2 == 0) {
+#pragma unroll
+      for (int i = 0; i < M / 2; ++i) {
+        blocked_exchange_in_lane(w[OFF + i], w[OFF + i + M / 2]);
+      }
+      lane_sort_bitonic_part<OFF, M / 2>(w);
+      lane_sort_bitonic_part<OFF + M / 2, M / 2>(w);
+    } else {
+      lane_sort_part<OFF, M>(w);
+    }
+  }
+}
 template <typename W, int E>
 __device__ __forceinline__ void lane_sort_bitonic(W (&w)[E])
 {
-  if constexpr ((E & (E - 1)) == 0) {
-    lane_half_cleaners<E / 2>(w);
-  } else if constexpr (E == 6) {
-    lane_exchange<0, 3>(w), lane_exchange<1, 4>(w), lane_exchange<2, 5>(w);
-    lane_exchange<0, 2>(w), lane_exchange<0, 1>(w), lane_exchange<1, 2>(w);
-    lane_exchange<3, 5>(w), lane_exchange<3, 4>(w), lane_exchange<4, 5>(w);
-  } else {
-    lane_sort(w);
-  }
+  lane_sort_bitonic_part<0, E>(w);
 }
 // The steps of a merge that cross lanes: the mirror image in the run of KL lanes, then the lanes at distance D.
 template <int KL, typename W, int E>
@@ -329,7 +338,7 @@ __global__ __launch_bounds__(256) void bitonic_row_sort_kernel(const KeyT* __res
 {
   static_assert(sizeof(KeyT) <= 8 && (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT),
                 "real keys of up to 8 bytes");
-  static_assert((E >= 5 && E <= 8) || E == 16, "elements per lane");
+  static_assert(E >= 8 && E <= 16 && E % 2 == 0, "elements per lane");
   static_assert(LANES >= 1 && LANES <= WAVE && (LANES & (LANES - 1)) == 0, "lanes per row: a power of two");
   constexpr int N = LANES * E;  // slots per row
   if (blockIdx.x == 0 && threadIdx.x == 0) {

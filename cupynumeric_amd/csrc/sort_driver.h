@@ -481,17 +481,19 @@ inline int launch_bitonic_rows(const SortRequest& r)
   CPN_HIP_TRY(hipGetLastError());
   return CPN_OK;
 }
-// A row of up to 8 LANES keys on LANES lanes: 5 ... 8 elements per lane, whichever covers the row.
+// A row of more than 4 LANES and up to 8 LANES keys: LANES lanes of 8 elements, or half as many lanes of 10, 12
+// or 14 (fewer of the network's steps cross lanes), whichever covers the row.
 template <typename KeyT, int CODEC, bool HAS_IDX, int LANES>
 inline int launch_bitonic_lanes(const SortRequest& r)
 {
+  static_assert(LANES >= 2, "half the lanes");
   const uint64_t e = (r.seg + LANES - 1) / LANES;
   if (e <= 5) {
-    return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, LANES, 5>(r);
+    return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, LANES / 2, 10>(r);
   } else if (e == 6) {
-    return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, LANES, 6>(r);
+    return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, LANES / 2, 12>(r);
   } else if (e == 7) {
-    return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, LANES, 7>(r);
+    return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, LANES / 2, 14>(r);
   }
   return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, LANES, 8>(r);
 }
@@ -527,7 +529,7 @@ inline int sort_rows_in_lds(const SortRequest& r)
     // (Rows just past 32 and 64 keys used to be sorted by counting, for every key, the keys of its row that come
     // before it, because the network ran in the next power of two of slots: 2^26 float32 keys in rows of 33 with
     // positions 0.33 ms counted, 0.18 in the network since a row takes 8 lanes of 5 elements.)
-    // rows of 2 ... 128 keys and more (bitonic_row_limit): a sorting network on five to eight elements per lane
+    // rows of 2 ... 128 keys and more (bitonic_row_limit): a sorting network on eight to fourteen elements per lane
     if (r.seg >= 2 && r.seg <= bitonic_row_limit(sizeof(KeyT), HAS_IDX) && r.seg <= wave_row_limit() && bitonic_rows_enabled()) {
       if constexpr (!HAS_IDX && sizeof(KeyT) == 8) {
         // full rows of a power of two of 8-byte keys, values only: sixteen elements per lane
