@@ -1,22 +1,21 @@
 // Short rows of real keys of up to 8 bytes (how long: bitonic_row_limit, 128 ... 512 keys), sorted by a
-// bitonic network of compare-exchanges on words held in registers, eight elements per lane: element i of
-// a row sits in register i % 8 of the row's lane i / 8, a row of N slots (N = the next power of two from 8
-// on) takes N / 8 lanes and a wavefront holds 512 / N rows.  The exchanges between elements less than 8
-// apart happen between the registers of a lane, only the others cross lanes, through DPP and swizzle
-// moves: of the 28 steps of a row of 128 keys, 18 are inside the lanes and 10 cross them.  (One element
-// per lane, the layout this kernel started with, crosses lanes in all 28 steps: 2^26 float32 keys in rows
-// of 128 took 0.28 ms, rows of 32 0.25, rows of 8 0.20.)
+// network of compare-exchanges on words held in registers, E = 8 ... 16 elements per lane: element i of a row
+// sits in register i % E of the row's lane i / E, a row takes a power of two of lanes (1 ... 64, with the E that
+// covers it) and a wavefront holds 64 / lanes rows.  The exchanges between elements of one lane happen between
+// its registers, only the others cross lanes, through DPP and swizzle moves: of the 28 steps of a row of 128
+// keys on 16 lanes of 8, 18 are inside the lanes and 10 cross them.  (One element per lane, the layout this
+// kernel started with, crosses lanes in all 28 steps: 2^26 float32 keys in rows of 128 took 0.28 ms, rows of 32
+// 0.25, rows of 8 0.20.)
 //
 // What is compared: a sort that returns values only, on keys whose image is a bijection of their bits
 // (integers; floats when no row of the wavefront holds a NaN or a -0.0), sorts the bare images and maps
 // them back (2^26 float32 keys in rows of 128 0.11 ms, of 32 0.09: the speed of the memory).  Otherwise
 // the words are (order-preserving image of the key, position in the row) as one word (32 bits for 1- and
 // 2-byte keys; for 4-byte keys a double whose mantissa holds both; an image and a position word for 8-byte
-// keys), so that no two are equal: the network, which is not stable by
-// itself, then yields exactly the stable order (NaNs tie with each other and +0.0 with -0.0 in the image,
+// keys), so that no two are equal: the network, which is not stable by itself, then yields exactly the stable order (NaNs tie with each other and +0.0 with -0.0 in the image,
 // and the position decides); the raw keys do not travel: they wait in LDS, and every lane fetches the
-// keys of the positions that ended up in its slots once, at the end (rows of 128 float32 keys 0.22 ms,
-// with positions out 0.25).  Slots past the end of a row hold the largest image and sort behind, or
+// keys of the positions that ended up in its slots once, at the end (rows of 128 float32 keys with positions
+// out 0.15 ms).  Slots past the end of a row hold the largest image and sort behind, or
 // beside, every real element.
 //
 // Memory is read and written in whole contiguous stretches: a lane of a full row moves its eight

@@ -528,7 +528,7 @@ inline int sort_rows_in_lds(const SortRequest& r)
   if constexpr (sizeof(KeyT) <= 8 && (CODEC == CODEC_UNSIGNED || CODEC == CODEC_SIGNED || CODEC == CODEC_FLOAT)) {
     // (Rows just past 32 and 64 keys used to be sorted by counting, for every key, the keys of its row that come
     // before it, because the network ran in the next power of two of slots: 2^26 float32 keys in rows of 33 with
-    // positions 0.33 ms counted, 0.18 in the network since a row takes 8 lanes of 5 elements.)
+    // positions 0.33 ms counted, 0.15 in the network since a row takes 4 lanes of 10 elements.)
     // rows of 2 ... 128 keys and more (bitonic_row_limit): a sorting network on eight to fourteen elements per lane
     if (r.seg >= 2 && r.seg <= bitonic_row_limit(sizeof(KeyT), HAS_IDX) && r.seg <= wave_row_limit() && bitonic_rows_enabled()) {
       if constexpr (!HAS_IDX && sizeof(KeyT) == 8) {
