@@ -96,10 +96,14 @@ uint64_t bitonic_row_limit(int key_bytes, bool with_positions)
   // 0.18 / 0.23; float64 rows of 129 0.29 / 0.51, of 256 0.26 / 0.33, of 257 0.36 / 0.40, of 512 0.30 / 0.28; int64
   // rows of 256 0.31 / 0.33, of 257 0.45 / 0.40; int8 rows of 129 0.29 / 0.18, of 256 0.11 / 0.11.  With
   // positions: float16 rows of 257 0.29 / 0.43, of 512 0.19 / 0.27; float32 rows of 257 0.33 / 0.41, of 512 0.27 /
-  // 0.30; float64 rows of 129 0.50 / 0.49, of 256 0.42 / 0.36.
+  // 0.30; float64 rows of 129 0.50 / 0.49, of 256 0.42 / 0.36.  A row per wavefront with up to 16 elements per
+  // lane, 513 ... 1024 keys: float32 rows of 513 0.26 / 0.25, of 640 0.22 / 0.25, of 896 0.24 / 0.27, of 1024
+  // 0.23 / 0.25 (int32 0.26 / 0.23, 0.22 / 0.22, 0.23 / 0.25, 0.21 / 0.23), with positions 0.34 / 0.35, 0.30 /
+  // 0.33, 0.30 / 0.32, 0.29 / 0.32; float16 rows of 513 0.24 / 0.28, of 768 0.20 / 0.21, of 896 0.22 / 0.19, of
+  // 1024 0.18 / 0.18, with positions 0.28 / 0.42, 0.25 / 0.32, 0.27 / 0.29, 0.23 / 0.27.
   uint64_t limit = 128;
   if (key_bytes == 2 || key_bytes == 4) {
-    limit = 512;
+    limit = (key_bytes == 2 && !with_positions) ? 768 : 1024;
   } else if (key_bytes == 1) {
     limit = with_positions ? 256 : 128;
   } else if (!with_positions) {

@@ -557,7 +557,19 @@ inline int sort_rows_in_lds(const SortRequest& r)
         return launch_bitonic_lanes<KeyT, CODEC, HAS_IDX, 32>(r);
       }
       if constexpr (sizeof(KeyT) == 2 || sizeof(KeyT) == 4) {
-        return launch_bitonic_lanes<KeyT, CODEC, HAS_IDX, 64>(r);  // (a row per wavefront)
+        // a row per wavefront: 8 ... 16 elements per lane
+        if (r.seg <= 512) {
+          return launch_bitonic_lanes<KeyT, CODEC, HAS_IDX, 64>(r);
+        }
+        const uint64_t e = (r.seg + WAVE - 1) / WAVE;
+        if (e <= 10) {
+          return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 64, 10>(r);
+        } else if (e <= 12) {
+          return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 64, 12>(r);
+        } else if (e <= 14) {
+          return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 64, 14>(r);
+        }
+        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 64, 16>(r);
       }
     }
   }

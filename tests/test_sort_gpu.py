@@ -282,7 +282,7 @@ def test_short_float_rows_without_nans_or_negative_zeros(lib, torch_cuda, dtype)
     of which a few hold a NaN or a -0.0, so that wavefronts of both kinds run in one launch."""
     dt = np.dtype(dtype)
     rng = np.random.default_rng(dt.num * 17 + 3)
-    for seg in list(range(2, 70)) + [80, 81, 95, 96, 100, 113, 127, 128, 129, 161, 200, 255, 256, 257, 321, 385, 449, 512]:
+    for seg in list(range(2, 70)) + [80, 81, 95, 96, 100, 113, 127, 128, 129, 161, 200, 255, 256, 257, 321, 385, 449, 512, 600, 768, 900, 1024]:
         rows = 1 + (seg * 5) % 19 if seg % 3 else 150 + seg
         x = rng.standard_normal((rows, seg)).astype(dtype)
         x[0] = x[0, 0]
@@ -366,7 +366,7 @@ def test_rows_of_up_to_128_keys_through_the_bitonic_network(lib, torch_cuda, dty
     dt = np.dtype(dtype)
     rng = np.random.default_rng(dt.num * 13 + 5)
     for seg in list(range(2, 70)) + [80, 81, 95, 96, 97, 100, 112, 113, 126, 127, 128, 129, 160, 161, 192, 193, 224, 225, 255, 256,
-                                     257, 320, 321, 384, 385, 448, 449, 511, 512, 513]:
+                                     257, 320, 321, 384, 385, 448, 449, 511, 512, 513, 640, 641, 768, 769, 896, 897, 1000, 1023, 1024, 1025]:
         rows = 1 + (seg * 7) % 23 if seg % 3 else 200 + seg
         x = make_input(dtype, (rows, seg), seed=seg)
         x[0] = x[0, 0]
@@ -389,7 +389,7 @@ def test_rows_of_up_to_128_keys_through_the_bitonic_network(lib, torch_cuda, dty
                 x[5, ::2] = np.iinfo(dtype).min
                 x[6] = rng.integers(0, 3, seg).astype(dtype)
         want_v, want_i = check_rows(lib, torch_cuda, x, f"{dt} seg={seg}")
-        if seg in (2, 3, 17, 32, 33, 64, 65, 100, 128, 161, 256, 321, 512):
+        if seg in (2, 3, 17, 32, 33, 64, 65, 100, 128, 161, 256, 321, 512, 641, 1024):
             v, i = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=True, offset=-5)
             assert_same_bits(v, want_v, f"{dt} seg={seg} values+positions")
             assert_same_bits(i, want_i - 5, f"{dt} seg={seg} values+positions, offset")
