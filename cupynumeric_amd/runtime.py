@@ -32,6 +32,8 @@ class Runtime:
         mode = os.environ.get("CUPYNUMERIC_AMD_CHECK_STATUS", "lazy").lower()
         self.check_mode = {"0": "off", "off": "off", "1": "eager", "eager": "eager"}.get(mode, "lazy")
         self._torch = None
+        self._device_seen = False
+        self._devices = {}
         self._status_slots = None
         self._status_kinds: list[str] = []
         self._status_used = 0
@@ -90,16 +92,27 @@ class Runtime:
 
     def require_device(self) -> "torch.device":
         torch = self.torch
-        if not torch.cuda.is_available():
-            raise RuntimeError(
-                "cupynumeric_amd needs a HIP device: no GPU is visible to this process "
-                "(there is no CPU fallback for the sort path)"
-            )
-        return torch.device("cuda", torch.cuda.current_device())
+        if not self._device_seen:  # (asked once: the answer does not change while the process lives, and the
+            # question costs about 2 us, which a sort of a thousand keys notices)
+            if not torch.cuda.is_available():
+                raise RuntimeError(
+                    "cupynumeric_amd needs a HIP device: no GPU is visible to this process "
+                    "(there is no CPU fallback for the sort path)"
+                )
+            self._device_seen = True
+        index = torch.cuda.current_device()
+        dev = self._devices.get(index)
+        if dev is None:
+            dev = self._devices[index] = torch.device("cuda", index)
+        return dev
 
     def stream_handle(self) -> int:
         """hipStream_t of torch's current stream, as an integer."""
-        return int(self.torch.cuda.current_stream().cuda_stream)
+        torch = self.torch
+        raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+        if raw is not None:  # (the same handle as current_stream().cuda_stream without building a Stream object)
+            return int(raw(torch.cuda.current_device()))
+        return int(torch.cuda.current_stream().cuda_stream)
 
     def empty_bytes(self, nbytes: int) -> "torch.Tensor":
         """Uninitialised device buffer of `nbytes` bytes (at least one, so that it has an address)."""
