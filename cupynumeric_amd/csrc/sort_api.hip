@@ -85,7 +85,7 @@ static std::atomic<int> g_bitonic_rows{[] {
 }()};
 
 bool bitonic_rows_enabled() { return g_bitonic_rows.load(std::memory_order_relaxed) != 0; }
-uint64_t bitonic_row_limit(int key_bytes, bool with_positions)
+uint64_t bitonic_row_limit(int key_bytes, bool with_positions, bool float_keys)
 {
   static const uint64_t cap = [] {
     const char* e = getenv("CPN_SORT_BITONIC_ROW_LIMIT");
@@ -100,14 +100,15 @@ uint64_t bitonic_row_limit(int key_bytes, bool with_positions)
   // lane, 513 ... 1024 keys: float32 rows of 513 0.26 / 0.25, of 640 0.22 / 0.25, of 896 0.24 / 0.27, of 1024
   // 0.23 / 0.25 (int32 0.26 / 0.23, 0.22 / 0.22, 0.23 / 0.25, 0.21 / 0.23), with positions 0.34 / 0.35, 0.30 /
   // 0.33, 0.30 / 0.32, 0.29 / 0.32; float16 rows of 513 0.24 / 0.28, of 768 0.20 / 0.21, of 896 0.22 / 0.19, of
-  // 1024 0.18 / 0.18, with positions 0.28 / 0.42, 0.25 / 0.32, 0.27 / 0.29, 0.23 / 0.27.
+  // 1024 0.18 / 0.18, with positions 0.28 / 0.42, 0.25 / 0.32, 0.27 / 0.29, 0.23 / 0.27.  float64, values only, 32
+  // lanes of 10 ... 16: rows of 257 0.36 / 0.42, of 384 0.30 / 0.35, of 448 0.32 / 0.31, of 500 0.34 / 0.31.
   uint64_t limit = 128;
   if (key_bytes == 2 || key_bytes == 4) {
     limit = (key_bytes == 2 && !with_positions) ? 768 : 1024;
   } else if (key_bytes == 1) {
     limit = with_positions ? 256 : 128;
   } else if (!with_positions) {
-    limit = 256;
+    limit = float_keys ? 384 : 256;  // (8-byte keys; float64 keys are compared as numbers)
   }
   return limit < cap ? limit : cap;
 }

@@ -111,7 +111,7 @@ __host__ __device__ constexpr int key_passes(int key_bytes, int codec)
 bool bitonic_rows_enabled();
 // Longest row that goes through the network, per key width and with or without positions; the environment
 // variable CPN_SORT_BITONIC_ROW_LIMIT lowers it (A/B runs).
-uint64_t bitonic_row_limit(int key_bytes, bool with_positions);
+uint64_t bitonic_row_limit(int key_bytes, bool with_positions, bool float_keys);
 
 // Row length up to which one wavefront (instead of one workgroup) sorts a row; at most 1024.
 // Changed by cpn_set_wave_row_limit / CPN_SORT_WAVE_ROW_LIMIT for A/B runs.
@@ -530,7 +530,8 @@ inline int sort_rows_in_lds(const SortRequest& r)
     // before it, because the network ran in the next power of two of slots: 2^26 float32 keys in rows of 33 with
     // positions 0.33 ms counted, 0.15 in the network since a row takes 4 lanes of 10 elements.)
     // rows of 2 ... 128 keys and more (bitonic_row_limit): a sorting network on eight to fourteen elements per lane
-    if (r.seg >= 2 && r.seg <= bitonic_row_limit(sizeof(KeyT), HAS_IDX) && r.seg <= wave_row_limit() && bitonic_rows_enabled()) {
+    if (r.seg >= 2 && r.seg <= bitonic_row_limit(sizeof(KeyT), HAS_IDX, CODEC == CODEC_FLOAT) && r.seg <= wave_row_limit() &&
+        bitonic_rows_enabled()) {
       if constexpr (!HAS_IDX && sizeof(KeyT) == 8) {
         // full rows of a power of two of 8-byte keys, values only: sixteen elements per lane
         if (r.seg == 32) {
@@ -555,6 +556,13 @@ inline int sort_rows_in_lds(const SortRequest& r)
         return launch_bitonic_lanes<KeyT, CODEC, HAS_IDX, 16>(r);
       } else if (r.seg <= 256) {
         return launch_bitonic_lanes<KeyT, CODEC, HAS_IDX, 32>(r);
+      }
+      if constexpr (sizeof(KeyT) == 8 && CODEC == CODEC_FLOAT && !HAS_IDX) {
+        // 257 ... 384 float64 keys, values only (compared as numbers): 32 lanes of 10 or 12
+        if (r.seg <= 320) {
+          return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 32, 10>(r);
+        }
+        return launch_bitonic_rows<KeyT, CODEC, HAS_IDX, 32, 12>(r);
       }
       if constexpr (sizeof(KeyT) == 2 || sizeof(KeyT) == 4) {
         // a row per wavefront: 8 ... 16 elements per lane

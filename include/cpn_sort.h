@@ -357,7 +357,7 @@ int64_t cpn_set_wave_row_limit(int64_t limit);
 
 /*
  * Process-wide switch: short rows of real keys of up to 8 bytes (2 ... 128 keys; up to 256 keys of 1 byte when
- * positions are returned and of 8 bytes when only values are; up to 1024 keys of 2 and 4 bytes) are sorted by a
+ * positions are returned and of 8 bytes when only values are, 384 for float64; up to 1024 keys of 2 and 4 bytes) are sorted by a
  * network of compare-exchanges on eight to fourteen keys per lane of a wavefront (enabled != 0, the default) or by
  * the ranking kernels that take the other key types of that length (0).  Returns the previous setting.  Also
  * initialised from the environment variable CPN_SORT_BITONIC_ROWS (0 switches it off);
