@@ -129,7 +129,7 @@ def make_config(name: str, log2n: int | None = None, rows: int | None = None) ->
 EDGE_LENGTHS = (
     ("float32", "sort", (32, 40, 64, 96, 128, 256, 512, 768, 1024, 1536, 2048, 3072, 4096, 6144, 8192, 12288, 16384, 32768, 65536)),
     ("float64", "sort", (32, 40, 64, 96, 128, 256, 384, 512, 768, 1024, 1536, 2048, 3072, 4096, 6144, 8192, 16384, 32768, 65536, 1048576)),
-    ("float16", "sort", (32, 40, 64, 96, 128, 256, 512, 768, 4096, 8192, 16384, 32768)),
+    ("float16", "sort", (32, 40, 64, 96, 128, 256, 512, 768, 4096, 8192, 16384, 32768, 57344)),
     ("float32", "argsort", (32, 40, 64, 96, 128, 256, 512, 1024, 2048, 4096, 6144, 8192, 16384, 32768, 65536)),
     ("float64", "argsort", (32, 40, 64, 96, 128, 256, 512, 2048, 4096, 6144, 8192, 14336, 28672, 57344, 458752)),
 )

@@ -353,7 +353,7 @@ __global__ __launch_bounds__(COUNT16_BLOCK) void count16_rows_kernel(const uint1
   }
 }
 
-// Rows of 8193 to 16 384 keys (ITEMS = 16) and of up to 32 768 (ITEMS = 32).  grid = rows, block = 1024,
+// Rows of 8193 to 16 384 keys (ITEMS = 16), of up to 32 768 (ITEMS = 32) and of up to 57 344 (ITEMS = 56).  grid = rows, block = 1024,
 // thread t owns elements [ITEMS t, ITEMS (t + 1)).
 // No LDS is left for a marker row here: every key takes its offset from an atomic on the scanned
 // histogram and is staged in the histogram's memory once that is no longer needed (65 536 bins of 16

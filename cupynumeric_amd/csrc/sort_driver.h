@@ -98,8 +98,8 @@ __host__ __device__ constexpr uint64_t lds_row_capacity(int key_bytes, bool with
   return key_bytes == 16 ? 4096 : (key_bytes == 8 ? (with_positions ? 14336 : 16384) : 16384);
 }
 // Values-only sorts of 2-byte keys: the counting kernel (count_row_sort.h) needs no room for the row beside
-// its 65 536 bins and takes rows of up to 32 768 keys (lds_row_limit says whether it is in use).
-constexpr uint64_t COUNT16_ROW_CAPACITY = 32768;
+// its 65 536 bins and takes rows of up to 57 344 keys (lds_row_limit says whether it is in use).
+constexpr uint64_t COUNT16_ROW_CAPACITY = 57344;
 // Radix passes of a key: one per byte, plus the NaN-class pass of complex keys.
 __host__ __device__ constexpr int key_passes(int key_bytes, int codec)
 {
@@ -437,9 +437,14 @@ inline int launch_count16_rows(const SortRequest& r)
       hipLaunchKernelGGL((count16_long_rows_kernel<CODEC, 16>), dim3(static_cast<uint32_t>(rows)), dim3(COUNT16_BLOCK), 0,
                          r.stream, static_cast<const uint16_t*>(r.values_in), static_cast<uint16_t*>(r.values_out),
                          static_cast<uint32_t>(r.seg), static_cast<uint32_t*>(r.temp));
-    } else {
+    } else if (r.seg <= 32768) {
       // 16 385 ... 32 768 keys: 32 keys per thread
       hipLaunchKernelGGL((count16_long_rows_kernel<CODEC, 32>), dim3(static_cast<uint32_t>(rows)), dim3(COUNT16_BLOCK), 0,
+                         r.stream, static_cast<const uint16_t*>(r.values_in), static_cast<uint16_t*>(r.values_out),
+                         static_cast<uint32_t>(r.seg), static_cast<uint32_t*>(r.temp));
+    } else {
+      // ... 57 344 keys: 56 keys per thread (counts and offsets of a row have to fit 16 bits)
+      hipLaunchKernelGGL((count16_long_rows_kernel<CODEC, 56>), dim3(static_cast<uint32_t>(rows)), dim3(COUNT16_BLOCK), 0,
                          r.stream, static_cast<const uint16_t*>(r.values_in), static_cast<uint16_t*>(r.values_out),
                          static_cast<uint32_t>(r.seg), static_cast<uint32_t*>(r.temp));
     }

@@ -99,8 +99,8 @@ def test_temp_bytes_layout(lib):
     # only, 14 336 when positions are staged beside them; 16-byte keys 4096
     f64, c128_ = 11, 13
     assert tb(f32, 4 * 16384, 16384, 1, 1, 0) == header and tb(f32, 4 * 16385, 16385, 1, 0, 0) > header
-    # float16: values-only rows are counted up to 32 768 keys; with positions the radix rows end at 16 384
-    assert tb(9, 4 * 32768, 32768, 1, 0, 0) == header and tb(9, 4 * 32769, 32769, 1, 0, 0) > header
+    # float16: values-only rows are counted up to 57 344 keys; with positions the radix rows end at 16 384
+    assert tb(9, 4 * 57344, 57344, 1, 0, 0) == header and tb(9, 4 * 57345, 57345, 1, 0, 0) > header
     assert tb(9, 4 * 16384, 16384, 0, 1, 0) == header and tb(9, 4 * 16385, 16385, 0, 1, 0) > header
     assert tb(f64, 4 * 16384, 16384, 1, 0, 0) == header and tb(f64, 4 * 16385, 16385, 1, 0, 0) > header
     assert tb(f64, 4 * 14336, 14336, 0, 1, 0) == header and tb(f64, 4 * 14337, 14337, 0, 1, 0) > header

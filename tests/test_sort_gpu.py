@@ -503,11 +503,11 @@ def test_two_byte_rows_of_8193_to_16384_keys_through_the_radix_shape(torch_cuda)
 
 
 @pytest.mark.parametrize("dtype", [np.float16, np.int16, np.uint16])
-def test_two_byte_rows_of_up_to_32768_keys_are_counted(lib, torch_cuda, dtype):
-    """Plain sorts of rows of 16 385 ... 32 768 two-byte keys: the counting kernel with 32 keys per thread
+def test_two_byte_rows_of_up_to_57344_keys_are_counted(lib, torch_cuda, dtype):
+    """Plain sorts of rows of 16 385 ... 57 344 two-byte keys: the counting kernel with 32 and 56 keys per thread
     (zeros and NaNs in input order); one key more, and the same rows with positions, take the global path."""
     u = np.uint16
-    for seg in (16385, 16392, 20001, 32767, 32768, 32769):
+    for seg in (16385, 16392, 20001, 32767, 32768, 32769, 40003, 49152, 57343, 57344, 57345):
         x = make_input(dtype, (5, seg), seed=seg)
         x[2] = x[2, 0]
         x[3] = np.sort(x[3])[::-1]
@@ -516,7 +516,7 @@ def test_two_byte_rows_of_up_to_32768_keys_are_counted(lib, torch_cuda, dtype):
         v, _ = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=False)
         labels = {k for k, _ in _lib.profile_collect()}
         lib.cpn_profile_enable(0)
-        assert ("count16_row_sort" in labels) == (seg <= 32768), (seg, labels)
+        assert ("count16_row_sort" in labels) == (seg <= 57344), (seg, labels)
         assert_same_bits(v, oracle.local_sort(x, argsort=False), f"{np.dtype(dtype)} seg={seg}")
         v, _ = abi_sort(lib, torch_cuda, x, want_values=True, want_indices=False, in_place=True)
         assert_same_bits(v, oracle.local_sort(x, argsort=False), f"{np.dtype(dtype)} seg={seg} in place")
