@@ -1,4 +1,4 @@
-// Short rows of real keys of up to 8 bytes (how long: bitonic_row_limit, 128 ... 512 keys), sorted by a
+// Short rows of real keys of up to 8 bytes (how long: bitonic_row_limit, 128 ... 1024 keys), sorted by a
 // network of compare-exchanges on words held in registers, E = 8 ... 16 elements per lane: element i of a row
 // sits in register i % E of the row's lane i / E, a row takes a power of two of lanes (1 ... 64, with the E that
 // covers it) and a wavefront holds 64 / lanes rows.  The exchanges between elements of one lane happen between

@@ -78,7 +78,7 @@ int merge_levels_limit(int key_bytes, bool want_indices)
   return key_bytes == 8 ? (want_indices ? 5 : 6) : 2;
 }
 
-// 1: rows of 2 ... 128 real keys go through the bitonic network; 0: through the ranking kernels
+// 1: short rows of real keys (2 ... bitonic_row_limit keys) go through the sorting network; 0: through the ranking kernels
 static std::atomic<int> g_bitonic_rows{[] {
   const char* e = getenv("CPN_SORT_BITONIC_ROWS");
   return (e != nullptr && e[0] == '0') ? 0 : 1;

@@ -106,7 +106,7 @@ __host__ __device__ constexpr int key_passes(int key_bytes, int codec)
   return codec == CODEC_COMPLEX ? key_bytes + 1 : key_bytes;
 }
 
-// Rows of 2 ... 128 real keys go through the bitonic network (bitonic_row_sort.h)
+// Short rows of real keys (2 ... bitonic_row_limit keys) go through the sorting network (bitonic_row_sort.h)
 // unless CPN_SORT_BITONIC_ROWS=0 in the environment sends them to the ranking kernels (A/B runs).
 bool bitonic_rows_enabled();
 // Longest row that goes through the network, per key width and with or without positions; the environment
